@@ -1,0 +1,175 @@
+"""The cache manager: everything a request holds between steps.
+
+It owns the groups of pages (pages.py), the state slots (state.py), the length
+of every request, and, when given an allocator, the device tensors behind them.
+The host logic runs without a GPU; device work (page copies for copy-on-write,
+zeroing of a fresh state slot) goes through two callbacks.
+
+Per step the step function calls `append_many([(request, n_tokens), ...])`,
+which is atomic: either every request gets its slots in every group, or
+OutOfPages is raised and nothing has changed (the reference preflights every
+layer before mutating any, runtime/model.py:98-102).
+"""
+from dataclasses import dataclass, field
+
+from .pages import CacheGroup, KVNeed, OutOfPages, StateNeed
+from .state import StateSlots
+
+
+@dataclass
+class Appended:
+    """What one request got in a step."""
+    request: object
+    start: int                                  # position of its first new token
+    count: int
+    slots: dict = field(default_factory=dict)   # group id -> [count] physical token slots
+    state_slot: int = 0
+
+
+class CacheManager:
+    def __init__(self, site_needs, n_pages, page_size, max_requests, state_needs=None,
+                 allocate_kv=None, allocate_state=None, copy_pages=None, zero_state=None, copy_state=None):
+        """site_needs: {site id: KVNeed}; state_needs: {site id: StateNeed}.
+        n_pages: pages per group (an int, or {KVNeed: int})."""
+        self.page_size = page_size
+        self.groups = []
+        self.group_of_site = {}
+        by_need = {}
+        for site, need in site_needs.items():
+            by_need.setdefault(need, []).append(site)
+        for gid, (need, sites) in enumerate(by_need.items()):
+            pages = n_pages[need] if isinstance(n_pages, dict) else n_pages
+            group = CacheGroup(need, sites, pages, page_size)
+            if allocate_kv is not None:
+                group.storage = allocate_kv(len(sites), pages, need.kv_heads, page_size, need.head_dim)
+            self.groups.append(group)
+            for index, site in enumerate(sites):
+                self.group_of_site[site] = (gid, index)
+        self.lengths = {}
+        self.slots = StateSlots(max_requests)
+        self.state_needs = dict(state_needs or {})
+        self.state_storage = {}
+        if allocate_state is not None:
+            for site, need in self.state_needs.items():
+                self.state_storage[site] = allocate_state(max_requests, need.shape, need.dtype)
+        self._copy_pages, self._zero_state, self._copy_state = copy_pages, zero_state, copy_state
+
+    # -- requests ---------------------------------------------------------
+    def create(self, request):
+        if request in self.lengths:
+            raise ValueError(f"duplicate request {request!r}")
+        slot = self.slots.acquire(request)
+        self.lengths[request] = 0
+        for group in self.groups:
+            group.create(request)
+        if self._zero_state is not None:
+            for site in self.state_needs:
+                self._zero_state(self.state_storage[site], slot)
+        return slot
+
+    def fork(self, source, target):
+        """target starts as a copy of source: pages shared, state copied."""
+        if target in self.lengths:
+            raise ValueError(f"duplicate request {target!r}")
+        slot = self.slots.acquire(target)
+        self.lengths[target] = self.lengths[source]
+        for group in self.groups:
+            group.fork(source, target)
+        if self._copy_state is not None:
+            for site in self.state_needs:
+                self._copy_state(self.state_storage[site], self.slots.slot_of(source), slot)
+        return slot
+
+    def release(self, request):
+        """Give back everything the request holds.  The caller makes sure no
+        device work that reads its pages is still running."""
+        del self.lengths[request]
+        for group in self.groups:
+            group.release(request)
+        self.slots.release(request)
+
+    def __contains__(self, request):
+        return request in self.lengths
+
+    def length(self, request):
+        return self.lengths[request]
+
+    # -- appending ----------------------------------------------------------
+    def pages_needed(self, items):
+        """Per group: fresh pages minus pages a window gives back first."""
+        out = []
+        for group in self.groups:
+            need = 0
+            for request, n in items:
+                length = self.lengths[request]
+                need += group.pages_needed(request, length, n) - group.trimmable(request, length)
+            out.append(need)
+        return out
+
+    def can_append(self, items):
+        return all(need <= len(group.pool.free) for need, group in zip(self.pages_needed(items), self.groups))
+
+    def append_many(self, items):
+        """items: [(request, n_new)], each request at most once.  Returns [Appended]."""
+        seen = set()
+        for request, n in items:
+            if request not in self.lengths:
+                raise KeyError(f"unknown request {request!r}")
+            if request in seen:
+                raise ValueError(f"request {request!r} appears twice in one step")
+            if n <= 0:
+                raise ValueError("a request must bring at least one token")
+            seen.add(request)
+        if not self.can_append(items):
+            raise OutOfPages("not enough free KV pages for this step")
+        result = []
+        for request, n in items:
+            length = self.lengths[request]
+            done = Appended(request, length, n, state_slot=self.slots.slot_of(request))
+            for gid, group in enumerate(self.groups):
+                group.trim(request, length)
+                slots, copies = group.append(request, length, n)
+                done.slots[gid] = slots
+                if copies and self._copy_pages is not None:
+                    self._copy_pages(group, copies)
+            self.lengths[request] = length + n
+            result.append(done)
+        return result
+
+    def trim(self, request):
+        """Give back pages that a window has passed (also done by every append)."""
+        for group in self.groups:
+            group.trim(request, self.lengths[request])
+
+    def table(self, gid, request):
+        return self.groups[gid].tables[request]
+
+    # -- views for mixers ---------------------------------------------------
+    def kv_of_site(self, site):
+        """(group id, keys [pages, kv_heads, P, D], values) of a site."""
+        gid, index = self.group_of_site[site]
+        storage = self.groups[gid].storage
+        return gid, storage[index, 0], storage[index, 1]
+
+    # -- bookkeeping --------------------------------------------------------
+    def check(self):
+        for group in self.groups:
+            group.check()
+            assert set(group.tables) == set(self.lengths), "a group knows other requests than the manager"
+            for request, table in group.tables.items():
+                assert len(table) == -(-self.lengths[request] // group.page_size), "table length differs from token count"
+        self.slots.check()
+        assert set(self.slots.owner) == set(self.lengths)
+
+    def free_pages(self):
+        return [len(g.pool.free) for g in self.groups]
+
+    def report(self):
+        out = []
+        for gid, g in enumerate(self.groups):
+            token_bytes = 2 * g.need.kv_heads * g.need.head_dim * len(g.sites)
+            out.append({"group": gid, "sites": len(g.sites), "window": g.need.window, "pages": g.pool.n_pages,
+                        "resident_pages": g.pool.used, "peak_pages": g.pool.peak, "free_pages": len(g.pool.free),
+                        "shared_pages": sum(1 for r in g.pool.refs if r > 1), "requests": len(g.tables),
+                        "elements_per_token": token_bytes})
+        return out

@@ -1,0 +1,239 @@
+// Row-wise and element-wise kernels of the forward pass: embedding gather,
+// RMSNorm (optionally on gathered rows), residual add, SwiGLU, rotary embedding
+// fused with the key/value scatter into the paged cache, and the page copy used
+// for copy-on-write.  The residual stream is float in every mode; `T` below is
+// the storage type of activations and weights (float or bf16).
+#include "common.h"
+
+// ---------------------------------------------------------------- embedding
+// out[r, :] = table[ids[r], :]  (reference: kernels/execution.cu:2-5)
+template <typename T>
+__global__ void embedding_kernel(const int* __restrict__ ids, const T* __restrict__ table,
+                                 float* __restrict__ out, int dim, int vocab) {
+    const int row = blockIdx.x;
+    int id = ids[row];
+    if (id < 0 || id >= vocab) id = 0;  // padding rows; real ids are checked on the host
+    const T* src = table + (size_t)id * dim;
+    float* dst = out + (size_t)row * dim;
+    for (int d = threadIdx.x; d < dim; d += blockDim.x) dst[d] = load_f32(src + d);
+}
+
+extern "C" int cisr_embedding(const int* ids, const void* table, float* out, int rows, int dim,
+                              int vocab, int dtype, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    if (dtype == DT_F32)
+        embedding_kernel<float><<<rows, 256, 0, stream>>>(ids, (const float*)table, out, dim, vocab);
+    else
+        embedding_kernel<bf16_t><<<rows, 256, 0, stream>>>(ids, (const bf16_t*)table, out, dim, vocab);
+    return CISR_LAUNCH_CHECK();
+}
+
+// ------------------------------------------------------------------ RMSNorm
+// y = x * rsqrt(mean(x^2) + eps) * w  (reference: kernels/ops.cu:3-19).
+// Input is the float residual stream; `rows` (may be null) picks input rows.
+template <typename T>
+__global__ void rmsnorm_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                               T* __restrict__ y, const int* __restrict__ rows, int dim, float eps) {
+    __shared__ float red[4];
+    const int orow = blockIdx.x;
+    const int irow = rows ? rows[orow] : orow;
+    const float* src = x + (size_t)irow * dim;
+    float ss = 0.f;
+    for (int d = threadIdx.x; d < dim; d += 256) { float a = src[d]; ss += a * a; }
+    const float total = block_sum<256>(ss, red);
+    const float scale = 1.0f / sqrtf(total / (float)dim + eps);
+    T* dst = y + (size_t)orow * dim;
+    for (int d = threadIdx.x; d < dim; d += 256) store_f32(dst + d, src[d] * scale * w[d]);
+}
+
+extern "C" int cisr_rmsnorm(const float* x, const float* w, void* y, const int* rows, int n_out,
+                            int dim, float eps, int out_dtype, hipStream_t stream) {
+    if (n_out <= 0) return 0;
+    if (out_dtype == DT_F32)
+        rmsnorm_kernel<float><<<n_out, 256, 0, stream>>>(x, w, (float*)y, rows, dim, eps);
+    else
+        rmsnorm_kernel<bf16_t><<<n_out, 256, 0, stream>>>(x, w, (bf16_t*)y, rows, dim, eps);
+    return CISR_LAUNCH_CHECK();
+}
+
+// x += delta, then y = rmsnorm(x) (reference: kernels/execution.cu:12-24; here
+// the sum stays float so nothing is rounded before the norm reads it).
+template <typename TD, typename T>
+__global__ void add_rmsnorm_kernel(float* __restrict__ x, const TD* __restrict__ delta,
+                                   const float* __restrict__ w, T* __restrict__ y, int dim, float eps) {
+    __shared__ float red[4];
+    const int row = blockIdx.x;
+    float* xr = x + (size_t)row * dim;
+    const TD* dr = delta + (size_t)row * dim;
+    float ss = 0.f;
+    for (int d = threadIdx.x; d < dim; d += 256) {
+        float a = xr[d] + load_f32(dr + d);
+        xr[d] = a;
+        ss += a * a;
+    }
+    const float total = block_sum<256>(ss, red);
+    const float scale = 1.0f / sqrtf(total / (float)dim + eps);
+    T* dst = y + (size_t)row * dim;
+    for (int d = threadIdx.x; d < dim; d += 256) store_f32(dst + d, xr[d] * scale * w[d]);
+}
+
+extern "C" int cisr_add_rmsnorm(float* x, const void* delta, const float* w, void* y, int rows, int dim,
+                                float eps, int dtype, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    if (dtype == DT_F32)
+        add_rmsnorm_kernel<float, float><<<rows, 256, 0, stream>>>(x, (const float*)delta, w, (float*)y, dim, eps);
+    else
+        add_rmsnorm_kernel<bf16_t, bf16_t><<<rows, 256, 0, stream>>>(x, (const bf16_t*)delta, w, (bf16_t*)y, dim, eps);
+    return CISR_LAUNCH_CHECK();
+}
+
+// x += delta (reference: kernels/execution.cu:42-44), float residual
+template <typename TD>
+__global__ void add_kernel(float* __restrict__ x, const TD* __restrict__ delta, size_t n) {
+    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) x[i] += load_f32(delta + i);
+}
+
+extern "C" int cisr_residual_add(float* x, const void* delta, long long n, int dtype, hipStream_t stream) {
+    if (n <= 0) return 0;
+    unsigned blocks = (unsigned)((n + 255) / 256);
+    if (dtype == DT_F32) add_kernel<float><<<blocks, 256, 0, stream>>>(x, (const float*)delta, (size_t)n);
+    else add_kernel<bf16_t><<<blocks, 256, 0, stream>>>(x, (const bf16_t*)delta, (size_t)n);
+    return CISR_LAUNCH_CHECK();
+}
+
+// ------------------------------------------------------------------- SwiGLU
+// act[r, i] = g * sigmoid(g) * u with g = gu[r, i], u = gu[r, inter + i]
+// (reference: kernels/execution.cu:7-10), arithmetic in float.
+template <typename T>
+__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ act, int inter, size_t n) {
+    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    size_t row = i / inter; int col = (int)(i % inter);
+    const T* base = gu + row * (size_t)(2 * inter);
+    float g = load_f32(base + col), u = load_f32(base + inter + col);
+    store_f32(act + i, g / (1.0f + expf(-g)) * u);
+}
+
+extern "C" int cisr_swiglu(const void* gu, void* act, int rows, int inter, int dtype, hipStream_t stream) {
+    size_t n = (size_t)rows * inter;
+    if (n == 0) return 0;
+    unsigned blocks = (unsigned)((n + 255) / 256);
+    if (dtype == DT_F32) swiglu_kernel<float><<<blocks, 256, 0, stream>>>((const float*)gu, (float*)act, inter, n);
+    else swiglu_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)act, inter, n);
+    return CISR_LAUNCH_CHECK();
+}
+
+// ------------------------------------------------- rotary embedding + scatter
+// One block per token row of the fused projection buffer
+//   qkv[r] = [ q: heads*D | k: kv_heads*D | v: kv_heads*D ].
+// q is rotated in place; k is rotated and written to the cache; v is copied to
+// the cache.  Pairing is split-half over the first `rot` coordinates of a head:
+// (i, i + rot/2) turns by the angle whose cosine and sine sit in
+// cos_tab/sin_tab[pos, i] (tables are float, [max_pos, rot/2]).
+// (reference: kernels/ops.cu:21-33, kernels/execution.cu:28-40)
+// Cache layout per site: [pages, kv_heads, page_size, D]; slot = page*page_size
+// + offset; a negative slot writes nothing (padding rows, read-only sites).
+template <typename T>
+__global__ void rope_scatter_kernel(T* __restrict__ qkv, const int* __restrict__ positions,
+                                    const int* __restrict__ slots, const float* __restrict__ cos_tab,
+                                    const float* __restrict__ sin_tab, T* __restrict__ kcache,
+                                    T* __restrict__ vcache, int heads, int kv_heads, int dim, int rot,
+                                    int page_size, int max_pos, int has_kv) {
+    const int row = blockIdx.x;
+    const int half = rot / 2;
+    int pos = positions[row];
+    if (pos < 0) pos = 0;
+    if (pos >= max_pos) pos = max_pos - 1;  // host rejects this before launch
+    const float* cs = cos_tab + (size_t)pos * half;
+    const float* sn = sin_tab + (size_t)pos * half;
+    const int row_width = (heads + (has_kv ? 2 * kv_heads : 0)) * dim;
+    T* base = qkv + (size_t)row * row_width;
+    const int slot = (has_kv && slots) ? slots[row] : -1;
+    const int page = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot % page_size : 0;
+
+    // q heads: rotate in place
+    for (int i = threadIdx.x; i < heads * half; i += blockDim.x) {
+        int h = i / half, d = i % half;
+        T* p = base + h * dim;
+        float a = load_f32(p + d), b = load_f32(p + d + half);
+        float c = cs[d], s = sn[d];
+        store_f32(p + d, a * c - b * s);
+        store_f32(p + d + half, b * c + a * s);
+    }
+    if (slot < 0) return;
+    // k heads: rotate and scatter
+    const T* kb = base + heads * dim;
+    for (int i = threadIdx.x; i < kv_heads * half; i += blockDim.x) {
+        int h = i / half, d = i % half;
+        const T* p = kb + h * dim;
+        float a = load_f32(p + d), b = load_f32(p + d + half);
+        float c = cs[d], s = sn[d];
+        T* dst = kcache + (((size_t)page * kv_heads + h) * page_size + off) * dim;
+        store_f32(dst + d, a * c - b * s);
+        store_f32(dst + d + half, b * c + a * s);
+    }
+    // coordinates beyond the rotated part of k pass through
+    if (rot < dim) {
+        int tail = dim - rot;
+        for (int i = threadIdx.x; i < kv_heads * tail; i += blockDim.x) {
+            int h = i / tail, d = rot + i % tail;
+            kcache[(((size_t)page * kv_heads + h) * page_size + off) * dim + d] = kb[h * dim + d];
+        }
+    }
+    // v heads: copy
+    const T* vb = kb + kv_heads * dim;
+    for (int i = threadIdx.x; i < kv_heads * dim; i += blockDim.x) {
+        int h = i / dim, d = i % dim;
+        vcache[(((size_t)page * kv_heads + h) * page_size + off) * dim + d] = vb[i];
+    }
+}
+
+extern "C" int cisr_rope_scatter(void* qkv, const int* positions, const int* slots, const float* cos_tab,
+                                 const float* sin_tab, void* kcache, void* vcache, int rows, int heads,
+                                 int kv_heads, int dim, int rot, int page_size, int max_pos, int has_kv,
+                                 int dtype, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    if (dtype == DT_F32)
+        rope_scatter_kernel<float><<<rows, 256, 0, stream>>>((float*)qkv, positions, slots, cos_tab, sin_tab,
+            (float*)kcache, (float*)vcache, heads, kv_heads, dim, rot, page_size, max_pos, has_kv);
+    else
+        rope_scatter_kernel<bf16_t><<<rows, 256, 0, stream>>>((bf16_t*)qkv, positions, slots, cos_tab, sin_tab,
+            (bf16_t*)kcache, (bf16_t*)vcache, heads, kv_heads, dim, rot, page_size, max_pos, has_kv);
+    return CISR_LAUNCH_CHECK();
+}
+
+// ------------------------------------------------------------- page copy
+// Copy whole pages inside one cache tensor laid out [slabs, pages, page_elems]:
+// for every slab, page dst[i] := page src[i].  Used for copy-on-write of a
+// shared, partly filled page (reference: runtime/cache.py:70-75).
+__global__ void page_copy_kernel(uint32_t* __restrict__ pool, const int* __restrict__ src,
+                                 const int* __restrict__ dst, size_t page_words, size_t slab_words) {
+    const int pair = blockIdx.x, slab = blockIdx.y;
+    const uint32_t* s = pool + slab * slab_words + (size_t)src[pair] * page_words;
+    uint32_t* d = pool + slab * slab_words + (size_t)dst[pair] * page_words;
+    for (size_t i = threadIdx.x; i < page_words; i += blockDim.x) d[i] = s[i];
+}
+
+extern "C" int cisr_page_copy(void* pool, const int* src, const int* dst, int n_pairs, int slabs,
+                              long long page_bytes, long long slab_bytes, hipStream_t stream) {
+    if (n_pairs <= 0 || slabs <= 0) return 0;
+    if (page_bytes % 4 || slab_bytes % 4) return (int)hipErrorInvalidValue;
+    page_copy_kernel<<<dim3(n_pairs, slabs), 256, 0, stream>>>((uint32_t*)pool, src, dst,
+        (size_t)(page_bytes / 4), (size_t)(slab_bytes / 4));
+    return CISR_LAUNCH_CHECK();
+}
+
+// ------------------------------------------------------------- conversions
+// float -> bf16 with round-to-nearest-even; used when a matrix stored in 32 bits
+// is run in bf16, and by the tests of the rounding rule.
+__global__ void f32_to_bf16_kernel(const float* __restrict__ x, bf16_t* __restrict__ y, size_t n) {
+    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) y[i] = f32_to_bf16(x[i]);
+}
+
+extern "C" int cisr_f32_to_bf16(const float* x, void* y, long long n, hipStream_t stream) {
+    if (n <= 0) return 0;
+    f32_to_bf16_kernel<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(x, (bf16_t*)y, (size_t)n);
+    return CISR_LAUNCH_CHECK();
+}

@@ -1,0 +1,111 @@
+// Token choice from float logits [R, V]: greedy (lowest index wins a tie, as
+// numpy/cupy argmax does in the reference, runtime/engine.py:99) and temperature
+// sampling p = softmax(logits / T) drawn by inverse CDF with a counter-based
+// random number per (seed, counter), so a request's draw does not depend on
+// what else is in the batch.  One block of 256 threads per row; every thread
+// owns one contiguous slice of the vocabulary, which fixes the summation order.
+#include "common.h"
+
+__device__ __forceinline__ uint64_t splitmix64(uint64_t x) {
+    x += 0x9E3779B97F4A7C15ull;
+    x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ull;
+    x = (x ^ (x >> 27)) * 0x94D049BB133111EBull;
+    return x ^ (x >> 31);
+}
+
+// uniform in [0, 1) with 24 random bits
+__device__ __forceinline__ float uniform01(uint64_t seed, uint64_t counter) {
+    uint64_t h = splitmix64(splitmix64(seed) ^ (counter * 0xD1342543DE82EF95ull));
+    return (float)(h >> 40) * (1.0f / 16777216.0f);
+}
+
+__device__ __forceinline__ void argmax_block(const float* __restrict__ x, int n, float* smax, int* sidx,
+                                             float& best, int& best_idx) {
+    float bv = -INFINITY; int bi = 0x7fffffff;
+    for (int i = threadIdx.x; i < n; i += 256) {
+        float v = x[i];
+        if (bi == 0x7fffffff || v > bv) { bv = v; bi = i; }  // indices ascend: a tie keeps the lower one
+    }
+    smax[threadIdx.x] = bv; sidx[threadIdx.x] = bi;
+    __syncthreads();
+    for (int s = 128; s > 0; s >>= 1) {
+        if (threadIdx.x < s) {
+            float ov = smax[threadIdx.x + s]; int oi = sidx[threadIdx.x + s];
+            float mv = smax[threadIdx.x]; int mi = sidx[threadIdx.x];
+            if (oi != 0x7fffffff && (mi == 0x7fffffff || ov > mv || (ov == mv && oi < mi))) {
+                smax[threadIdx.x] = ov; sidx[threadIdx.x] = oi;
+            }
+        }
+        __syncthreads();
+    }
+    best = smax[0]; best_idx = sidx[0];
+    __syncthreads();
+}
+
+__global__ void __launch_bounds__(256)
+argmax_kernel(const float* __restrict__ logits, int* __restrict__ out, int vocab) {
+    __shared__ float smax[256];
+    __shared__ int sidx[256];
+    const float* x = logits + (size_t)blockIdx.x * vocab;
+    float best; int idx;
+    argmax_block(x, vocab, smax, sidx, best, idx);
+    if (threadIdx.x == 0) out[blockIdx.x] = idx == 0x7fffffff ? 0 : idx;
+}
+
+extern "C" int cisr_argmax(const float* logits, int* out, int rows, int vocab, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    argmax_kernel<<<rows, 256, 0, stream>>>(logits, out, vocab);
+    return CISR_LAUNCH_CHECK();
+}
+
+__global__ void __launch_bounds__(256)
+sample_kernel(const float* __restrict__ logits, const float* __restrict__ temperature,
+              const unsigned long long* __restrict__ seeds, const unsigned long long* __restrict__ counters,
+              int* __restrict__ out, int vocab) {
+    __shared__ float smax[256];
+    __shared__ int sidx[256];
+    __shared__ float ssum[256];
+    const int row = blockIdx.x;
+    const float* x = logits + (size_t)row * vocab;
+    float best; int best_idx;
+    argmax_block(x, vocab, smax, sidx, best, best_idx);
+    const float temp = temperature[row];
+    if (!(temp > 0.f)) {  // greedy
+        if (threadIdx.x == 0) out[row] = best_idx == 0x7fffffff ? 0 : best_idx;
+        return;
+    }
+    const float inv_t = 1.0f / temp;
+    const int per = (vocab + 255) / 256;
+    const int lo = threadIdx.x * per, hi = min(vocab, lo + per);
+    float part = 0.f;
+    for (int i = lo; i < hi; ++i) part += expf((x[i] - best) * inv_t);
+    ssum[threadIdx.x] = part;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float total = 0.f;
+        for (int t = 0; t < 256; ++t) total += ssum[t];
+        const float target = uniform01(seeds[row], counters[row]) * total;
+        // find the slice, then the token inside it; fall back to the last token
+        // with non-zero mass if rounding pushes the target past the end
+        float run = 0.f; int choice = -1;
+        int t = 0;
+        for (; t < 256; ++t) { if (run + ssum[t] > target) break; run += ssum[t]; }
+        if (t < 256) {
+            const int a = t * per, b = min(vocab, a + per);
+            for (int i = a; i < b; ++i) {
+                run += expf((x[i] - best) * inv_t);
+                if (run > target) { choice = i; break; }
+            }
+            if (choice < 0) choice = b - 1;
+        }
+        if (choice < 0) choice = best_idx;
+        out[row] = choice;
+    }
+}
+
+extern "C" int cisr_sample(const float* logits, const float* temperature, const unsigned long long* seeds,
+                           const unsigned long long* counters, int* out, int rows, int vocab, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    sample_kernel<<<rows, 256, 0, stream>>>(logits, temperature, seeds, counters, out, vocab);
+    return CISR_LAUNCH_CHECK();
+}

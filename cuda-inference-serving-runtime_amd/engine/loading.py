@@ -1,0 +1,47 @@
+"""From a model folder to a model on the GPU, and the random-weights mode.
+
+The architecture is chosen by config.json through the registry; weights are
+bound by tensor name (reference: runtime/checkpoint.py:9-41 for loading,
+runtime/model.py:38-55 for seeded random weights)."""
+import torch
+
+from ..config import architecture_of, read_config_json, preset
+from ..weights import load_folder, write_model_folder
+
+DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+def parse_dtype(dtype):
+    if isinstance(dtype, torch.dtype):
+        if dtype not in DTYPES.values():
+            raise ValueError(f"dtype {dtype} is not float32 or bfloat16")
+        return dtype
+    try:
+        return DTYPES[dtype]
+    except KeyError:
+        raise ValueError(f"dtype {dtype!r} is not one of {sorted(DTYPES)}") from None
+
+
+def build_from_config_dict(raw):
+    arch = architecture_of(raw)
+    config = arch.config_cls.from_dict(raw)
+    return arch, config, arch.build(config)
+
+
+def load_model(folder, dtype="bfloat16", device="cuda:0"):
+    """The model of `folder` with its weights on `device`, ready to step."""
+    dtype = parse_dtype(dtype)
+    raw = read_config_json(folder)
+    _, _, model = build_from_config_dict(raw)
+    tensors = load_folder(folder, model.tensor_specs(), dtype, torch.device(device))
+    model.bind(tensors, dtype, torch.device(device))
+    return model
+
+
+def write_random_model(folder, config, seed, dtype="bfloat16"):
+    """Write config.json and model.safetensors for `config` (a config.json dict or
+    the name of a preset) with seeded random weights."""
+    raw = preset(config) if isinstance(config, str) else dict(config)
+    _, typed, model = build_from_config_dict(raw)
+    return write_model_folder(folder, typed.to_dict() if hasattr(typed, "to_dict") else raw,
+                              model.tensor_specs(), seed, parse_dtype(dtype))

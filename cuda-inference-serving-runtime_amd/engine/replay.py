@@ -1,0 +1,71 @@
+"""Trace replay: feeds given token ids through a model step by step and writes
+logits.  It samples nothing and has no forward pass, cache or loader of its
+own: it drives load_model, ModelRunner.step and the cache manager, the ones that
+generation uses.
+
+Input, one JSON object per line on standard input:
+    {"step": 0, "entries": [{"id": "a", "tokens": [5, 17, 3], "want": [0, 2]}], "end": []}
+For a step in which something is wanted, ``<out>/<step>.f32`` receives the
+logits at the wanted places as little-endian float32 [wanted, vocab], in the
+order of the entries and of ``want``.  After every step ``done <step>`` is
+printed and flushed.  (The reference's nearest relatives are its fixed step
+schedules in tests/test_model.py:24-25 and tests/test_execution.py:25-30.)
+"""
+import argparse
+import json
+import sys
+from pathlib import Path
+
+import numpy as np
+import torch
+
+from .loading import load_model
+from .runner import ModelRunner, StepEntry
+
+PAGE_SIZE = 16          # divides 64, so a request rounded up to 64 tokens never holds more than its share
+MAX_LIVE = 4
+
+
+def replay(model_dir, dtype, out_dir, max_tokens, lines, page_size=PAGE_SIZE, echo=print):
+    out_dir = Path(out_dir)
+    out_dir.mkdir(parents=True, exist_ok=True)
+    model = load_model(model_dir, dtype=dtype)
+    pages = max(1, -(-int(max_tokens) // page_size))
+    runner = ModelRunner(model, n_pages=pages, page_size=page_size, max_requests=max(MAX_LIVE, 8))
+    for line in lines:
+        line = line.strip()
+        if not line:
+            continue
+        record = json.loads(line)
+        entries = []
+        for item in record.get("entries", []):
+            if item["id"] not in runner.cache:
+                runner.create(item["id"])
+            entries.append(StepEntry(item["id"], item["tokens"], item.get("want", [])))
+        if entries:
+            logits = runner.step(entries)
+            if logits.shape[0]:
+                data = logits.to(torch.float32).cpu().numpy().astype("<f4", copy=False)
+                data.tofile(out_dir / f"{record['step']}.f32")
+        for request in record.get("end", []):
+            if request in runner.cache:
+                runner.release(request)
+        torch.cuda.synchronize()
+        echo(f"done {record['step']}")
+    return runner
+
+
+def main(argv=None):
+    parser = argparse.ArgumentParser(prog="trace_run", description="Replay a token trace and write logits.")
+    parser.add_argument("--model", required=True, help="folder with config.json and model.safetensors")
+    parser.add_argument("--dtype", choices=["bfloat16", "float32"], required=True)
+    parser.add_argument("--out", required=True, help="folder for <step>.f32 files")
+    parser.add_argument("--max-tokens", type=int, required=True,
+                        help="most tokens live requests hold at any time (each rounded up to 64)")
+    args = parser.parse_args(argv)
+
+    def echo(text):
+        print(text, flush=True)
+
+    replay(args.model, args.dtype, args.out, args.max_tokens, sys.stdin, echo=echo)
+    return 0

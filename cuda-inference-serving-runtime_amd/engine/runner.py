@@ -1,0 +1,206 @@
+"""The step function.
+
+`ModelRunner.step(entries)` takes a batch of (request, its next tokens, wanted
+places), prompt portions beside single decoded tokens, cut anywhere; reserves
+cache slots for the new tokens; runs the model on exactly those tokens as one
+batch against the cache; and returns the float logits at the wanted places, in
+the order of the entries and of their `want` lists.
+
+The reference's step takes exactly one token per request and returns logits for
+every row (runtime/model.py:86-120); its order of checks is kept: batch shape,
+context limit, token range, page preflight, then execution
+(runtime/model.py:93-102).
+"""
+from dataclasses import dataclass, field
+from typing import List, Sequence
+
+import numpy as np
+import torch
+
+from ..cache import CacheManager, OutOfPages
+from ..kernels import ops
+from .context import GroupView, StepContext, Workspace
+
+
+@dataclass
+class StepEntry:
+    request: object
+    tokens: Sequence[int]
+    want: Sequence[int] = field(default_factory=list)  # indices into `tokens` whose logits are returned
+
+
+_TORCH_OF = {"float32": torch.float32, "bfloat16": torch.bfloat16, "int32": torch.int32}
+
+
+class ModelRunner:
+    def __init__(self, model, n_pages, page_size=16, max_requests=64, device="cuda:0"):
+        if not torch.cuda.is_available():
+            raise RuntimeError("no GPU: the engine runs on an MI355X only and has no CPU path")
+        ops.lib()  # fail now if the kernel library is missing
+        self.model = model
+        self.device = torch.device(device)
+        self.page_size = page_size
+        self.max_requests = max_requests
+        dtype = model.dtype
+
+        def allocate_kv(sites, pages, kv_heads, psize, head_dim):
+            return torch.zeros((sites, 2, pages, kv_heads, psize, head_dim), dtype=dtype, device=self.device)
+
+        def allocate_state(slots, shape, dt):
+            return torch.zeros((slots, *shape), dtype=_TORCH_OF[dt], device=self.device)
+
+        self.cache = CacheManager(model.cache_needs(), n_pages, page_size, max_requests,
+                                  state_needs=model.state_needs(), allocate_kv=allocate_kv,
+                                  allocate_state=allocate_state, copy_pages=self._copy_pages,
+                                  zero_state=lambda t, s: t[s].zero_(),
+                                  copy_state=lambda t, a, b: t[b].copy_(t[a]))
+        self.workspace = Workspace(self.device)
+        self.max_context = model.max_positions
+        self.table_width = -(-self.max_context // page_size)
+        self._staging = []
+        self._staging_next = 0
+        self.steps = 0
+
+    # -- requests -------------------------------------------------------------
+    def create(self, request):
+        return self.cache.create(request)
+
+    def fork(self, source, target):
+        return self.cache.fork(source, target)
+
+    def release(self, request):
+        # later work that reuses the pages runs on the same stream, after every reader
+        self.cache.release(request)
+
+    def length(self, request):
+        return self.cache.length(request)
+
+    def _copy_pages(self, group, copies):
+        src = torch.tensor([c[0] for c in copies], dtype=torch.int32, device=self.device)
+        dst = torch.tensor([c[1] for c in copies], dtype=torch.int32, device=self.device)
+        ops.page_copy(group.storage, src, dst, group.storage.shape[0] * 2, group.pool.n_pages)
+
+    # -- the step -------------------------------------------------------------
+    def check(self, entries):
+        if not entries:
+            raise ValueError("a step needs at least one entry")
+        seen = set()
+        for e in entries:
+            if e.request in seen:
+                raise ValueError(f"request {e.request!r} appears twice in one step")
+            seen.add(e.request)
+            if e.request not in self.cache:
+                raise KeyError(f"unknown request {e.request!r}")
+            n = len(e.tokens)
+            if n == 0:
+                raise ValueError(f"request {e.request!r} brings no tokens")
+            if self.cache.length(e.request) + n > self.max_context:
+                raise ValueError(f"request {e.request!r} exceeds the context limit of {self.max_context}")
+            if any((not 0 <= int(t) < self.model.vocab_size) for t in e.tokens):
+                raise ValueError(f"request {e.request!r} has a token outside the vocabulary")
+            if any((not 0 <= int(w) < n) for w in e.want):
+                raise ValueError(f"request {e.request!r} wants a place outside its tokens")
+
+    def step(self, entries: List[StepEntry]):
+        """Float logits [sum(len(want)), vocab] on the GPU (valid until the next step)."""
+        self.check(entries)
+        done = self.cache.append_many([(e.request, len(e.tokens)) for e in entries])  # OutOfPages changes nothing
+        ctx = self._context(entries, done)
+        self.steps += 1
+        logits = self.model.forward(ctx)
+        if logits is None:
+            return torch.empty((0, self.model.vocab_size), dtype=torch.float32, device=self.device)
+        return logits
+
+    def _context(self, entries, done):
+        T = sum(len(e.tokens) for e in entries)
+        S = len(entries)
+        R = sum(len(e.want) for e in entries)
+        W = self.table_width
+        G = len(self.cache.groups)
+        # one packed int32 upload: tokens, positions, seg_of_row, seg_start, seg_first_pos, state_slots,
+        # logit_rows, then per group slots and tables
+        sizes = [T, T, T, S + 1, S, S, R] + [T, S * W] * G
+        offsets = np.concatenate(([0], np.cumsum(sizes)))
+        host = self._stage(int(offsets[-1]))
+        arr = host.numpy()
+        tokens, positions, seg_of_row, seg_start, seg_first, state_slots, logit_rows = (
+            arr[offsets[i]:offsets[i + 1]] for i in range(7))
+        row = 0
+        out_row = 0
+        max_context = 0
+        for s, (e, d) in enumerate(zip(entries, done)):
+            n = len(e.tokens)
+            tokens[row:row + n] = e.tokens
+            positions[row:row + n] = np.arange(d.start, d.start + n)
+            seg_of_row[row:row + n] = s
+            seg_start[s] = row
+            seg_first[s] = d.start
+            state_slots[s] = d.state_slot
+            for w in e.want:
+                logit_rows[out_row] = row + int(w)
+                out_row += 1
+            for g in range(G):
+                base = 7 + 2 * g
+                arr[offsets[base] + row: offsets[base] + row + n] = d.slots[g]
+                table = self.cache.table(g, e.request)
+                trow = arr[offsets[base + 1] + s * W: offsets[base + 1] + (s + 1) * W]
+                trow[:len(table)] = table
+                trow[len(table):] = -1
+            row += n
+            max_context = max(max_context, d.start + n)
+        seg_start[S] = T
+        dev = self._upload(host, int(offsets[-1]))
+
+        def view(i, shape=None):
+            t = dev[int(offsets[i]):int(offsets[i + 1])]
+            return t if shape is None else t.view(shape)
+
+        ctx = StepContext(self)
+        ctx.n_rows, ctx.n_segments = T, S
+        ctx.tokens, ctx.positions, ctx.seg_of_row = view(0), view(1), view(2)
+        ctx.seg_start, ctx.seg_first_pos, ctx.state_slots, ctx.logit_rows = view(3), view(4), view(5), view(6)
+        ctx.kv = [GroupView(view(7 + 2 * g), view(8 + 2 * g, (S, W)), self.page_size, W) for g in range(G)]
+        ctx.segments = [(d.request, d.start, d.count) for d in done]
+        ctx.max_context = max_context
+        ctx.decode_only = all(d.count == 1 for d in done)
+        return ctx
+
+    def _stage(self, n):
+        """A pinned host buffer of at least n int32, not in flight."""
+        slot = self._staging_next % 4
+        self._staging_next += 1
+        while len(self._staging) <= slot:
+            self._staging.append(None)
+        entry = self._staging[slot]
+        if entry is None or entry[0].numel() < n:
+            cap = max(4096, 1 << (n - 1).bit_length())
+            entry = [torch.empty(cap, dtype=torch.int32, pin_memory=True),
+                     torch.empty(cap, dtype=torch.int32, device=self.device), None]
+            self._staging[slot] = entry
+        if entry[2] is not None:
+            entry[2].synchronize()  # the copy that last read this buffer is over
+        self._current = entry
+        return entry[0]
+
+    def _upload(self, host, n):
+        entry = self._current
+        entry[1][:n].copy_(host[:n], non_blocking=True)
+        entry[2] = torch.cuda.Event()
+        entry[2].record()
+        return entry[1]
+
+    # -- attention dispatch -------------------------------------------------------
+    def attention(self, ctx, q, q_row_stride, kcache, vcache, view, out, heads, kv_heads, head_dim, window, scale):
+        rows = out.shape[0]
+        span = ctx.max_context if not window else min(ctx.max_context, window)
+        splits = 1
+        waves = rows * heads
+        if waves < 2048 and span > 256:
+            splits = int(min(32, -(-span // 256), max(1, 4096 // waves)))
+        workspace = None
+        if splits > 1:
+            workspace = (ctx.buffer("attn.part_o", (rows * heads * splits * head_dim,), torch.float32),
+                         ctx.buffer("attn.part_ml", (rows * heads * splits * 2,), torch.float32))
+        ops.attention_rowwise(q, q_row_stride, kcache, vcache, view.tables, ctx.seg_of_row, ctx.positions, out,
+                              heads, kv_heads, head_dim, view.page_size, window, scale, splits, workspace)

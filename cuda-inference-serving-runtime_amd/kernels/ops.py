@@ -1,0 +1,265 @@
+"""Checked Python entry points of the HIP kernels.
+
+Every function validates device, dtype, contiguity and shapes on the host
+before the launch, because a kernel that reads out of bounds can take the GPU
+down.  Tensors are torch tensors on the GPU; launches go to torch's current
+stream, so they are ordered with torch's own work and can be captured into a
+graph.  Nothing here computes on the CPU.
+"""
+import ctypes as C
+
+import torch
+
+from . import library
+
+F32, BF16 = 0, 1
+_DT = {torch.float32: F32, torch.bfloat16: BF16}
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+_configured = False
+
+
+def lib():
+    global _configured
+    handle = library.load()
+    if not _configured:
+        _declare(handle)
+        _configured = True
+    return handle
+
+
+def _declare(h):
+    p, i, f, ll = C.c_void_p, C.c_int, C.c_float, C.c_longlong
+    sig = {
+        "cisr_embedding": [p, p, p, i, i, i, i, p],
+        "cisr_rmsnorm": [p, p, p, p, i, i, f, i, p],
+        "cisr_add_rmsnorm": [p, p, p, p, i, i, f, i, p],
+        "cisr_residual_add": [p, p, ll, i, p],
+        "cisr_swiglu": [p, p, i, i, i, p],
+        "cisr_rope_scatter": [p, p, p, p, p, p, p, i, i, i, i, i, i, i, i, i, p],
+        "cisr_page_copy": [p, p, p, i, i, ll, ll, p],
+        "cisr_f32_to_bf16": [p, p, ll, p],
+        "cisr_attn_rowwise": [p, i, p, p, p, p, p, p, p, p, i, i, i, i, i, i, i, f, i, i, p],
+        "cisr_gemm_f32": [p, i, p, i, p, i, p, i, i, i, i, p],
+        "cisr_gemm_bf16": [p, i, p, i, p, i, p, i, i, i, i, i, p],
+        "cisr_argmax": [p, p, i, i, p],
+        "cisr_sample": [p, p, p, p, p, i, i, p],
+    }
+    for name, args in sig.items():
+        fn = getattr(h, name)
+        fn.argtypes = args
+        fn.restype = C.c_int
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _check(code, what):
+    if code != 0:
+        raise KernelError(f"{what}: HIP error {code}")
+
+
+def _dev(t, name, dtype=None, shape=None):
+    if not isinstance(t, torch.Tensor) or not t.is_cuda:
+        raise KernelError(f"{name}: expected a GPU tensor")
+    if not t.is_contiguous():
+        raise KernelError(f"{name}: tensor must be contiguous")
+    if dtype is not None:
+        allowed = dtype if isinstance(dtype, (tuple, list)) else (dtype,)
+        if t.dtype not in allowed:
+            raise KernelError(f"{name}: dtype {t.dtype}, expected {allowed}")
+    if shape is not None and tuple(t.shape) != tuple(shape):
+        raise KernelError(f"{name}: shape {tuple(t.shape)}, expected {tuple(shape)}")
+    return t.data_ptr()
+
+
+def _storage(t, name):
+    if t.dtype not in _DT:
+        raise KernelError(f"{name}: storage dtype {t.dtype} is not float32 or bfloat16")
+    return _DT[t.dtype]
+
+
+def embedding(tokens, table, out):
+    """out[r] = table[tokens[r]] widened to float.  tokens int32 [T], table [V, H], out float [T, H]."""
+    rows = tokens.shape[0]
+    vocab, dim = table.shape
+    _check(lib().cisr_embedding(_dev(tokens, "tokens", torch.int32, (rows,)), _dev(table, "table"),
+                                _dev(out, "out", torch.float32, (rows, dim)), rows, dim, vocab,
+                                _storage(table, "table"), _stream()), "embedding")
+    return out
+
+
+def rmsnorm(x, weight, out, eps, rows=None):
+    """out = rmsnorm(x[rows]) * weight.  x float [T, H]; weight float [H]; out [R, H] float or bf16."""
+    dim = x.shape[1]
+    n_out = out.shape[0]
+    if rows is None and n_out != x.shape[0]:
+        raise KernelError("rmsnorm: out rows differ from input rows")
+    rp = None if rows is None else _dev(rows, "rows", torch.int32, (n_out,))
+    _check(lib().cisr_rmsnorm(_dev(x, "x", torch.float32), _dev(weight, "weight", torch.float32, (dim,)),
+                              _dev(out, "out", None, (n_out, dim)), rp, n_out, dim, float(eps),
+                              _storage(out, "out"), _stream()), "rmsnorm")
+    return out
+
+
+def add_rmsnorm(x, delta, weight, out, eps):
+    """x += delta (float residual, in place), out = rmsnorm(x) * weight."""
+    rows, dim = x.shape
+    dt = _storage(delta, "delta")
+    if out.dtype != delta.dtype:
+        raise KernelError("add_rmsnorm: out and delta must share a dtype")
+    _check(lib().cisr_add_rmsnorm(_dev(x, "x", torch.float32), _dev(delta, "delta", None, (rows, dim)),
+                                  _dev(weight, "weight", torch.float32, (dim,)), _dev(out, "out", None, (rows, dim)),
+                                  rows, dim, float(eps), dt, _stream()), "add_rmsnorm")
+    return out
+
+
+def residual_add(x, delta):
+    """x += delta, x float, delta float or bf16 of the same shape."""
+    if x.shape != delta.shape:
+        raise KernelError("residual_add: shapes differ")
+    _check(lib().cisr_residual_add(_dev(x, "x", torch.float32), _dev(delta, "delta"), x.numel(),
+                                   _storage(delta, "delta"), _stream()), "residual_add")
+    return x
+
+
+def swiglu(gate_up, out):
+    """out[r, i] = silu(gate_up[r, i]) * gate_up[r, I + i]."""
+    rows, two_i = gate_up.shape
+    if two_i % 2:
+        raise KernelError("swiglu: input width must be even")
+    inter = two_i // 2
+    _check(lib().cisr_swiglu(_dev(gate_up, "gate_up"), _dev(out, "out", gate_up.dtype, (rows, inter)), rows, inter,
+                             _storage(gate_up, "gate_up"), _stream()), "swiglu")
+    return out
+
+
+def rope_scatter(qkv, positions, slots, cos, sin, kcache, vcache, heads, kv_heads, dim, page_size):
+    """Rotate q (in place) and k of the fused projection rows, write k and v into
+    the cache at `slots`.  kcache/vcache None: q only (a layer reading another's cache).
+    qkv [T, (heads + 2 kv_heads) * dim] (or [T, heads * dim] without a cache);
+    cos/sin float [max_pos, rot/2]; cache [pages, kv_heads, page_size, dim]."""
+    rows = qkv.shape[0]
+    has_kv = kcache is not None
+    width = (heads + (2 * kv_heads if has_kv else 0)) * dim
+    dt = _storage(qkv, "qkv")
+    max_pos, half = cos.shape
+    rot = 2 * half
+    if rot > dim or rot <= 0:
+        raise KernelError(f"rope_scatter: rotary size {rot} does not fit head size {dim}")
+    kp = vp = sp = None
+    if has_kv:
+        pages = kcache.shape[0]
+        kp = _dev(kcache, "kcache", qkv.dtype, (pages, kv_heads, page_size, dim))
+        vp = _dev(vcache, "vcache", qkv.dtype, (pages, kv_heads, page_size, dim))
+        sp = _dev(slots, "slots", torch.int32, (rows,))
+    _check(lib().cisr_rope_scatter(_dev(qkv, "qkv", None, (rows, width)), _dev(positions, "positions", torch.int32, (rows,)),
+                                   sp, _dev(cos, "cos", torch.float32), _dev(sin, "sin", torch.float32, (max_pos, half)),
+                                   kp, vp, rows, heads, kv_heads, dim, rot, page_size, max_pos, int(has_kv), dt,
+                                   _stream()), "rope_scatter")
+
+
+def page_copy(pool, src, dst, slabs, pages_per_slab):
+    """pool viewed as [slabs, pages_per_slab, page]: page dst[i] := page src[i] in every slab."""
+    n = src.shape[0]
+    total = pool.numel() * pool.element_size()
+    if total % (slabs * pages_per_slab):
+        raise KernelError("page_copy: pool does not divide into slabs and pages")
+    slab_bytes = total // slabs
+    page_bytes = slab_bytes // pages_per_slab
+    _check(lib().cisr_page_copy(_dev(pool, "pool"), _dev(src, "src", torch.int32, (n,)), _dev(dst, "dst", torch.int32, (n,)),
+                                n, slabs, page_bytes, slab_bytes, _stream()), "page_copy")
+
+
+def f32_to_bf16(x, out):
+    _check(lib().cisr_f32_to_bf16(_dev(x, "x", torch.float32), _dev(out, "out", torch.bfloat16, x.shape), x.numel(),
+                                  _stream()), "f32_to_bf16")
+    return out
+
+
+def attention_rowwise(q, q_row_stride, kcache, vcache, tables, seg_of_row, positions, out, heads, kv_heads, dim,
+                      page_size, window, scale, splits=1, workspace=None):
+    """Each row attends to its request's cached keys lo..position.  q is a view
+    into a row-major buffer with `q_row_stride` elements per row; out [T, heads*dim]."""
+    rows = out.shape[0]
+    dt = _storage(out, "out")
+    if dim % 2 or dim > 256:
+        raise KernelError(f"attention: head size {dim} must be even and at most 256")
+    if heads % kv_heads:
+        raise KernelError(f"attention: {heads} query heads do not divide into {kv_heads} key heads")
+    pages = kcache.shape[0]
+    width = tables.shape[1]
+    if q.dtype != out.dtype or kcache.dtype != out.dtype:
+        raise KernelError("attention: q, cache and out must share a dtype")
+    if q.numel() < (rows - 1) * q_row_stride + heads * dim:
+        raise KernelError("attention: q buffer too small for its stride")
+    po = pm = None
+    if splits > 1:
+        if workspace is None:
+            raise KernelError("attention: split runs need a workspace")
+        part_o, part_ml = workspace
+        po = _dev(part_o, "part_o", torch.float32)
+        pm = _dev(part_ml, "part_ml", torch.float32)
+        if part_o.numel() < rows * heads * splits * dim or part_ml.numel() < rows * heads * splits * 2:
+            raise KernelError("attention: split workspace too small")
+    _check(lib().cisr_attn_rowwise(q.data_ptr(), q_row_stride, _dev(kcache, "kcache", None, (pages, kv_heads, page_size, dim)),
+                                   _dev(vcache, "vcache", None, (pages, kv_heads, page_size, dim)),
+                                   _dev(tables, "tables", torch.int32), _dev(seg_of_row, "seg_of_row", torch.int32, (rows,)),
+                                   _dev(positions, "positions", torch.int32, (rows,)), _dev(out, "out", None, (rows, heads * dim)),
+                                   po, pm, rows, heads, kv_heads, dim, page_size, width, int(window or 0), float(scale),
+                                   int(splits), dt, _stream()), "attention_rowwise")
+    return out
+
+
+def gemm(a, w, out, residual=None):
+    """out[M, N] = a[M, K] . w[N, K]^T (+ residual).  float operands run the true
+    32-bit kernel; bf16 operands run on the matrix cores with float accumulation.
+    out may be float or (bf16 operands only) bf16; residual is float and may be `out`."""
+    m, k = a.shape
+    n, k2 = w.shape
+    if k != k2:
+        raise KernelError(f"gemm: inner sizes differ ({k} vs {k2})")
+    if a.dtype != w.dtype:
+        raise KernelError(f"gemm: operand dtypes differ ({a.dtype} vs {w.dtype})")
+    if a.stride(1) != 1 or w.stride(1) != 1 or out.stride(1) != 1:
+        raise KernelError("gemm: rows must be contiguous")
+    if tuple(out.shape) != (m, n) or not out.is_cuda or not a.is_cuda or not w.is_cuda:
+        raise KernelError("gemm: bad output shape or device")
+    rp, ldr = None, 0
+    if residual is not None:
+        if residual.dtype != torch.float32 or out.dtype != torch.float32 or tuple(residual.shape) != (m, n) or residual.stride(1) != 1:
+            raise KernelError("gemm: residual needs float [M, N] and a float output")
+        rp, ldr = residual.data_ptr(), residual.stride(0)
+    if a.dtype == torch.float32:
+        if out.dtype != torch.float32:
+            raise KernelError("gemm: float operands need a float output")
+        code = lib().cisr_gemm_f32(a.data_ptr(), a.stride(0), w.data_ptr(), w.stride(0), out.data_ptr(), out.stride(0),
+                                   rp, ldr, m, n, k, _stream())
+    elif a.dtype == torch.bfloat16:
+        code = lib().cisr_gemm_bf16(a.data_ptr(), a.stride(0), w.data_ptr(), w.stride(0), out.data_ptr(), out.stride(0),
+                                    rp, ldr, m, n, k, _storage(out, "out"), _stream())
+    else:
+        raise KernelError(f"gemm: unsupported dtype {a.dtype}")
+    _check(code, "gemm")
+    return out
+
+
+def argmax(logits, out):
+    rows, vocab = logits.shape
+    _check(lib().cisr_argmax(_dev(logits, "logits", torch.float32), _dev(out, "out", torch.int32, (rows,)), rows, vocab,
+                             _stream()), "argmax")
+    return out
+
+
+def sample(logits, temperature, seeds, counters, out):
+    """Temperature sampling per row; temperature <= 0 is greedy.  seeds/counters int64 [R]."""
+    rows, vocab = logits.shape
+    _check(lib().cisr_sample(_dev(logits, "logits", torch.float32), _dev(temperature, "temperature", torch.float32, (rows,)),
+                             _dev(seeds, "seeds", torch.int64, (rows,)), _dev(counters, "counters", torch.int64, (rows,)),
+                             _dev(out, "out", torch.int32, (rows,)), rows, vocab, _stream()), "sample")
+    return out

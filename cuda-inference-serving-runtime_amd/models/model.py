@@ -1,0 +1,96 @@
+"""A decoder model as data: an embedding, a list of layers, the order in which
+they run, a final norm and an output head.
+
+`schedule` is a list of ScheduleEntry.  An entry names the layer to run; the
+same layer may be named twice (its weights are shared, every run has a cache
+of its own), and an entry may say `reads` = index of an earlier entry, in which
+case it keeps no cache and attends to what that entry wrote.  Cache *sites* are
+schedule indices.  The reference's model is the fixed loop of
+runtime/model.py:106-120; here the loop is over the schedule.
+"""
+from dataclasses import dataclass
+from typing import Optional
+
+
+@dataclass(frozen=True)
+class ScheduleEntry:
+    layer: int
+    reads: Optional[int] = None  # schedule index whose cache this run reads instead of keeping its own
+
+
+class Model:
+    def __init__(self, config, embedding, layers, final_norm, head, schedule=None):
+        self.config = config
+        self.embedding, self.layers, self.final_norm, self.head = embedding, list(layers), final_norm, head
+        self.schedule = list(schedule) if schedule is not None else [ScheduleEntry(i) for i in range(len(self.layers))]
+        for index, entry in enumerate(self.schedule):
+            if not 0 <= entry.layer < len(self.layers):
+                raise ValueError(f"schedule entry {index} names layer {entry.layer}, which does not exist")
+            if entry.reads is not None:
+                if not 0 <= entry.reads < index or self.schedule[entry.reads].reads is not None:
+                    raise ValueError(f"schedule entry {index} must read an earlier entry that keeps a cache")
+                if self.layers[entry.layer].mixer.cache_need() is not None:
+                    raise ValueError(f"schedule entry {index} reads another cache but its mixer keeps one")
+        self.dtype = None
+        self.device = None
+
+    # -- weights ------------------------------------------------------------
+    def parts(self):
+        return [self.embedding, *self.layers, self.final_norm, self.head]
+
+    def tensor_specs(self):
+        specs, seen = [], set()
+        for part in self.parts():
+            for spec in part.tensor_specs():
+                if spec.name in seen:
+                    raise ValueError(f"tensor {spec.name} is declared twice")
+                seen.add(spec.name)
+                specs.append(spec)
+        return specs
+
+    def bind(self, tensors, dtype, device):
+        self.dtype, self.device = dtype, device
+        for part in self.parts():
+            part.bind(tensors, dtype)
+            part.prepare(device, dtype)
+
+    # -- what the cache manager must provide ------------------------------------
+    def site_of(self, index):
+        entry = self.schedule[index]
+        return index if entry.reads is None else entry.reads
+
+    def cache_needs(self):
+        needs = {}
+        for index, entry in enumerate(self.schedule):
+            need = self.layers[entry.layer].mixer.cache_need()
+            if need is not None and entry.reads is None:
+                needs[index] = need
+        return needs
+
+    def state_needs(self):
+        needs = {}
+        for index, entry in enumerate(self.schedule):
+            need = self.layers[entry.layer].mixer.state_need()
+            if need is not None:
+                needs[index] = need
+        return needs
+
+    @property
+    def max_positions(self):
+        return self.config.max_position_embeddings
+
+    @property
+    def vocab_size(self):
+        return self.config.vocab_size
+
+    # -- the forward pass over one step's rows ------------------------------------
+    def forward(self, ctx):
+        """Logits [R, vocab] (float) at ctx.logit_rows; None if no row is wanted
+        (the layers still run: they fill the cache)."""
+        x = self.embedding.forward(ctx)
+        for index, entry in enumerate(self.schedule):
+            x = self.layers[entry.layer].forward(x, ctx, self.site_of(index))
+        if ctx.logit_rows.shape[0] == 0:
+            return None
+        h = self.final_norm.forward(x, ctx, rows=ctx.logit_rows, tag="final_norm")
+        return self.head.forward(h, ctx)

@@ -1,0 +1,89 @@
+"""Interfaces of the parts a layer is put together from, and their registry.
+
+A part knows its own sizes and constants (constructor parameters), the tensors
+it owns (names, shapes), and how to run on a step's rows.  It does not know
+which model it is in.  Kinds of part:
+
+  norm      forward(x_float[T, H], ctx, rows=None) -> activations [T or R, H]
+  position  tables(device) -> (cos, sin) float [max_pos, rot/2] used by mixers
+  mixer     forward(h[T, H], residual[T, H] float, ctx, site) -> residual
+  ffn       forward(h[T, H], residual[T, H] float, ctx) -> residual
+  block     forward(residual, ctx, site) -> residual  (the arrangement of the four)
+
+Mixers and feed-forwards add their result to the float residual stream
+themselves (their last matrix product does it in its epilogue) and return it.
+A mixer states what it keeps between steps: `cache_need()` (pages of keys and
+values) and/or `state_need()` (a fixed-size state per request), or neither.
+"""
+from ..weights.loader import TensorSpec
+
+_PARTS = {}
+
+KINDS = ("norm", "position", "mixer", "ffn", "block")
+
+
+def register_part(kind, name, factory):
+    if kind not in KINDS:
+        raise ValueError(f"unknown kind of part {kind!r}; kinds: {KINDS}")
+    if (kind, name) in _PARTS:
+        raise ValueError(f"{kind} {name!r} is already registered")
+    _PARTS[(kind, name)] = factory
+
+
+def unregister_part(kind, name):
+    _PARTS.pop((kind, name), None)
+
+
+def make_part(kind, family, /, **params):
+    """Build the part registered as (kind, family) with its own parameters."""
+    try:
+        factory = _PARTS[(kind, family)]
+    except KeyError:
+        known = sorted(n for k, n in _PARTS if k == kind)
+        raise KeyError(f"no {kind} named {family!r}; registered: {known}") from None
+    return factory(**params)
+
+
+class Part:
+    """Base of every part."""
+
+    def tensor_specs(self):
+        return []
+
+    def bind(self, tensors, dtype):
+        """Take the loaded tensors this part declared (dict by full name).
+        `dtype` is the compute dtype (torch.float32 or torch.bfloat16)."""
+
+    def prepare(self, device, dtype):
+        """Build tables and the like on the device (no weights involved)."""
+
+
+class Mixer(Part):
+    def cache_need(self):
+        return None
+
+    def state_need(self):
+        return None
+
+    def forward(self, h, residual, ctx, site):
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, h, residual, ctx):
+        raise NotImplementedError
+
+
+def matrix_operand(t, dtype):
+    """A stored matrix as a GEMM operand of the compute dtype.  bf16 -> float
+    widening is exact; a 32-bit matrix run in bf16 is rounded to nearest even by
+    the conversion kernel."""
+    import torch
+    from ..kernels import ops
+    if t.dtype == dtype:
+        return t.contiguous()
+    if dtype == torch.float32:
+        return t.to(torch.float32).contiguous()
+    if t.dtype == torch.float32 and dtype == torch.bfloat16:
+        return ops.f32_to_bf16(t.contiguous(), torch.empty_like(t, dtype=torch.bfloat16))
+    raise TypeError(f"cannot use a {t.dtype} matrix in {dtype} arithmetic")

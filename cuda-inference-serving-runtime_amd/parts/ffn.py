@@ -1,0 +1,37 @@
+"""Gated feed-forward (SwiGLU): x + (silu(h Wg^T) * (h Wu^T)) Wd^T
+(reference: runtime/model.py:116-119).  Gate and up run as one product against
+the concatenated weight [gate; up]."""
+import torch
+
+from ..kernels import ops
+from .base import FeedForward, TensorSpec, matrix_operand, register_part
+
+
+class GatedMLP(FeedForward):
+    def __init__(self, name, hidden, intermediate, activation="silu"):
+        if activation != "silu":
+            raise ValueError(f"activation {activation!r}: only silu has a kernel")
+        self.name, self.hidden, self.intermediate = name, hidden, intermediate
+        self.w_gate_up = self.w_down = None
+
+    def tensor_specs(self):
+        n, H, I = self.name, self.hidden, self.intermediate
+        return [TensorSpec(f"{n}.gate_proj.weight", (I, H)), TensorSpec(f"{n}.up_proj.weight", (I, H)),
+                TensorSpec(f"{n}.down_proj.weight", (H, I))]
+
+    def bind(self, tensors, dtype):
+        gate = matrix_operand(tensors[f"{self.name}.gate_proj.weight"], dtype)
+        up = matrix_operand(tensors[f"{self.name}.up_proj.weight"], dtype)
+        self.w_gate_up = torch.cat([gate, up], dim=0).contiguous()
+        self.w_down = matrix_operand(tensors[f"{self.name}.down_proj.weight"], dtype)
+
+    def forward(self, h, residual, ctx):
+        T = h.shape[0]
+        gu = ctx.buffer("ffn.gate_up", (T, 2 * self.intermediate), ctx.dtype)
+        ops.gemm(h, self.w_gate_up, gu)
+        act = ctx.buffer("ffn.act", (T, self.intermediate), ctx.dtype)
+        ops.swiglu(gu, act)
+        return ops.gemm(act, self.w_down, residual, residual=residual)
+
+
+register_part("ffn", "gated_mlp", GatedMLP)

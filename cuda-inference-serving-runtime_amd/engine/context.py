@@ -34,6 +34,7 @@ class StepContext:
         self.segments = []        # host: [(request, start, count)]
         self.max_context = 0      # host: largest position + 1 among the rows
         self.decode_only = False  # host: every segment brings exactly one token
+        self.fixed_splits = None  # set when the step runs as a captured program
 
     def buffer(self, name, shape, dtype):
         return self.runner.workspace.get(name, shape, dtype)

@@ -33,11 +33,15 @@ _TORCH_OF = {"float32": torch.float32, "bfloat16": torch.bfloat16, "int32": torc
 
 
 class ModelRunner:
-    def __init__(self, model, n_pages, page_size=16, max_requests=64, device="cuda:0"):
+    def __init__(self, model, n_pages, page_size=16, max_requests=64, device="cuda:0", execution="eager"):
         if not torch.cuda.is_available():
             raise RuntimeError("no GPU: the engine runs on an MI355X only and has no CPU path")
         ops.lib()  # fail now if the kernel library is missing
+        if execution not in ("eager", "graph"):
+            raise ValueError(f"execution {execution!r} is not eager or graph")
         self.model = model
+        self.execution = execution
+        self.programs, self.program_capacity = {}, 16
         self.device = torch.device(device)
         self.page_size = page_size
         self.max_requests = max_requests
@@ -105,30 +109,49 @@ class ModelRunner:
         """Float logits [sum(len(want)), vocab] on the GPU (valid until the next step)."""
         self.check(entries)
         done = self.cache.append_many([(e.request, len(e.tokens)) for e in entries])  # OutOfPages changes nothing
-        ctx = self._context(entries, done)
         self.steps += 1
+        key = self._program_key(entries, done) if self.execution == "graph" else None
+        if key is not None:
+            return self._run_program(key, entries, done)
+        ctx = self._context(entries, done)
         logits = self.model.forward(ctx)
         if logits is None:
             return torch.empty((0, self.model.vocab_size), dtype=torch.float32, device=self.device)
         return logits
 
-    def _context(self, entries, done):
-        T = sum(len(e.tokens) for e in entries)
-        S = len(entries)
-        R = sum(len(e.want) for e in entries)
-        W = self.table_width
-        G = len(self.cache.groups)
-        # one packed int32 upload: tokens, positions, seg_of_row, seg_start, seg_first_pos, state_slots,
-        # logit_rows, then per group slots and tables
+    def _layout(self, T, S, R):
+        """Offsets of the packed int32 metadata: tokens, positions, seg_of_row, seg_start, seg_first_pos,
+        state_slots, logit_rows, then per group slots and tables."""
+        W, G = self.table_width, len(self.cache.groups)
         sizes = [T, T, T, S + 1, S, S, R] + [T, S * W] * G
-        offsets = np.concatenate(([0], np.cumsum(sizes)))
-        host = self._stage(int(offsets[-1]))
+        return np.concatenate(([0], np.cumsum(sizes))).astype(np.int64)
+
+    def _context(self, entries, done, pad=None, device_buffer=None):
+        """Build the step's metadata on the host, upload it in one copy and wrap it.
+        `pad` = (T, S, R) pads the batch with inert rows (for captured programs):
+        token 0 at position 0, no segment, no cache slot."""
+        n_rows = sum(len(e.tokens) for e in entries)
+        n_want = sum(len(e.want) for e in entries)
+        T, S, R = pad if pad is not None else (n_rows, len(entries), n_want)
+        W, G = self.table_width, len(self.cache.groups)
+        offsets = self._layout(T, S, R)
+        total = int(offsets[-1])
+        host = self._stage(total)
         arr = host.numpy()
         tokens, positions, seg_of_row, seg_start, seg_first, state_slots, logit_rows = (
             arr[offsets[i]:offsets[i + 1]] for i in range(7))
-        row = 0
-        out_row = 0
-        max_context = 0
+        if pad is not None:
+            tokens[:] = 0
+            positions[:] = 0
+            seg_of_row[:] = -1
+            seg_start[:] = n_rows
+            seg_first[:] = 0
+            state_slots[:] = 0
+            logit_rows[:] = 0
+            for g in range(G):
+                arr[offsets[7 + 2 * g]:offsets[8 + 2 * g]] = -1
+                arr[offsets[8 + 2 * g]:offsets[9 + 2 * g]] = -1
+        row = out_row = max_context = 0
         for s, (e, d) in enumerate(zip(entries, done)):
             n = len(e.tokens)
             tokens[row:row + n] = e.tokens
@@ -149,8 +172,8 @@ class ModelRunner:
                 trow[len(table):] = -1
             row += n
             max_context = max(max_context, d.start + n)
-        seg_start[S] = T
-        dev = self._upload(host, int(offsets[-1]))
+        seg_start[len(entries):] = n_rows
+        dev = self._upload(host, total, device_buffer)
 
         def view(i, shape=None):
             t = dev[int(offsets[i]):int(offsets[i + 1])]
@@ -183,24 +206,72 @@ class ModelRunner:
         self._current = entry
         return entry[0]
 
-    def _upload(self, host, n):
+    def _upload(self, host, n, device_buffer=None):
         entry = self._current
-        entry[1][:n].copy_(host[:n], non_blocking=True)
+        target = entry[1] if device_buffer is None else device_buffer
+        target[:n].copy_(host[:n], non_blocking=True)
         entry[2] = torch.cuda.Event()
         entry[2].record()
-        return entry[1]
+        return target
+
+    # -- captured programs (decode steps) -------------------------------------------
+    def _program_key(self, entries, done):
+        """Decode-only steps that want every row's logits run as a captured graph,
+        keyed by the padded batch size and the attention split count."""
+        if not all(d.count == 1 and list(e.want) == [0] for e, d in zip(entries, done)):
+            return None
+        batch = 1 << (len(entries) - 1).bit_length()
+        context = 1 << (max(d.start + 1 for d in done) - 1).bit_length()
+        return (batch, self._splits(batch * self._max_heads(), context))
+
+    def _max_heads(self):
+        return max((getattr(layer.mixer, "heads", 1) for layer in self.model.layers), default=1)
+
+    def _run_program(self, key, entries, done):
+        batch, splits = key
+        program = self.programs.get(key)
+        if program is None:
+            total = int(self._layout(batch, batch, batch)[-1])
+            program = {"meta": torch.zeros(total, dtype=torch.int32, device=self.device), "graph": None, "runs": 0}
+            self.programs[key] = program
+            while len(self.programs) > self.program_capacity:
+                oldest = next(iter(self.programs))
+                torch.cuda.synchronize()
+                del self.programs[oldest]
+        else:
+            self.programs[key] = self.programs.pop(key)  # most recently used last
+        ctx = self._context(entries, done, pad=(batch, batch, batch), device_buffer=program["meta"])
+        ctx.fixed_splits = splits
+        if program["graph"] is None and program["runs"] >= 1:
+            # the first run was eager and allocated every buffer; capture launches nothing
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                program["logits"] = self.model.forward(ctx)
+            program["graph"] = graph
+        if program["graph"] is not None:
+            program["graph"].replay()
+            logits = program["logits"]
+        else:
+            logits = self.model.forward(ctx)
+        program["runs"] += 1
+        return logits[:len(entries)]
 
     # -- attention dispatch -------------------------------------------------------
     def attention(self, ctx, q, q_row_stride, kcache, vcache, view, out, heads, kv_heads, head_dim, window, scale):
         rows = out.shape[0]
         span = ctx.max_context if not window else min(ctx.max_context, window)
-        splits = 1
-        waves = rows * heads
-        if waves < 2048 and span > 256:
-            splits = int(min(32, -(-span // 256), max(1, 4096 // waves)))
+        splits = ctx.fixed_splits if ctx.fixed_splits is not None else self._splits(rows * heads, span)
         workspace = None
         if splits > 1:
             workspace = (ctx.buffer("attn.part_o", (rows * heads * splits * head_dim,), torch.float32),
                          ctx.buffer("attn.part_ml", (rows * heads * splits * 2,), torch.float32))
         ops.attention_rowwise(q, q_row_stride, kcache, vcache, view.tables, ctx.seg_of_row, ctx.positions, out,
                               heads, kv_heads, head_dim, view.page_size, window, scale, splits, workspace)
+
+    @staticmethod
+    def _splits(waves, span):
+        """How many ways a row's keys are split among wavefronts: enough to fill the
+        GPU when the batch alone does not, never finer than 256 keys a split."""
+        if waves >= 2048 or span <= 256:
+            return 1
+        return int(min(32, -(-span // 256), max(1, 4096 // waves)))

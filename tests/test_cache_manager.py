@@ -1,0 +1,193 @@
+"""The cache manager on the host: no page lost, held twice or freed twice, under
+random orders of requests; copy-on-write; windows giving pages back; state slots."""
+import random
+
+import pytest
+
+from runtime.cache import CacheManager, KVNeed, OutOfPages, StateNeed, StateSlots
+
+
+def manager(pages=8, page_size=4, sites=2, window=None, max_requests=8, **kw):
+    needs = {i: KVNeed(2, 16, None) for i in range(sites)}
+    if window:
+        needs[sites] = KVNeed(2, 16, window)
+    return CacheManager(needs, pages, page_size, max_requests, **kw)
+
+
+def test_append_slots_follow_the_block_table():
+    m = manager()
+    m.create("a")
+    (d,) = m.append_many([("a", 6)])
+    assert d.start == 0 and d.count == 6 and m.length("a") == 6
+    table = m.table(0, "a")
+    assert len(table) == 2
+    assert d.slots[0] == [table[i // 4] * 4 + i % 4 for i in range(6)]
+    (d,) = m.append_many([("a", 3)])
+    assert d.start == 6 and d.slots[0][:2] == [table[1] * 4 + 2, table[1] * 4 + 3] and len(m.table(0, "a")) == 3
+    m.check()
+
+
+def test_sites_with_equal_needs_share_one_group():
+    m = manager(sites=3, window=5)
+    assert len(m.groups) == 2 and len(m.groups[0].sites) == 3 and m.groups[1].need.window == 5
+    assert m.group_of_site[2] == (0, 2) and m.group_of_site[3] == (1, 0)
+
+
+def test_exhaustion_is_atomic_and_duplicates_are_rejected():
+    # reference tests/test_cache.py:20-31 and tests/test_model.py:42-46
+    m = manager(pages=2, page_size=2)
+    m.create("a"); m.create("b")
+    with pytest.raises(ValueError):
+        m.create("a")
+    m.append_many([("a", 3)])
+    before = (m.length("a"), m.length("b"), list(m.table(0, "a")), m.free_pages())
+    with pytest.raises(OutOfPages):
+        m.append_many([("a", 1), ("b", 1)])   # a fits in its page, b needs a third page
+    assert before == (m.length("a"), m.length("b"), list(m.table(0, "a")), m.free_pages())
+    m.check()
+    with pytest.raises(ValueError):
+        m.append_many([("a", 1), ("a", 1)])
+    with pytest.raises(KeyError):
+        m.append_many([("zzz", 1)])
+
+
+def test_fork_shares_pages_and_copies_a_partial_page_on_write():
+    # reference tests/test_cache.py:7-18
+    copies = []
+    m = manager(pages=3, page_size=2, sites=1, copy_pages=lambda g, c: copies.extend(c))
+    m.create("a")
+    m.append_many([("a", 1)])
+    m.fork("a", "b")
+    assert m.table(0, "a") == m.table(0, "b") and m.groups[0].pool.refs[m.table(0, "a")[0]] == 2
+    (d,) = m.append_many([("b", 1)])
+    assert m.table(0, "a") != m.table(0, "b") and m.length("a") == 1 and m.length("b") == 2
+    assert copies == [(m.table(0, "a")[0], m.table(0, "b")[0])]
+    assert d.slots[0] == [m.table(0, "b")[0] * 2 + 1]
+    m.check()
+    m.release("a"); m.release("b"); m.check()
+    assert m.free_pages() == [3]
+
+
+def test_fork_at_a_page_edge_copies_nothing():
+    copies = []
+    m = manager(pages=4, page_size=2, sites=1, copy_pages=lambda g, c: copies.extend(c))
+    m.create("a"); m.append_many([("a", 2)]); m.fork("a", "b")
+    m.append_many([("b", 3)]); m.append_many([("a", 1)])
+    assert not copies and m.table(0, "a")[0] == m.table(0, "b")[0] and m.table(0, "a")[1] != m.table(0, "b")[1]
+    m.check()
+
+
+def test_pages_are_reused_lowest_first_after_release():
+    m = manager(pages=4, page_size=2, sites=1)
+    m.create("a"); m.append_many([("a", 8)])
+    with pytest.raises(OutOfPages):
+        m.create("b"); m.append_many([("b", 1)])
+    m.release("a")
+    assert m.free_pages() == [4]
+    m.append_many([("b", 5)])
+    assert sorted(m.table(0, "b")) == sorted(set(m.table(0, "b"))) and len(m.table(0, "b")) == 3
+    m.check()
+
+
+def test_window_gives_pages_back_once_passed():
+    m = manager(pages=6, page_size=4, sites=1, window=6)
+    m.create("a")
+    full, win = 0, 1
+    m.append_many([("a", 4)])
+    for _ in range(16):
+        m.append_many([("a", 1)])
+        m.check()
+    # length 20: the next query (position 20) sees keys 15..20, i.e. logical pages 3.. -> pages 0,1,2 are back
+    assert m.table(win, "a")[:3] == [-1, -1, -1] and all(p >= 0 for p in m.table(win, "a")[3:])
+    assert all(p >= 0 for p in m.table(full, "a"))
+    assert m.groups[win].pool.used == 2 and m.groups[full].pool.used == 5
+    # a long portion: pages behind the window of its FIRST token are given back before it is placed
+    m.release("a"); m.create("b")
+    m.append_many([("b", 9)])
+    assert m.table(win, "b") .count(-1) == 0       # nothing passed yet when the portion started
+    m.append_many([("b", 2)])
+    assert m.table(win, "b")[0] == -1 and m.table(win, "b")[1] >= 0  # first visible key is 9-6+1 = 4: page 0 is passed
+    m.check()
+
+
+def test_window_group_never_needs_more_than_window_plus_portion():
+    m = manager(pages=4, page_size=4, sites=0, window=8)
+    m.create("a")
+    for _ in range(50):            # 200 tokens through 4 pages of 4
+        m.append_many([("a", 4)])
+        m.check()
+    assert m.length("a") == 200 and m.groups[0].pool.used <= 3
+
+
+def test_state_slots():
+    s = StateSlots(2)
+    assert s.acquire("a") == 0 and s.acquire("b") == 1
+    with pytest.raises(MemoryError):
+        s.acquire("c")
+    with pytest.raises(ValueError):
+        s.acquire("a")
+    s.release("a"); s.check()
+    assert s.acquire("c") == 0
+    s.check()
+
+
+def test_state_is_zeroed_on_create_and_copied_on_fork():
+    log = []
+    m = CacheManager({0: KVNeed(1, 8)}, 4, 4, 3, state_needs={1: StateNeed((5,), "float32")},
+                     allocate_state=lambda n, shape, dt: ("state", n, shape, dt),
+                     zero_state=lambda t, s: log.append(("zero", s)), copy_state=lambda t, a, b: log.append(("copy", a, b)))
+    assert m.state_storage[1] == ("state", 3, (5,), "float32")
+    m.create("a"); m.fork("a", "b")
+    assert log == [("zero", 0), ("copy", 0, 1)]
+    (d,) = m.append_many([("b", 1)])
+    assert d.state_slot == 1
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_orders_keep_every_page_accounted_for(seed):
+    rng = random.Random(seed)
+    m = manager(pages=12, page_size=4, sites=2, window=rng.choice([None, 3, 9]), max_requests=5)
+    live, counter = {}, 0
+    for _ in range(400):
+        action = rng.random()
+        if action < 0.25 and len(live) < 5:
+            name = f"r{counter}"; counter += 1
+            if live and rng.random() < 0.3:
+                src = rng.choice(list(live))
+                m.fork(src, name); live[name] = live[src]
+            else:
+                m.create(name); live[name] = 0
+        elif action < 0.85 and live:
+            picks = rng.sample(list(live), rng.randint(1, len(live)))
+            items = [(r, rng.choice([1, 1, 1, 2, 5, 9])) for r in picks]
+            snapshot = ({r: m.length(r) for r in live}, m.free_pages(),
+                        [{r: list(t) for r, t in g.tables.items()} for g in m.groups])
+            try:
+                done = m.append_many(items)
+            except OutOfPages:
+                after = ({r: m.length(r) for r in live}, m.free_pages(),
+                         [{r: list(t) for r, t in g.tables.items()} for g in m.groups])
+                assert snapshot[0] == after[0], "a failed step changed a length"
+                # a window may have given pages back (always valid); full groups are untouched
+                for g, before_t, after_t in zip(m.groups, snapshot[2], after[2]):
+                    if g.need.window is None:
+                        assert before_t == after_t
+                victim = rng.choice(list(live)); m.release(victim); del live[victim]
+            else:
+                for (r, n), d in zip(items, done):
+                    assert d.start == live[r] and d.count == n
+                    live[r] += n
+                    for gid, g in enumerate(m.groups):
+                        assert all(0 <= s < g.pool.n_pages * 4 for s in d.slots[gid])
+                        assert len(set(d.slots[gid])) == n
+                # no slot of this step is shared between two requests
+                for gid in range(len(m.groups)):
+                    flat = [s for d in done for s in d.slots[gid]]
+                    assert len(flat) == len(set(flat))
+        elif live:
+            victim = rng.choice(list(live)); m.release(victim); del live[victim]
+        m.check()
+    for r in list(live):
+        m.release(r)
+    m.check()
+    assert all(free == 12 for free in m.free_pages()) and len(m.slots.free) == 5

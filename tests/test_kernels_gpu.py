@@ -1,0 +1,369 @@
+"""Each HIP kernel alone against a plain float64 reference, at sizes other than
+the engine's tiny configurations (tails, non powers of two, every head size)."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import plain_llama as P
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from runtime.kernels import ops as o
+    o.lib()
+    return o
+
+
+def tol(dtype):
+    return dict(rtol=2e-5, atol=2e-6) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+
+
+def rnd(*shape, dtype=torch.float32, seed=0, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).to(DEV)
+
+
+def f64(t):
+    return t.detach().double().cpu().numpy()
+
+
+def test_library_is_loaded_from_the_tree(ops):
+    from runtime.kernels import library
+    assert library.loaded_path() and "libcisr_kernels_" in library.loaded_path()
+
+
+def test_bf16_rounding_vector(ops):
+    # reference tests/test_precision.py:65-70: specials kept, -0 keeps its sign, ties to even
+    values = torch.tensor([0., -0., math.inf, -math.inf, math.nan, 1., 1.00390625, 1.01171875], device=DEV)
+    out = ops.f32_to_bf16(values, torch.empty(8, dtype=torch.bfloat16, device=DEV)).float().cpu().numpy()
+    assert np.isnan(out[4])
+    np.testing.assert_array_equal(out[:4], values.cpu().numpy()[:4])
+    assert np.signbit(out[1]) and out[5] == 1.0 and out[6] == 1.0   # 1 + 2^-8 is a tie: rounds to even (1.0)
+    assert out[7] == 1.015625                                        # 1 + 3*2^-8 ties up to the even 1 + 2^-6
+    x = rnd(1000, seed=3)
+    np.testing.assert_array_equal(ops.f32_to_bf16(x, torch.empty(1000, dtype=torch.bfloat16, device=DEV)).float().cpu().numpy(),
+                                  x.bfloat16().float().cpu().numpy())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_embedding(ops, dtype):
+    table = rnd(37, 70, dtype=dtype)
+    ids = torch.tensor([0, 36, 5, 5, 17], dtype=torch.int32, device=DEV)
+    out = ops.embedding(ids, table, torch.empty(5, 70, device=DEV))
+    np.testing.assert_array_equal(f64(out), f64(table)[ids.cpu().numpy()])
+
+
+@pytest.mark.parametrize("dim", [10, 64, 130, 576, 4100])
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+def test_rmsnorm(ops, dim, out_dtype):
+    # reference tests/test_cuda.py:28-36 (dims 10/64/130/512)
+    x, w = rnd(7, dim, seed=1, scale=3.0), rnd(dim, seed=2)
+    for eps in (1e-5, 1e-2):
+        out = ops.rmsnorm(x, w, torch.empty(7, dim, dtype=out_dtype, device=DEV), eps)
+        np.testing.assert_allclose(f64(out), P.rmsnorm(f64(x), f64(w), eps), **tol(out_dtype))
+    rows = torch.tensor([6, 0, 3], dtype=torch.int32, device=DEV)
+    out = ops.rmsnorm(x, w, torch.empty(3, dim, dtype=out_dtype, device=DEV), 1e-6, rows)
+    np.testing.assert_allclose(f64(out), P.rmsnorm(f64(x)[[6, 0, 3]], f64(w), 1e-6), **tol(out_dtype))
+    assert (ops.rmsnorm(torch.zeros(2, dim, device=DEV), w, torch.empty(2, dim, dtype=out_dtype, device=DEV), 1e-5) == 0).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_add_rmsnorm_and_residual_add(ops, dtype):
+    x, d, w = rnd(5, 130, seed=1), rnd(5, 130, dtype=dtype, seed=2), rnd(130, seed=3)
+    want_sum = f64(x) + f64(d)
+    x1 = x.clone()
+    out = ops.add_rmsnorm(x1, d, w, torch.empty(5, 130, dtype=dtype, device=DEV), 1e-5)
+    np.testing.assert_allclose(f64(x1), want_sum, rtol=1e-6, atol=1e-6)       # the sum stays float
+    np.testing.assert_allclose(f64(out), P.rmsnorm(want_sum, f64(w), 1e-5), **tol(dtype))
+    x2 = x.clone()
+    ops.residual_add(x2, d)
+    np.testing.assert_allclose(f64(x2), want_sum, rtol=1e-6, atol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_swiglu(ops, dtype):
+    gu = rnd(6, 2 * 173, dtype=dtype, scale=4.0)
+    gu[0, 0], gu[0, 1], gu[0, 2] = 0.0, 60.0, -60.0
+    out = ops.swiglu(gu, torch.empty(6, 173, dtype=dtype, device=DEV))
+    np.testing.assert_allclose(f64(out), P.swiglu(f64(gu)[:, :173], f64(gu)[:, 173:]), **tol(dtype))
+    assert torch.isfinite(out.float()).all() and out[0, 0] == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("heads, kv_heads, dim, theta", [(4, 2, 10, 1e4), (6, 6, 24, 5e5), (9, 3, 64, 1e5), (2, 1, 256, 1e4)])
+def test_rope_scatter(ops, dtype, heads, kv_heads, dim, theta):
+    # reference tests/test_cuda.py:37-39 (D=10, positions 0/17/500)
+    from runtime.parts import RotaryEmbedding
+    rope = RotaryEmbedding(dim, theta, 600)
+    rope.prepare(DEV, dtype)
+    cos, sin = rope.tables()
+    T, P_, pages = 5, 4, 6
+    qkv = rnd(T, (heads + 2 * kv_heads) * dim, dtype=dtype, seed=4)
+    ref = f64(qkv)
+    pos = [0, 17, 500, 599, 3]
+    slots = [5, 0, 22, -1, 9]
+    kc = torch.full((pages, kv_heads, P_, dim), 7.0, dtype=dtype, device=DEV)
+    vc = torch.full((pages, kv_heads, P_, dim), 7.0, dtype=dtype, device=DEV)
+    ops.rope_scatter(qkv, torch.tensor(pos, dtype=torch.int32, device=DEV), torch.tensor(slots, dtype=torch.int32, device=DEV),
+                     cos, sin, kc, vc, heads, kv_heads, dim, P_)
+    q_ref = P.rope(ref[:, :heads * dim].reshape(T, heads, dim), pos, theta)
+    k_ref = P.rope(ref[:, heads * dim:(heads + kv_heads) * dim].reshape(T, kv_heads, dim), pos, theta)
+    v_ref = ref[:, (heads + kv_heads) * dim:].reshape(T, kv_heads, dim)
+    np.testing.assert_allclose(f64(qkv)[:, :heads * dim].reshape(T, heads, dim), q_ref, **tol(dtype))
+    kc64, vc64 = f64(kc), f64(vc)
+    written = set()
+    for t, s in enumerate(slots):
+        if s < 0:
+            continue
+        np.testing.assert_allclose(kc64[s // P_, :, s % P_], k_ref[t], **tol(dtype))
+        np.testing.assert_array_equal(vc64[s // P_, :, s % P_], v_ref[t])
+        written.add(s)
+    for s in range(pages * P_):
+        if s not in written:   # nothing else is touched, a negative slot writes nothing
+            assert (kc64[s // P_, :, s % P_] == 7).all() and (vc64[s // P_, :, s % P_] == 7).all()
+
+
+def test_rope_partial_rotation_and_identity(ops):
+    from runtime.parts import RotaryEmbedding, NoPosition
+    dim, rot = 16, 8
+    rope = RotaryEmbedding(dim, 1e4, 50, rotary_dim=rot); rope.prepare(DEV, torch.float32)
+    qkv = rnd(3, 3 * dim, seed=9); ref = f64(qkv)
+    kc = torch.zeros(1, 1, 4, dim, device=DEV); vc = torch.zeros_like(kc)
+    pos = [3, 40, 7]
+    ops.rope_scatter(qkv, torch.tensor(pos, dtype=torch.int32, device=DEV), torch.tensor([0, 1, 2], dtype=torch.int32, device=DEV),
+                     *rope.tables(), kc, vc, 1, 1, dim, 4)
+    q = ref[:, :dim].reshape(3, 1, dim)
+    want = np.concatenate([P.rope(q[..., :rot], pos, 1e4), q[..., rot:]], -1)
+    np.testing.assert_allclose(f64(qkv)[:, :dim].reshape(3, 1, dim), want, rtol=2e-5, atol=2e-6)
+    k = ref[:, dim:2 * dim].reshape(3, 1, dim)
+    want_k = np.concatenate([P.rope(k[..., :rot], pos, 1e4), k[..., rot:]], -1)
+    np.testing.assert_allclose(f64(kc)[0, :, :3].transpose(1, 0, 2), want_k, rtol=2e-5, atol=2e-6)
+    none = NoPosition(dim, 50); none.prepare(DEV, torch.float32)
+    qkv2 = rnd(3, 3 * dim, seed=9)
+    ops.rope_scatter(qkv2, torch.tensor(pos, dtype=torch.int32, device=DEV), torch.tensor([0, 1, 2], dtype=torch.int32, device=DEV),
+                     *none.tables(), kc, vc, 1, 1, dim, 4)
+    np.testing.assert_array_equal(f64(qkv2), ref)
+
+
+def paged_case(heads, kv_heads, dim, page_size, lengths, dtype, seed=0, pages=None, sharpen=None):
+    """A cache with scattered pages holding `lengths[i]` keys for request i, one
+    query row per request at its last position plus extra rows at earlier positions."""
+    rng = np.random.default_rng(seed)
+    per = [-(-n // page_size) for n in lengths]
+    pages = pages or sum(per) + 3
+    order = rng.permutation(pages).tolist()
+    width = max(per) + 2
+    tables = np.full((len(lengths), width), -1, np.int32)
+    K = rng.standard_normal((pages, kv_heads, page_size, dim)).astype(np.float32)
+    V = rng.standard_normal((pages, kv_heads, page_size, dim)).astype(np.float32)
+    for i, n in enumerate(lengths):
+        for j in range(per[i]):
+            tables[i, j] = order.pop()
+    rows = []  # (segment, position)
+    for i, n in enumerate(lengths):
+        rows.append((i, n - 1))
+        if n > 3:
+            rows.append((i, n // 2))
+            rows.append((i, 0))
+    q = rng.standard_normal((len(rows), heads, dim)).astype(np.float32)
+    if sharpen is not None:   # one far key gets a score that stands out
+        seg, key_pos = sharpen
+        page, off = tables[seg, key_pos // page_size], key_pos % page_size
+        r = next(i for i, (s, p) in enumerate(rows) if s == seg and p == lengths[seg] - 1)
+        group = heads // kv_heads
+        for h in range(heads):   # heads of one group ask the same question, the key answers it
+            q[r, h] = q[r, (h // group) * group]
+            K[page, h // group, off] = q[r, h] * 4.0
+    kt = torch.from_numpy(K).to(dtype).to(DEV)
+    vt = torch.from_numpy(V).to(dtype).to(DEV)
+    qt = torch.from_numpy(q).to(dtype).to(DEV)
+    return qt, kt, vt, torch.from_numpy(tables).to(DEV), rows
+
+
+def reference_attention(qt, kt, vt, tables, rows, page_size, window=None, scale=None):
+    q, K, V, tab = f64(qt), f64(kt), f64(vt), tables.cpu().numpy()
+    out = []
+    for r, (seg, pos) in enumerate(rows):
+        lo = 0 if not window else max(0, pos + 1 - window)
+        ks = np.stack([K[tab[seg, t // page_size], :, t % page_size] for t in range(lo, pos + 1)])
+        vs = np.stack([V[tab[seg, t // page_size], :, t % page_size] for t in range(lo, pos + 1)])
+        qq = q[r] if scale is None else q[r] * scale * math.sqrt(q.shape[-1])
+        out.append(P.attention_one_query(qq, ks, vs))
+    return np.stack(out)
+
+
+def run_rowwise(ops, qt, kt, vt, tables, rows, page_size, splits=1, window=None, scale=None):
+    T, heads, dim = qt.shape
+    kv_heads = kt.shape[1]
+    seg = torch.tensor([r[0] for r in rows], dtype=torch.int32, device=DEV)
+    pos = torch.tensor([r[1] for r in rows], dtype=torch.int32, device=DEV)
+    out = torch.empty(T, heads * dim, dtype=qt.dtype, device=DEV)
+    ws = (torch.empty(T * heads * splits * dim, device=DEV), torch.empty(T * heads * splits * 2, device=DEV))
+    ops.attention_rowwise(qt.reshape(T, heads * dim), heads * dim, kt, vt, tables, seg, pos, out, heads, kv_heads, dim,
+                          page_size, window, scale if scale is not None else 1 / math.sqrt(dim), splits, ws)
+    return f64(out).reshape(T, heads, dim)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("heads, kv_heads, dim, page_size", [
+    (4, 2, 10, 4), (6, 6, 24, 8), (9, 3, 64, 16), (8, 1, 128, 64), (2, 2, 256, 1), (5, 5, 16, 3)])
+def test_attention_rowwise(ops, dtype, heads, kv_heads, dim, page_size):
+    # reference tests/test_cuda.py:41-63: head sizes 10..256, interleaved pages, grouped heads,
+    # split counts 1/3/16 where 16 exceeds the shorter request's tokens
+    qt, kt, vt, tables, rows = paged_case(heads, kv_heads, dim, page_size, [17, 7, 1, 130], dtype, seed=dim)
+    want = reference_attention(qt, kt, vt, tables, rows, page_size)
+    for splits in (1, 3, 16):
+        got = run_rowwise(ops, qt, kt, vt, tables, rows, page_size, splits)
+        np.testing.assert_allclose(got, want, **tol(dtype), err_msg=f"splits={splits}")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_window_scale_and_padding_rows(ops, dtype):
+    qt, kt, vt, tables, rows = paged_case(4, 2, 32, 8, [70, 9], dtype, seed=11)
+    for window in (1, 8, 9, 33):   # the edge: exactly `window` keys lo..pos
+        want = reference_attention(qt, kt, vt, tables, rows, 8, window=window)
+        for splits in (1, 4):
+            np.testing.assert_allclose(run_rowwise(ops, qt, kt, vt, tables, rows, 8, splits, window=window), want, **tol(dtype))
+    want = reference_attention(qt, kt, vt, tables, rows, 8, scale=0.3)
+    np.testing.assert_allclose(run_rowwise(ops, qt, kt, vt, tables, rows, 8, 1, scale=0.3), want, **tol(dtype))
+    # a row without a segment (padding) gives zeros and touches nothing else
+    rows2 = list(rows); rows2[1] = (-1, 0)
+    got = run_rowwise(ops, qt, kt, vt, tables, rows2, 8, 2)
+    assert (got[1] == 0).all()
+    np.testing.assert_allclose(got[0], reference_attention(qt, kt, vt, tables, rows, 8)[0], **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_finds_one_far_key_among_hundreds(ops, dtype):
+    # key 3 of 700 carries a score far above the rest: the output must be its value row
+    qt, kt, vt, tables, rows = paged_case(4, 2, 64, 16, [700, 40], dtype, seed=5, sharpen=(0, 3))
+    want = reference_attention(qt, kt, vt, tables, rows, 16)
+    page, off = tables[0, 0].item(), 3
+    np.testing.assert_allclose(want[0, 0], f64(vt)[page, 0, off], atol=1e-6)   # the case is what it claims to be
+    for splits in (1, 8):
+        np.testing.assert_allclose(run_rowwise(ops, qt, kt, vt, tables, rows, 16, splits), want, **tol(dtype))
+
+
+def test_attention_equal_large_scores_give_the_mean(ops):
+    # reference tests/test_reference.py:7-13 on the kernel
+    heads, kv, dim, n = 4, 2, 8, 3
+    q = torch.full((1, heads * dim), 1e3, device=DEV)
+    kc = torch.full((1, kv, 4, dim), 1e3, device=DEV)
+    vc = torch.arange(kv * 4 * dim, dtype=torch.float32, device=DEV).reshape(1, kv, 4, dim)
+    out = torch.empty(1, heads * dim, device=DEV)
+    ops.attention_rowwise(q, heads * dim, kc, vc, torch.zeros(1, 1, dtype=torch.int32, device=DEV),
+                          torch.zeros(1, dtype=torch.int32, device=DEV), torch.tensor([n - 1], dtype=torch.int32, device=DEV),
+                          out, heads, kv, dim, 4, None, 1 / math.sqrt(dim))
+    assert torch.isfinite(out).all()
+    np.testing.assert_allclose(f64(out).reshape(heads, dim)[0], f64(vc)[0, 0, :n].mean(0), rtol=1e-6)
+    np.testing.assert_allclose(f64(out).reshape(heads, dim)[3], f64(vc)[0, 1, :n].mean(0), rtol=1e-6)
+
+
+GEMM_SHAPES = [(1, 1, 1), (5, 7, 9), (64, 64, 32), (130, 200, 172), (33, 513, 144), (17, 130, 1000), (300, 129, 72), (8, 1536, 576)]
+
+
+@pytest.mark.parametrize("M, N, K", GEMM_SHAPES)
+def test_gemm_f32(ops, M, N, K):
+    a, w, r = rnd(M, K, seed=1), rnd(N, K, seed=2), rnd(M, N, seed=3)
+    want = f64(a) @ f64(w).T
+    # unit-variance operands summed in ascending k: partial sums grow like sqrt(k), each
+    # addition rounds at 6e-8 of it, so the error of a length-K sum is a few 1e-7 * K
+    atol = 3e-7 * K + 2e-6
+    np.testing.assert_allclose(f64(ops.gemm(a, w, torch.empty(M, N, device=DEV))), want, rtol=2e-5, atol=atol)
+    out = r.clone()
+    ops.gemm(a, w, out, residual=out)   # in place on the residual
+    np.testing.assert_allclose(f64(out), want + f64(r), rtol=2e-5, atol=atol)
+
+
+@pytest.mark.parametrize("M, N, K", GEMM_SHAPES)
+def test_gemm_bf16(ops, M, N, K):
+    a, w, r = rnd(M, K, dtype=torch.bfloat16, seed=1), rnd(N, K, dtype=torch.bfloat16, seed=2), rnd(M, N, seed=3)
+    want = f64(a) @ f64(w).T   # products of bf16 values are exact in float: only the sum order differs
+    np.testing.assert_allclose(f64(ops.gemm(a, w, torch.empty(M, N, device=DEV))), want, rtol=1e-4, atol=1e-4 * math.sqrt(K))
+    got = ops.gemm(a, w, torch.empty(M, N, dtype=torch.bfloat16, device=DEV))
+    np.testing.assert_allclose(f64(got), want, rtol=1e-2, atol=1e-2 * math.sqrt(K))
+    out = r.clone()
+    ops.gemm(a, w, out, residual=out)
+    np.testing.assert_allclose(f64(out), want + f64(r), rtol=1e-4, atol=1e-4 * math.sqrt(K))
+
+
+def test_gemm_strided_rows_and_bad_operands(ops):
+    from runtime.kernels.ops import KernelError
+    big = rnd(9, 50, dtype=torch.bfloat16)
+    a = big[:, 10:31]   # 21 columns of a wider buffer: rows are strided and unaligned
+    w = rnd(13, 21, dtype=torch.bfloat16, seed=2)
+    np.testing.assert_allclose(f64(ops.gemm(a, w, torch.empty(9, 13, device=DEV))), f64(a) @ f64(w).T, rtol=1e-4, atol=1e-3)
+    with pytest.raises(KernelError):
+        ops.gemm(rnd(4, 8), rnd(5, 9), torch.empty(4, 5, device=DEV))
+    with pytest.raises(KernelError):
+        ops.gemm(rnd(4, 8), rnd(5, 8, dtype=torch.bfloat16), torch.empty(4, 5, device=DEV))
+    with pytest.raises(KernelError):
+        ops.gemm(rnd(4, 8), rnd(5, 8), torch.empty(4, 5, dtype=torch.bfloat16, device=DEV))
+    with pytest.raises(KernelError):
+        ops.gemm(torch.zeros(4, 8), torch.zeros(5, 8), torch.empty(4, 5))  # CPU tensors: no fallback
+
+
+def test_argmax_lowest_index_wins(ops):
+    logits = rnd(6, 1003, seed=8)
+    logits[1, 500] = logits[1, 17] = 50.0
+    logits[2, :] = 1.0
+    logits[3, 1002] = 99.0
+    out = ops.argmax(logits, torch.empty(6, dtype=torch.int32, device=DEV)).cpu().numpy()
+    want = f64(logits).argmax(-1)
+    np.testing.assert_array_equal(out, want)
+    assert out[1] == 17 and out[2] == 0 and out[3] == 1002
+
+
+def test_sampling_kernel(ops):
+    from runtime.sampling import uniform01
+    V = 11
+    logits = torch.tensor(np.log(np.arange(1, V + 1, dtype=np.float64)), dtype=torch.float32, device=DEV)[None].repeat(4000, 1).contiguous()
+    temp = torch.full((4000,), 1.0, device=DEV)
+    seeds = torch.full((4000,), 1234, dtype=torch.int64, device=DEV)
+    counters = torch.arange(4000, dtype=torch.int64, device=DEV)
+    out = ops.sample(logits, temp, seeds, counters, torch.empty(4000, dtype=torch.int32, device=DEV)).cpu().numpy()
+    freq = np.bincount(out, minlength=V) / 4000
+    p = np.arange(1, V + 1) / np.arange(1, V + 1).sum()
+    assert np.abs(freq - p).max() < 0.03
+    # the draw is the inverse CDF at the documented random number
+    cdf = np.cumsum(p)
+    want = [int(np.searchsorted(cdf, uniform01(1234, c), side="right")) for c in range(50)]
+    assert (out[:50] == np.minimum(want, V - 1)).mean() > 0.95   # equal but for rounding at a CDF edge
+    # temperature 0 is greedy; a tiny temperature too; rows do not influence each other
+    z = rnd(5, 777, seed=3)
+    greedy = ops.argmax(z, torch.empty(5, dtype=torch.int32, device=DEV)).cpu().numpy()
+    for t in (0.0, 1e-4):
+        got = ops.sample(z, torch.full((5,), t, device=DEV), torch.zeros(5, dtype=torch.int64, device=DEV),
+                         torch.zeros(5, dtype=torch.int64, device=DEV), torch.empty(5, dtype=torch.int32, device=DEV))
+        np.testing.assert_array_equal(got.cpu().numpy(), greedy)
+    one = ops.sample(z[2:3].contiguous(), torch.full((1,), 0.8, device=DEV), torch.full((1,), 5, dtype=torch.int64, device=DEV),
+                     torch.full((1,), 9, dtype=torch.int64, device=DEV), torch.empty(1, dtype=torch.int32, device=DEV))
+    five = ops.sample(z, torch.full((5,), 0.8, device=DEV), torch.full((5,), 5, dtype=torch.int64, device=DEV),
+                      torch.full((5,), 9, dtype=torch.int64, device=DEV), torch.empty(5, dtype=torch.int32, device=DEV))
+    assert one[0] == five[2]
+
+
+def test_page_copy(ops):
+    pool = rnd(3, 2, 5, 2, 4, 8, dtype=torch.bfloat16)   # [sites, k/v, pages, kv_heads, page, dim]
+    before = pool.clone()
+    ops.page_copy(pool, torch.tensor([1, 4], dtype=torch.int32, device=DEV), torch.tensor([3, 0], dtype=torch.int32, device=DEV), 6, 5)
+    assert torch.equal(pool[:, :, 3], before[:, :, 1]) and torch.equal(pool[:, :, 0], before[:, :, 4])
+    assert torch.equal(pool[:, :, [1, 2, 4]], before[:, :, [1, 2, 4]])
+
+
+def test_kernels_refuse_what_they_cannot_take(ops):
+    from runtime.kernels.ops import KernelError
+    with pytest.raises(KernelError, match="head size"):
+        run_rowwise(ops, rnd(1, 2, 258), rnd(1, 2, 4, 258), rnd(1, 2, 4, 258), torch.zeros(1, 1, dtype=torch.int32, device=DEV), [(0, 0)], 4)
+    with pytest.raises(KernelError, match="divide"):
+        run_rowwise(ops, rnd(1, 3, 16), rnd(1, 2, 4, 16), rnd(1, 2, 4, 16), torch.zeros(1, 1, dtype=torch.int32, device=DEV), [(0, 0)], 4)
+    with pytest.raises(KernelError):
+        ops.rmsnorm(rnd(2, 8), rnd(9), torch.empty(2, 8, device=DEV), 1e-5)
+    with pytest.raises(KernelError):
+        ops.embedding(torch.zeros(2, dtype=torch.int64, device=DEV), rnd(4, 8), torch.empty(2, 8, device=DEV))

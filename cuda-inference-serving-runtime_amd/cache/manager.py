@@ -146,10 +146,12 @@ class CacheManager:
 
     # -- views for mixers ---------------------------------------------------
     def kv_of_site(self, site):
-        """(group id, keys [pages, kv_heads, P, D], values) of a site."""
+        """(group id, keys [pages, kv_heads, P, D], values [pages, kv_heads, D, P]) of a site.
+        Values are stored transposed inside a page (same bytes per page as keys)."""
         gid, index = self.group_of_site[site]
         storage = self.groups[gid].storage
-        return gid, storage[index, 0], storage[index, 1]
+        pages, kv_heads, psize, dim = storage.shape[2:]
+        return gid, storage[index, 0], storage[index, 1].view(pages, kv_heads, dim, psize)
 
     # -- bookkeeping --------------------------------------------------------
     def check(self):

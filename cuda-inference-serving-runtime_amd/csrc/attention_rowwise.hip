@@ -24,7 +24,7 @@ attn_rowwise_kernel(const T* __restrict__ q, int q_row_stride, const T* __restri
                     float scale, int splits) {
     __shared__ float qs[MAX_HEAD_DIM];
     __shared__ float ps[WAVE];
-    __shared__ long long rowoff[WAVE];
+    __shared__ long long rowoff[WAVE];   // offset of a key's first value element (values are [D, page_size] in a page)
 
     const int row = blockIdx.x, head = blockIdx.y, split = blockIdx.z, lane = threadIdx.x;
     const int kvh = head / (heads / kv_heads);
@@ -54,8 +54,9 @@ attn_rowwise_kernel(const T* __restrict__ q, int q_row_stride, const T* __restri
             long long off = 0;
             if (valid) {
                 const int page = table[t / page_size];
-                off = (((long long)page * kv_heads + kvh) * page_size + (t % page_size)) * dim;
-                const T* kr = kcache + off;
+                const long long head_base = ((long long)page * kv_heads + kvh) * page_size * dim;
+                off = head_base + (t % page_size);
+                const T* kr = kcache + head_base + (long long)(t % page_size) * dim;
                 float dot = 0.f;
                 for (int d = 0; d < dim; ++d) dot += qs[d] * load_f32(kr + d);
                 s = dot * scale;
@@ -76,7 +77,7 @@ attn_rowwise_kernel(const T* __restrict__ q, int q_row_stride, const T* __restri
                     const int d = lane + c * WAVE;
                     float a = acc[c] * alpha;
                     if (d < dim)
-                        for (int j = 0; j < nvalid; ++j) a += ps[j] * load_f32(vcache + rowoff[j] + d);
+                        for (int j = 0; j < nvalid; ++j) a += ps[j] * load_f32(vcache + rowoff[j] + (long long)d * page_size);
                     acc[c] = a;
                 }
             }
@@ -121,6 +122,17 @@ __global__ void attn_merge_kernel(const float* __restrict__ part_o, const float*
         }
         store_f32(out + ((size_t)row * heads + head) * dim + d, den > 0.f ? num / den : 0.f);
     }
+}
+
+extern "C" int cisr_attn_merge(const float* part_o, const float* part_ml, void* out, int rows, int heads, int dim,
+                               int splits, int dtype, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    if (heads > 65535 || splits < 1) return (int)hipErrorInvalidValue;
+    if (dtype == DT_F32)
+        attn_merge_kernel<float><<<dim3(rows, heads), 64, 0, stream>>>(part_o, part_ml, (float*)out, heads, dim, splits);
+    else
+        attn_merge_kernel<bf16_t><<<dim3(rows, heads), 64, 0, stream>>>(part_o, part_ml, (bf16_t*)out, heads, dim, splits);
+    return CISR_LAUNCH_CHECK();
 }
 
 extern "C" int cisr_attn_rowwise(const void* q, int q_row_stride, const void* kcache, const void* vcache,

@@ -132,8 +132,10 @@ extern "C" int cisr_swiglu(const void* gu, void* act, int rows, int inter, int d
 // (i, i + rot/2) turns by the angle whose cosine and sine sit in
 // cos_tab/sin_tab[pos, i] (tables are float, [max_pos, rot/2]).
 // (reference: kernels/ops.cu:21-33, kernels/execution.cu:28-40)
-// Cache layout per site: [pages, kv_heads, page_size, D]; slot = page*page_size
-// + offset; a negative slot writes nothing (padding rows, read-only sites).
+// Cache layout per site: keys [pages, kv_heads, page_size, D], values transposed
+// inside a page, [pages, kv_heads, D, page_size] (so that the attention kernels
+// read runs of keys for one coordinate); slot = page*page_size + offset; a
+// negative slot writes nothing (padding rows, read-only sites).
 template <typename T>
 __global__ void rope_scatter_kernel(T* __restrict__ qkv, const int* __restrict__ positions,
                                     const int* __restrict__ slots, const float* __restrict__ cos_tab,
@@ -185,7 +187,7 @@ __global__ void rope_scatter_kernel(T* __restrict__ qkv, const int* __restrict__
     const T* vb = kb + kv_heads * dim;
     for (int i = threadIdx.x; i < kv_heads * dim; i += blockDim.x) {
         int h = i / dim, d = i % dim;
-        vcache[(((size_t)page * kv_heads + h) * page_size + off) * dim + d] = vb[i];
+        vcache[(((size_t)page * kv_heads + h) * dim + d) * page_size + off] = vb[i];
     }
 }
 

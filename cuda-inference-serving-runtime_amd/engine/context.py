@@ -34,10 +34,25 @@ class StepContext:
         self.segments = []        # host: [(request, start, count)]
         self.max_context = 0      # host: largest position + 1 among the rows
         self.decode_only = False  # host: every segment brings exactly one token
-        self.fixed_splits = None  # set when the step runs as a captured program
+        self.span_hint = 0        # host: context length that sizes attention launches (a bucket under capture)
+        self._tasks = {}
 
     def buffer(self, name, shape, dtype):
         return self.runner.workspace.get(name, shape, dtype)
+
+    def attention_tasks(self, rows_per_tile):
+        """int32 [n, 4] on the device: (segment, first row, rows, 0) for tiles of at most
+        `rows_per_tile` consecutive rows of one segment."""
+        tasks = self._tasks.get(rows_per_tile)
+        if tasks is None:
+            items, row = [], 0
+            for seg, (_, _, count) in enumerate(self.segments):
+                for first in range(0, count, rows_per_tile):
+                    items.append((seg, row + first, min(rows_per_tile, count - first), 0))
+                row += count
+            tasks = torch.tensor(items, dtype=torch.int32).to(self.device, non_blocking=False)
+            self._tasks[rows_per_tile] = tasks
+        return tasks
 
     def attend(self, q, q_row_stride, kcache, vcache, view, out, heads, kv_heads, head_dim, window, scale):
         """out[r] = attention of row r's queries over its request's cache."""

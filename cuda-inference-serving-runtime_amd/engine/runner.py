@@ -185,7 +185,7 @@ class ModelRunner:
         ctx.seg_start, ctx.seg_first_pos, ctx.state_slots, ctx.logit_rows = view(3), view(4), view(5), view(6)
         ctx.kv = [GroupView(view(7 + 2 * g), view(8 + 2 * g, (S, W)), self.page_size, W) for g in range(G)]
         ctx.segments = [(d.request, d.start, d.count) for d in done]
-        ctx.max_context = max_context
+        ctx.max_context = ctx.span_hint = max_context
         ctx.decode_only = all(d.count == 1 for d in done)
         return ctx
 
@@ -217,18 +217,16 @@ class ModelRunner:
     # -- captured programs (decode steps) -------------------------------------------
     def _program_key(self, entries, done):
         """Decode-only steps that want every row's logits run as a captured graph,
-        keyed by the padded batch size and the attention split count."""
+        keyed by the padded batch size and the context length rounded up to a power
+        of two (it decides how attention splits the keys)."""
         if not all(d.count == 1 and list(e.want) == [0] for e, d in zip(entries, done)):
             return None
         batch = 1 << (len(entries) - 1).bit_length()
         context = 1 << (max(d.start + 1 for d in done) - 1).bit_length()
-        return (batch, self._splits(batch * self._max_heads(), context))
-
-    def _max_heads(self):
-        return max((getattr(layer.mixer, "heads", 1) for layer in self.model.layers), default=1)
+        return (batch, max(context, 256))
 
     def _run_program(self, key, entries, done):
-        batch, splits = key
+        batch, context = key
         program = self.programs.get(key)
         if program is None:
             total = int(self._layout(batch, batch, batch)[-1])
@@ -241,7 +239,7 @@ class ModelRunner:
         else:
             self.programs[key] = self.programs.pop(key)  # most recently used last
         ctx = self._context(entries, done, pad=(batch, batch, batch), device_buffer=program["meta"])
-        ctx.fixed_splits = splits
+        ctx.span_hint = context   # launch shapes inside a captured program depend on the key only
         if program["graph"] is None and program["runs"] >= 1:
             # the first run was eager and allocated every buffer; capture launches nothing
             graph = torch.cuda.CUDAGraph()
@@ -258,9 +256,29 @@ class ModelRunner:
 
     # -- attention dispatch -------------------------------------------------------
     def attention(self, ctx, q, q_row_stride, kcache, vcache, view, out, heads, kv_heads, head_dim, window, scale):
+        """bfloat16 with a head size in steps of 8 and pages of a power of two >= 4 run
+        on the matrix cores (one block per row for decode steps, tiles of rows from a
+        task list otherwise); everything else runs the exact row-wise kernel."""
         rows = out.shape[0]
-        span = ctx.max_context if not window else min(ctx.max_context, window)
-        splits = ctx.fixed_splits if ctx.fixed_splits is not None else self._splits(rows * heads, span)
+        span = ctx.span_hint if not window else min(ctx.span_hint, window + 31)
+        if ops.mfma_attention_supported(out.dtype, head_dim, view.page_size):
+            group = heads // kv_heads
+            heads_per_chunk = min(group, 16)
+            if ctx.decode_only:
+                blocks = rows * kv_heads * -(-group // heads_per_chunk)
+                splits = self._splits_rows(blocks, span)
+                workspace = None
+                if splits > 1:
+                    workspace = (ctx.buffer("attn.part_o", (rows * heads * splits * head_dim,), torch.float32),
+                                 ctx.buffer("attn.part_ml", (rows * heads * splits * 2,), torch.float32))
+                ops.attention_mfma(q, q_row_stride, kcache, vcache, view.tables, ctx.seg_of_row, ctx.positions, out,
+                                   heads, kv_heads, head_dim, view.page_size, window, scale, None, splits, workspace)
+            else:
+                tasks = ctx.attention_tasks(16 // heads_per_chunk)
+                ops.attention_mfma(q, q_row_stride, kcache, vcache, view.tables, ctx.seg_of_row, ctx.positions, out,
+                                   heads, kv_heads, head_dim, view.page_size, window, scale, tasks)
+            return
+        splits = self._splits(rows * heads, span)
         workspace = None
         if splits > 1:
             workspace = (ctx.buffer("attn.part_o", (rows * heads * splits * head_dim,), torch.float32),
@@ -270,8 +288,15 @@ class ModelRunner:
 
     @staticmethod
     def _splits(waves, span):
-        """How many ways a row's keys are split among wavefronts: enough to fill the
-        GPU when the batch alone does not, never finer than 256 keys a split."""
+        """Row-wise kernel: how many ways a row's keys are split among wavefronts: enough to
+        fill the GPU when the batch alone does not, never finer than 256 keys a split."""
         if waves >= 2048 or span <= 256:
             return 1
         return int(min(32, -(-span // 256), max(1, 4096 // waves)))
+
+    @staticmethod
+    def _splits_rows(blocks, span):
+        """Matrix-core decode kernel: blocks along the keys so that about a thousand
+        blocks are in flight, each with at least four 32-key steps (one per wave)."""
+        steps = -(-span // 32)
+        return int(max(1, min(steps // 4, -(-1024 // blocks), 64)))

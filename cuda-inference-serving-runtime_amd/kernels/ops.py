@@ -13,6 +13,8 @@ import torch
 from . import library
 
 F32, BF16 = 0, 1
+MFMA_HEAD_PADS = (32, 64, 96, 128, 160, 192, 224, 256)
+SKINNY_ROWS = 64   # products with at most this many rows run the weight-streaming kernel
 _DT = {torch.float32: F32, torch.bfloat16: BF16}
 
 
@@ -46,9 +48,13 @@ def _declare(h):
         "cisr_attn_rowwise": [p, i, p, p, p, p, p, p, p, p, i, i, i, i, i, i, i, f, i, i, p],
         "cisr_gemm_f32": [p, i, p, i, p, i, p, i, i, i, i, p],
         "cisr_gemm_bf16": [p, i, p, i, p, i, p, i, i, i, i, i, p],
+        "cisr_gemm_skinny_bf16": [p, i, p, i, p, i, p, i, i, i, i, i, i, p],
+        "cisr_attn_merge": [p, p, p, i, i, i, i, i, p],
         "cisr_argmax": [p, p, i, i, p],
         "cisr_sample": [p, p, p, p, p, i, i, p],
     }
+    for d in MFMA_HEAD_PADS:
+        sig[f"cisr_attn_mfma_d{d}"] = [p, i, p, p, p, i, p, i, p, p, p, p, p, i, i, i, i, i, f, i, i, p]
     for name, args in sig.items():
         fn = getattr(h, name)
         fn.argtypes = args
@@ -143,7 +149,8 @@ def rope_scatter(qkv, positions, slots, cos, sin, kcache, vcache, heads, kv_head
     """Rotate q (in place) and k of the fused projection rows, write k and v into
     the cache at `slots`.  kcache/vcache None: q only (a layer reading another's cache).
     qkv [T, (heads + 2 kv_heads) * dim] (or [T, heads * dim] without a cache);
-    cos/sin float [max_pos, rot/2]; cache [pages, kv_heads, page_size, dim]."""
+    cos/sin float [max_pos, rot/2]; keys [pages, kv_heads, page_size, dim],
+    values transposed in a page: [pages, kv_heads, dim, page_size]."""
     rows = qkv.shape[0]
     has_kv = kcache is not None
     width = (heads + (2 * kv_heads if has_kv else 0)) * dim
@@ -156,7 +163,7 @@ def rope_scatter(qkv, positions, slots, cos, sin, kcache, vcache, heads, kv_head
     if has_kv:
         pages = kcache.shape[0]
         kp = _dev(kcache, "kcache", qkv.dtype, (pages, kv_heads, page_size, dim))
-        vp = _dev(vcache, "vcache", qkv.dtype, (pages, kv_heads, page_size, dim))
+        vp = _dev(vcache, "vcache", qkv.dtype, (pages, kv_heads, dim, page_size))
         sp = _dev(slots, "slots", torch.int32, (rows,))
     _check(lib().cisr_rope_scatter(_dev(qkv, "qkv", None, (rows, width)), _dev(positions, "positions", torch.int32, (rows,)),
                                    sp, _dev(cos, "cos", torch.float32), _dev(sin, "sin", torch.float32, (max_pos, half)),
@@ -208,7 +215,7 @@ def attention_rowwise(q, q_row_stride, kcache, vcache, tables, seg_of_row, posit
         if part_o.numel() < rows * heads * splits * dim or part_ml.numel() < rows * heads * splits * 2:
             raise KernelError("attention: split workspace too small")
     _check(lib().cisr_attn_rowwise(q.data_ptr(), q_row_stride, _dev(kcache, "kcache", None, (pages, kv_heads, page_size, dim)),
-                                   _dev(vcache, "vcache", None, (pages, kv_heads, page_size, dim)),
+                                   _dev(vcache, "vcache", None, (pages, kv_heads, dim, page_size)),
                                    _dev(tables, "tables", torch.int32), _dev(seg_of_row, "seg_of_row", torch.int32, (rows,)),
                                    _dev(positions, "positions", torch.int32, (rows,)), _dev(out, "out", None, (rows, heads * dim)),
                                    po, pm, rows, heads, kv_heads, dim, page_size, width, int(window or 0), float(scale),
@@ -240,6 +247,9 @@ def gemm(a, w, out, residual=None):
             raise KernelError("gemm: float operands need a float output")
         code = lib().cisr_gemm_f32(a.data_ptr(), a.stride(0), w.data_ptr(), w.stride(0), out.data_ptr(), out.stride(0),
                                    rp, ldr, m, n, k, _stream())
+    elif a.dtype == torch.bfloat16 and m <= SKINNY_ROWS and _skinny_ok(a, w):
+        code = lib().cisr_gemm_skinny_bf16(a.data_ptr(), a.stride(0), w.data_ptr(), w.stride(0), out.data_ptr(),
+                                           out.stride(0), rp, ldr, m, n, k, _storage(out, "out"), 0, _stream())
     elif a.dtype == torch.bfloat16:
         code = lib().cisr_gemm_bf16(a.data_ptr(), a.stride(0), w.data_ptr(), w.stride(0), out.data_ptr(), out.stride(0),
                                     rp, ldr, m, n, k, _storage(out, "out"), _stream())
@@ -247,6 +257,77 @@ def gemm(a, w, out, residual=None):
         raise KernelError(f"gemm: unsupported dtype {a.dtype}")
     _check(code, "gemm")
     return out
+
+
+def _skinny_ok(a, w):
+    k = a.shape[1]
+    return (k % 8 == 0 and a.stride(0) % 8 == 0 and w.stride(0) % 8 == 0 and a.data_ptr() % 16 == 0
+            and w.data_ptr() % 16 == 0)
+
+
+def gemm_swiglu(a, w_gate_up, out, scratch=None):
+    """out[M, I] = silu(a . Wg^T) * (a . Wu^T) with w_gate_up = [Wg; Wu] ([2I, K]).
+    Few rows of bf16 run one fused weight-streaming kernel; otherwise the product
+    goes to `scratch` [M, 2I] and the activation is a second kernel."""
+    m, k = a.shape
+    two_i, k2 = w_gate_up.shape
+    inter = two_i // 2
+    if k != k2 or two_i % 2 or tuple(out.shape) != (m, inter) or out.dtype != a.dtype or a.dtype != w_gate_up.dtype:
+        raise KernelError("gemm_swiglu: shapes or dtypes do not fit")
+    if a.dtype == torch.bfloat16 and m <= SKINNY_ROWS and _skinny_ok(a, w_gate_up) and a.is_cuda and out.is_contiguous():
+        _check(lib().cisr_gemm_skinny_bf16(a.data_ptr(), a.stride(0), w_gate_up.data_ptr(), w_gate_up.stride(0),
+                                           out.data_ptr(), out.stride(0), None, 0, m, inter, k, BF16, inter, _stream()),
+               "gemm_swiglu")
+        return out
+    if scratch is None:
+        raise KernelError("gemm_swiglu: this shape needs a scratch buffer [M, 2I]")
+    gemm(a, w_gate_up, scratch)
+    return swiglu(scratch, out)
+
+
+def attention_mfma(q, q_row_stride, kcache, vcache, tables, seg_of_row, positions, out, heads, kv_heads, dim,
+                   page_size, window, scale, tasks=None, splits=1, workspace=None):
+    """Matrix-core attention (bf16).  tasks int32 [n, 4] = (segment, first row, rows, 0) runs tiles of
+    prompt rows; tasks None runs one block per row (decode) with `splits` blocks along the keys."""
+    rows = out.shape[0]
+    if not mfma_attention_supported(out.dtype, dim, page_size):
+        raise KernelError(f"attention_mfma: head size {dim} / page size {page_size} / dtype {out.dtype} not supported")
+    if heads % kv_heads:
+        raise KernelError(f"attention: {heads} query heads do not divide into {kv_heads} key heads")
+    if q.dtype != out.dtype or kcache.dtype != out.dtype or q_row_stride % 8 or q.data_ptr() % 16:
+        raise KernelError("attention_mfma: q, cache and out must be bfloat16 with 16-byte aligned rows")
+    if q.numel() < (rows - 1) * q_row_stride + heads * dim:
+        raise KernelError("attention: q buffer too small for its stride")
+    pages = kcache.shape[0]
+    dpad = -(-dim // 32) * 32
+    fn = getattr(lib(), f"cisr_attn_mfma_d{dpad}")
+    po = pm = tp = None
+    if tasks is not None:
+        n_tasks, mode, splits = tasks.shape[0], 0, 1
+        tp = _dev(tasks, "tasks", torch.int32, (n_tasks, 4))
+    else:
+        n_tasks, mode = rows, 1
+        if splits > 1:
+            if workspace is None:
+                raise KernelError("attention: split runs need a workspace")
+            part_o, part_ml = workspace
+            po, pm = _dev(part_o, "part_o", torch.float32), _dev(part_ml, "part_ml", torch.float32)
+            if part_o.numel() < rows * heads * splits * dim or part_ml.numel() < rows * heads * splits * 2:
+                raise KernelError("attention: split workspace too small")
+    _check(fn(q.data_ptr(), q_row_stride, _dev(kcache, "kcache", None, (pages, kv_heads, page_size, dim)),
+              _dev(vcache, "vcache", None, (pages, kv_heads, dim, page_size)), _dev(tables, "tables", torch.int32),
+              tables.shape[1], tp, n_tasks, _dev(seg_of_row, "seg_of_row", torch.int32, (rows,)),
+              _dev(positions, "positions", torch.int32, (rows,)), _dev(out, "out", None, (rows, heads * dim)), po, pm,
+              heads, kv_heads, dim, page_size.bit_length() - 1, int(window or 0), float(scale), int(splits), mode, _stream()),
+           "attention_mfma")
+    if mode == 1 and splits > 1:
+        _check(lib().cisr_attn_merge(po, pm, out.data_ptr(), rows, heads, dim, int(splits), BF16, _stream()), "attention_merge")
+    return out
+
+
+def mfma_attention_supported(dtype, dim, page_size):
+    return (dtype == torch.bfloat16 and dim % 8 == 0 and dim <= 256 and page_size >= 4
+            and page_size & (page_size - 1) == 0)
 
 
 def argmax(logits, out):

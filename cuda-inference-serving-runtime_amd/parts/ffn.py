@@ -27,10 +27,11 @@ class GatedMLP(FeedForward):
 
     def forward(self, h, residual, ctx):
         T = h.shape[0]
-        gu = ctx.buffer("ffn.gate_up", (T, 2 * self.intermediate), ctx.dtype)
-        ops.gemm(h, self.w_gate_up, gu)
         act = ctx.buffer("ffn.act", (T, self.intermediate), ctx.dtype)
-        ops.swiglu(gu, act)
+        if ctx.dtype == torch.bfloat16 and T <= ops.SKINNY_ROWS:
+            ops.gemm_swiglu(h, self.w_gate_up, act)   # fused when the fast kernel takes the shape
+        else:
+            ops.gemm_swiglu(h, self.w_gate_up, act, scratch=ctx.buffer("ffn.gate_up", (T, 2 * self.intermediate), ctx.dtype))
         return ops.gemm(act, self.w_down, residual, residual=residual)
 
 

@@ -109,7 +109,7 @@ def test_rope_scatter(ops, dtype, heads, kv_heads, dim, theta):
     pos = [0, 17, 500, 599, 3]
     slots = [5, 0, 22, -1, 9]
     kc = torch.full((pages, kv_heads, P_, dim), 7.0, dtype=dtype, device=DEV)
-    vc = torch.full((pages, kv_heads, P_, dim), 7.0, dtype=dtype, device=DEV)
+    vc = torch.full((pages, kv_heads, dim, P_), 7.0, dtype=dtype, device=DEV)   # values: transposed inside a page
     ops.rope_scatter(qkv, torch.tensor(pos, dtype=torch.int32, device=DEV), torch.tensor(slots, dtype=torch.int32, device=DEV),
                      cos, sin, kc, vc, heads, kv_heads, dim, P_)
     q_ref = P.rope(ref[:, :heads * dim].reshape(T, heads, dim), pos, theta)
@@ -122,11 +122,11 @@ def test_rope_scatter(ops, dtype, heads, kv_heads, dim, theta):
         if s < 0:
             continue
         np.testing.assert_allclose(kc64[s // P_, :, s % P_], k_ref[t], **tol(dtype))
-        np.testing.assert_array_equal(vc64[s // P_, :, s % P_], v_ref[t])
+        np.testing.assert_array_equal(vc64[s // P_, :, :, s % P_], v_ref[t])
         written.add(s)
     for s in range(pages * P_):
         if s not in written:   # nothing else is touched, a negative slot writes nothing
-            assert (kc64[s // P_, :, s % P_] == 7).all() and (vc64[s // P_, :, s % P_] == 7).all()
+            assert (kc64[s // P_, :, s % P_] == 7).all() and (vc64[s // P_, :, :, s % P_] == 7).all()
 
 
 def test_rope_partial_rotation_and_identity(ops):
@@ -134,7 +134,7 @@ def test_rope_partial_rotation_and_identity(ops):
     dim, rot = 16, 8
     rope = RotaryEmbedding(dim, 1e4, 50, rotary_dim=rot); rope.prepare(DEV, torch.float32)
     qkv = rnd(3, 3 * dim, seed=9); ref = f64(qkv)
-    kc = torch.zeros(1, 1, 4, dim, device=DEV); vc = torch.zeros_like(kc)
+    kc = torch.zeros(1, 1, 4, dim, device=DEV); vc = torch.zeros(1, 1, dim, 4, device=DEV)
     pos = [3, 40, 7]
     ops.rope_scatter(qkv, torch.tensor(pos, dtype=torch.int32, device=DEV), torch.tensor([0, 1, 2], dtype=torch.int32, device=DEV),
                      *rope.tables(), kc, vc, 1, 1, dim, 4)
@@ -181,13 +181,13 @@ def paged_case(heads, kv_heads, dim, page_size, lengths, dtype, seed=0, pages=No
             q[r, h] = q[r, (h // group) * group]
             K[page, h // group, off] = q[r, h] * 4.0
     kt = torch.from_numpy(K).to(dtype).to(DEV)
-    vt = torch.from_numpy(V).to(dtype).to(DEV)
+    vt = torch.from_numpy(np.ascontiguousarray(V.transpose(0, 1, 3, 2))).to(dtype).to(DEV)   # [pages, kv, D, P]
     qt = torch.from_numpy(q).to(dtype).to(DEV)
     return qt, kt, vt, torch.from_numpy(tables).to(DEV), rows
 
 
 def reference_attention(qt, kt, vt, tables, rows, page_size, window=None, scale=None):
-    q, K, V, tab = f64(qt), f64(kt), f64(vt), tables.cpu().numpy()
+    q, K, V, tab = f64(qt), f64(kt), f64(vt).transpose(0, 1, 3, 2), tables.cpu().numpy()
     out = []
     for r, (seg, pos) in enumerate(rows):
         lo = 0 if not window else max(0, pos + 1 - window)
@@ -245,7 +245,7 @@ def test_attention_finds_one_far_key_among_hundreds(ops, dtype):
     qt, kt, vt, tables, rows = paged_case(4, 2, 64, 16, [700, 40], dtype, seed=5, sharpen=(0, 3))
     want = reference_attention(qt, kt, vt, tables, rows, 16)
     page, off = tables[0, 0].item(), 3
-    np.testing.assert_allclose(want[0, 0], f64(vt)[page, 0, off], atol=1e-6)   # the case is what it claims to be
+    np.testing.assert_allclose(want[0, 0], f64(vt)[page, 0, :, off], atol=1e-6)   # the case is what it claims to be
     for splits in (1, 8):
         np.testing.assert_allclose(run_rowwise(ops, qt, kt, vt, tables, rows, 16, splits), want, **tol(dtype))
 
@@ -255,14 +255,129 @@ def test_attention_equal_large_scores_give_the_mean(ops):
     heads, kv, dim, n = 4, 2, 8, 3
     q = torch.full((1, heads * dim), 1e3, device=DEV)
     kc = torch.full((1, kv, 4, dim), 1e3, device=DEV)
-    vc = torch.arange(kv * 4 * dim, dtype=torch.float32, device=DEV).reshape(1, kv, 4, dim)
+    vc = torch.arange(kv * 4 * dim, dtype=torch.float32, device=DEV).reshape(1, kv, dim, 4)
     out = torch.empty(1, heads * dim, device=DEV)
     ops.attention_rowwise(q, heads * dim, kc, vc, torch.zeros(1, 1, dtype=torch.int32, device=DEV),
                           torch.zeros(1, dtype=torch.int32, device=DEV), torch.tensor([n - 1], dtype=torch.int32, device=DEV),
                           out, heads, kv, dim, 4, None, 1 / math.sqrt(dim))
     assert torch.isfinite(out).all()
-    np.testing.assert_allclose(f64(out).reshape(heads, dim)[0], f64(vc)[0, 0, :n].mean(0), rtol=1e-6)
-    np.testing.assert_allclose(f64(out).reshape(heads, dim)[3], f64(vc)[0, 1, :n].mean(0), rtol=1e-6)
+    np.testing.assert_allclose(f64(out).reshape(heads, dim)[0], f64(vc)[0, 0, :, :n].mean(-1), rtol=1e-6)
+    np.testing.assert_allclose(f64(out).reshape(heads, dim)[3], f64(vc)[0, 1, :, :n].mean(-1), rtol=1e-6)
+
+
+def run_mfma(ops, qt, kt, vt, tables, rows, page_size, mode, splits=1, window=None, scale=None, rows_per_tile=None):
+    """mode "tiles": rows are grouped into tiles of consecutive rows of one segment;
+    mode "rows": one block per row with `splits` blocks along the keys."""
+    T, heads, dim = qt.shape
+    kv_heads = kt.shape[1]
+    seg = torch.tensor([r[0] for r in rows], dtype=torch.int32, device=DEV)
+    pos = torch.tensor([r[1] for r in rows], dtype=torch.int32, device=DEV)
+    out = torch.full((T, heads * dim), 9.0, dtype=qt.dtype, device=DEV)
+    tasks = None
+    ws = (torch.empty(T * heads * splits * dim, device=DEV), torch.empty(T * heads * splits * 2, device=DEV))
+    if mode == "tiles":
+        group = heads // kv_heads
+        rpt = rows_per_tile or 16 // min(group, 16)
+        items, i = [], 0
+        while i < T:   # consecutive rows of one segment with consecutive positions form a tile
+            n = 1
+            while i + n < T and n < rpt and rows[i + n][0] == rows[i][0] and rows[i + n][1] == rows[i + n - 1][1] + 1:
+                n += 1
+            items.append((rows[i][0], i, n, 0)); i += n
+        tasks = torch.tensor(items, dtype=torch.int32, device=DEV)
+    ops.attention_mfma(qt.reshape(T, heads * dim), heads * dim, kt, vt, tables, seg, pos, out, heads, kv_heads, dim,
+                       page_size, window, scale if scale is not None else 1 / math.sqrt(dim), tasks, splits, ws)
+    return f64(out).reshape(T, heads, dim)
+
+
+MFMA_TOL = dict(rtol=2e-2, atol=2e-2)
+
+
+@pytest.mark.parametrize("heads, kv_heads, dim, page_size", [
+    (4, 2, 16, 4), (6, 6, 24, 8), (9, 3, 64, 16), (8, 1, 128, 64), (2, 2, 256, 4), (5, 5, 40, 16), (32, 1, 64, 16), (20, 1, 32, 8)])
+def test_attention_mfma_rows(ops, heads, kv_heads, dim, page_size):
+    """Decode form: single rows at scattered positions, every split count, including more splits than 32-key steps."""
+    qt, kt, vt, tables, rows = paged_case(heads, kv_heads, dim, page_size, [17, 7, 1, 130, 333], torch.bfloat16, seed=dim + heads)
+    want = reference_attention(qt, kt, vt, tables, rows, page_size)
+    for splits in (1, 2, 3, 16):
+        got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, "rows", splits)
+        np.testing.assert_allclose(got, want, **MFMA_TOL, err_msg=f"splits={splits}")
+    rows2 = list(rows); rows2[0] = (-1, 0)            # a padding row gives zeros
+    got = run_mfma(ops, qt, kt, vt, tables, rows2, page_size, "rows", 2)
+    assert (got[0] == 0).all()
+    np.testing.assert_allclose(got[1:], want[1:], **MFMA_TOL)
+
+
+def portion_case(heads, kv_heads, dim, page_size, plan, seed):
+    """plan: [(cached keys before the portion, portion length)] per request: every row of every portion is a query."""
+    rng = np.random.default_rng(seed)
+    lengths = [a + b for a, b in plan]
+    qt, kt, vt, tables, _ = paged_case(heads, kv_heads, dim, page_size, lengths, torch.bfloat16, seed=seed)
+    rows = [(s, p) for s, (a, b) in enumerate(plan) for p in range(a, a + b)]
+    q = rng.standard_normal((len(rows), heads, dim)).astype(np.float32)
+    return torch.from_numpy(q).to(torch.bfloat16).to(DEV), kt, vt, tables, rows
+
+
+@pytest.mark.parametrize("heads, kv_heads, dim, page_size", [
+    (4, 2, 16, 4), (6, 6, 24, 8), (9, 3, 64, 16), (8, 2, 128, 16), (3, 3, 256, 64), (32, 1, 64, 16), (7, 7, 48, 16)])
+def test_attention_mfma_tiles(ops, heads, kv_heads, dim, page_size):
+    """Prompt portions: rows of a portion attend to the cached prefix and causally to
+    the portion itself; portions of 1, 2 and many rows, starting at and off page edges."""
+    plan = [(0, 70), (33, 2), (64, 1), (5, 37), (100, 45)]
+    qt, kt, vt, tables, rows = portion_case(heads, kv_heads, dim, page_size, plan, seed=dim * 3 + heads)
+    want = reference_attention(qt, kt, vt, tables, rows, page_size)
+    got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, "tiles")
+    np.testing.assert_allclose(got, want, **MFMA_TOL)
+    got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, "tiles", rows_per_tile=1)   # tiles need not be full
+    np.testing.assert_allclose(got, want, **MFMA_TOL)
+
+
+def test_attention_mfma_window_and_far_key(ops):
+    qt, kt, vt, tables, rows = portion_case(4, 2, 32, 8, [(40, 30), (0, 9)], seed=21)
+    for window in (1, 8, 9, 33, 64):
+        want = reference_attention(qt, kt, vt, tables, rows, 8, window=window)
+        np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables, rows, 8, "tiles", window=window), want, **MFMA_TOL)
+        np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables, rows, 8, "rows", 2, window=window), want, **MFMA_TOL)
+    want = reference_attention(qt, kt, vt, tables, rows, 8, scale=0.3)
+    np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables, rows, 8, "tiles", scale=0.3), want, **MFMA_TOL)
+    # pages the window has passed are marked -1 in the table and must never be needed
+    tables2 = tables.clone(); tables2[0, :4] = -1          # keys 0..31 of request 0; window 8 from position 40 starts at 33
+    want = reference_attention(qt, kt, vt, tables, rows, 8, window=8)
+    np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables2, rows, 8, "tiles", window=8), want, **MFMA_TOL)
+    np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables2, rows, 8, "rows", 3, window=8), want, **MFMA_TOL)
+    # one far key among hundreds stands out
+    qt, kt, vt, tables, rows = paged_case(4, 2, 64, 16, [700, 40], torch.bfloat16, seed=5, sharpen=(0, 3))
+    want = reference_attention(qt, kt, vt, tables, rows, 16)
+    for mode, splits in (("rows", 1), ("rows", 8), ("tiles", 1)):
+        np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables, rows, 16, mode, splits), want, **MFMA_TOL)
+
+
+def test_gemm_skinny_and_fused_swiglu(ops):
+    """Few rows of bf16 run the weight-streaming kernel: every row count up to 64, output widths off
+    the 16-column tile, float/bf16 outputs, residual, and the fused SwiGLU against the two-kernel path."""
+    for M, N, K in [(1, 16, 32), (3, 100, 72), (8, 1728, 576), (16, 576, 1536), (17, 49, 264), (33, 130, 200), (64, 96, 4096), (50, 1003, 200)]:
+        a, w, r = rnd(M, K, dtype=torch.bfloat16, seed=1), rnd(N, K, dtype=torch.bfloat16, seed=2), rnd(M, N, seed=3)
+        want = f64(a) @ f64(w).T
+        np.testing.assert_allclose(f64(ops.gemm(a, w, torch.empty(M, N, device=DEV))), want, rtol=1e-4, atol=1e-4 * math.sqrt(K))
+        np.testing.assert_allclose(f64(ops.gemm(a, w, torch.empty(M, N, dtype=torch.bfloat16, device=DEV))), want, rtol=1e-2, atol=1e-2 * math.sqrt(K))
+        out = r.clone(); ops.gemm(a, w, out, residual=out)
+        np.testing.assert_allclose(f64(out), want + f64(r), rtol=1e-4, atol=1e-4 * math.sqrt(K))
+    for M, I, K in [(1, 16, 32), (8, 1536, 576), (40, 172, 64), (64, 264, 200)]:
+        a = rnd(M, K, dtype=torch.bfloat16, seed=4, scale=0.5)
+        w = rnd(2 * I, K, dtype=torch.bfloat16, seed=5, scale=0.2)
+        gu = f64(a) @ f64(w).T
+        gq = torch.from_numpy(gu).to(torch.bfloat16).double().numpy()   # the two-kernel path rounds the product first
+        want = P.swiglu(gq[:, :I], gq[:, I:])
+        got = ops.gemm_swiglu(a, w, torch.empty(M, I, dtype=torch.bfloat16, device=DEV))
+        np.testing.assert_allclose(f64(got), want, rtol=2e-2, atol=2e-2)
+        two = ops.gemm_swiglu(rnd(70, K, dtype=torch.bfloat16, seed=4, scale=0.5), w, torch.empty(70, I, dtype=torch.bfloat16, device=DEV),
+                              scratch=torch.empty(70, 2 * I, dtype=torch.bfloat16, device=DEV))   # more rows: product + activation
+        assert two.shape == (70, I)
+    # a row's result does not depend on how many rows are beside it
+    a, w = rnd(64, 576, dtype=torch.bfloat16, seed=6), rnd(300, 576, dtype=torch.bfloat16, seed=7)
+    full = ops.gemm(a, w, torch.empty(64, 300, device=DEV))
+    for m in (1, 5, 16, 17, 48):
+        assert torch.equal(ops.gemm(a[:m].contiguous(), w, torch.empty(m, 300, device=DEV)), full[:m])
 
 
 GEMM_SHAPES = [(1, 1, 1), (5, 7, 9), (64, 64, 32), (130, 200, 172), (33, 513, 144), (17, 130, 1000), (300, 129, 72), (8, 1536, 576)]
@@ -360,9 +475,14 @@ def test_page_copy(ops):
 def test_kernels_refuse_what_they_cannot_take(ops):
     from runtime.kernels.ops import KernelError
     with pytest.raises(KernelError, match="head size"):
-        run_rowwise(ops, rnd(1, 2, 258), rnd(1, 2, 4, 258), rnd(1, 2, 4, 258), torch.zeros(1, 1, dtype=torch.int32, device=DEV), [(0, 0)], 4)
+        run_rowwise(ops, rnd(1, 2, 258), rnd(1, 2, 4, 258), rnd(1, 2, 258, 4), torch.zeros(1, 1, dtype=torch.int32, device=DEV), [(0, 0)], 4)
     with pytest.raises(KernelError, match="divide"):
-        run_rowwise(ops, rnd(1, 3, 16), rnd(1, 2, 4, 16), rnd(1, 2, 4, 16), torch.zeros(1, 1, dtype=torch.int32, device=DEV), [(0, 0)], 4)
+        run_rowwise(ops, rnd(1, 3, 16), rnd(1, 2, 4, 16), rnd(1, 2, 16, 4), torch.zeros(1, 1, dtype=torch.int32, device=DEV), [(0, 0)], 4)
+    with pytest.raises(KernelError, match="not supported"):   # the matrix-core kernel takes bf16, head sizes in steps of 8, pages 4, 8, 16, ...
+        ops.attention_mfma(rnd(1, 2 * 12, dtype=torch.bfloat16), 24, rnd(1, 2, 4, 12, dtype=torch.bfloat16), rnd(1, 2, 12, 4, dtype=torch.bfloat16),
+                           torch.zeros(1, 1, dtype=torch.int32, device=DEV), torch.zeros(1, dtype=torch.int32, device=DEV),
+                           torch.zeros(1, dtype=torch.int32, device=DEV), torch.empty(1, 24, dtype=torch.bfloat16, device=DEV), 2, 2, 12, 4, None, 1.0)
+    assert not ops.mfma_attention_supported(torch.bfloat16, 64, 3) and not ops.mfma_attention_supported(torch.float32, 64, 16)
     with pytest.raises(KernelError):
         ops.rmsnorm(rnd(2, 8), rnd(9), torch.empty(2, 8, device=DEV), 1e-5)
     with pytest.raises(KernelError):

@@ -104,8 +104,8 @@ attn_rowwise_kernel(const T* __restrict__ q, int q_row_stride, const T* __restri
 
 // Merge split partials: m = max m_i; w_i = l_i > 0 ? exp(m_i - m) * l_i : 0;
 // out = sum w_i o_i / sum w_i (reference: kernels/ops.cu:72-86).  A row with no
-// keys at all (padding) gives zeros.
-template <typename T>
+// keys at all (padding) gives zeros.  LOG2: the maxima are in units of log2.
+template <typename T, bool LOG2>
 __global__ void attn_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                   T* __restrict__ out, int heads, int dim, int splits) {
     const int row = blockIdx.x, head = blockIdx.y;
@@ -116,7 +116,8 @@ __global__ void attn_merge_kernel(const float* __restrict__ part_o, const float*
         float den = 0.f, num = 0.f;
         for (int s = 0; s < splits; ++s) {
             const float l = part_ml[(base + s) * 2 + 1];
-            const float w = l > 0.f ? expf(part_ml[(base + s) * 2] - m) * l : 0.f;
+            const float dm = part_ml[(base + s) * 2] - m;
+            const float w = l > 0.f ? (LOG2 ? exp2f(dm) : expf(dm)) * l : 0.f;
             den += w;
             num += w * part_o[(base + s) * dim + d];
         }
@@ -124,14 +125,12 @@ __global__ void attn_merge_kernel(const float* __restrict__ part_o, const float*
     }
 }
 
+// merge of the matrix-core kernel's partials (bf16 output, maxima in log2 units)
 extern "C" int cisr_attn_merge(const float* part_o, const float* part_ml, void* out, int rows, int heads, int dim,
-                               int splits, int dtype, hipStream_t stream) {
+                               int splits, hipStream_t stream) {
     if (rows <= 0) return 0;
     if (heads > 65535 || splits < 1) return (int)hipErrorInvalidValue;
-    if (dtype == DT_F32)
-        attn_merge_kernel<float><<<dim3(rows, heads), 64, 0, stream>>>(part_o, part_ml, (float*)out, heads, dim, splits);
-    else
-        attn_merge_kernel<bf16_t><<<dim3(rows, heads), 64, 0, stream>>>(part_o, part_ml, (bf16_t*)out, heads, dim, splits);
+    attn_merge_kernel<bf16_t, true><<<dim3(rows, heads), 64, 0, stream>>>(part_o, part_ml, (bf16_t*)out, heads, dim, splits);
     return CISR_LAUNCH_CHECK();
 }
 
@@ -155,8 +154,8 @@ extern "C" int cisr_attn_rowwise(const void* q, int q_row_stride, const void* kc
     int err = CISR_LAUNCH_CHECK();
     if (err || splits == 1) return err;
     if (dtype == DT_F32)
-        attn_merge_kernel<float><<<dim3(rows, heads), 64, 0, stream>>>(part_o, part_ml, (float*)out, heads, dim, splits);
+        attn_merge_kernel<float, false><<<dim3(rows, heads), 64, 0, stream>>>(part_o, part_ml, (float*)out, heads, dim, splits);
     else
-        attn_merge_kernel<bf16_t><<<dim3(rows, heads), 64, 0, stream>>>(part_o, part_ml, (bf16_t*)out, heads, dim, splits);
+        attn_merge_kernel<bf16_t, false><<<dim3(rows, heads), 64, 0, stream>>>(part_o, part_ml, (bf16_t*)out, heads, dim, splits);
     return CISR_LAUNCH_CHECK();
 }

@@ -74,6 +74,15 @@ class Workspace:
             self.buffers[key] = buf
         return buf
 
+    def get_zeroed(self, name, shape, dtype):
+        """A buffer that is zero when first handed out; its users leave it zero."""
+        key = (name, tuple(shape), dtype)
+        buf = self.buffers.get(key)
+        if buf is None:
+            buf = torch.zeros(tuple(shape), dtype=dtype, device=self.device)
+            self.buffers[key] = buf
+        return buf
+
     def bytes(self):
         return sum(b.numel() * b.element_size() for b in self.buffers.values())
 

@@ -11,6 +11,7 @@ every row (runtime/model.py:86-120); its order of checks is kept: batch shape,
 context limit, token range, page preflight, then execution
 (runtime/model.py:93-102).
 """
+import gc
 from dataclasses import dataclass, field
 from typing import List, Sequence
 
@@ -242,9 +243,17 @@ class ModelRunner:
         ctx.span_hint = context   # launch shapes inside a captured program depend on the key only
         if program["graph"] is None and program["runs"] >= 1:
             # the first run was eager and allocated every buffer; capture launches nothing
+            # nothing but kernel launches may happen while the stream records: keep the garbage
+            # collector from freeing device objects (other graphs, events) in the middle of it
             graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
-                program["logits"] = self.model.forward(ctx)
+            collecting = gc.isenabled()
+            gc.disable()
+            try:
+                with torch.cuda.graph(graph, capture_error_mode="thread_local"):
+                    program["logits"] = self.model.forward(ctx)
+            finally:
+                if collecting:
+                    gc.enable()
             program["graph"] = graph
         if program["graph"] is not None:
             program["graph"].replay()
@@ -266,13 +275,13 @@ class ModelRunner:
             heads_per_chunk = min(group, 16)
             if ctx.decode_only:
                 blocks = rows * kv_heads * -(-group // heads_per_chunk)
-                splits = self._splits_rows(blocks, span)
+                waves, splits = self._rows_launch(blocks, span, heads_per_chunk, head_dim)
                 workspace = None
                 if splits > 1:
                     workspace = (ctx.buffer("attn.part_o", (rows * heads * splits * head_dim,), torch.float32),
                                  ctx.buffer("attn.part_ml", (rows * heads * splits * 2,), torch.float32))
                 ops.attention_mfma(q, q_row_stride, kcache, vcache, view.tables, ctx.seg_of_row, ctx.positions, out,
-                                   heads, kv_heads, head_dim, view.page_size, window, scale, None, splits, workspace)
+                                   heads, kv_heads, head_dim, view.page_size, window, scale, None, splits, workspace, waves)
             else:
                 tasks = ctx.attention_tasks(16 // heads_per_chunk)
                 ops.attention_mfma(q, q_row_stride, kcache, vcache, view.tables, ctx.seg_of_row, ctx.positions, out,
@@ -295,8 +304,18 @@ class ModelRunner:
         return int(min(32, -(-span // 256), max(1, 4096 // waves)))
 
     @staticmethod
-    def _splits_rows(blocks, span):
-        """Matrix-core decode kernel: blocks along the keys so that about a thousand
-        blocks are in flight, each with at least four 32-key steps (one per wave)."""
+    def _rows_launch(blocks, span, heads_per_chunk, head_dim):
+        """Matrix-core decode kernel: (wavefronts a block, blocks along the keys).  Few rows:
+        sixteen waves share a row's keys inside one block, so no second kernel has to merge
+        partials; only when even that leaves the GPU idle and the context is long are the keys
+        also split over blocks.  Many rows: four waves a block, one block a row and head group."""
         steps = -(-span // 32)
-        return int(max(1, min(steps // 4, -(-1024 // blocks), 64)))
+        dpad = -(-head_dim // 32) * 32
+        wide_fits = 16 * heads_per_chunk * (dpad + 2) * 4 <= 128 * 1024
+        if blocks >= 512 or not wide_fits:
+            waves = 4
+        else:
+            waves = 16
+        per_block = 4 * waves            # at least four 32-key steps a wave
+        splits = int(max(1, min(steps // per_block, -(-512 // blocks), 64)))
+        return waves, splits

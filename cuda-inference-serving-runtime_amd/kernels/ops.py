@@ -48,13 +48,14 @@ def _declare(h):
         "cisr_attn_rowwise": [p, i, p, p, p, p, p, p, p, p, i, i, i, i, i, i, i, f, i, i, p],
         "cisr_gemm_f32": [p, i, p, i, p, i, p, i, i, i, i, p],
         "cisr_gemm_bf16": [p, i, p, i, p, i, p, i, i, i, i, i, p],
-        "cisr_gemm_skinny_bf16": [p, i, p, i, p, i, p, i, i, i, i, i, i, p],
-        "cisr_attn_merge": [p, p, p, i, i, i, i, i, p],
+        "cisr_gemm_skinny_bf16": [p, i, p, i, p, i, p, i, i, i, i, i, i, p, f, p, p],
+        "cisr_qkv_rope_skinny": [p, i, p, i, p, i, i, i, p, f, p, p, p, p, p, p, i, i, i, i, i, p],
+        "cisr_attn_merge": [p, p, p, i, i, i, i, p],
         "cisr_argmax": [p, p, i, i, p],
         "cisr_sample": [p, p, p, p, p, i, i, p],
     }
     for d in MFMA_HEAD_PADS:
-        sig[f"cisr_attn_mfma_d{d}"] = [p, i, p, p, p, i, p, i, p, p, p, p, p, i, i, i, i, i, f, i, i, p]
+        sig[f"cisr_attn_mfma_d{d}"] = [p, i, p, p, p, i, p, i, p, p, p, p, p, i, i, i, i, i, f, i, i, i, p]
     for name, args in sig.items():
         fn = getattr(h, name)
         fn.argtypes = args
@@ -249,7 +250,8 @@ def gemm(a, w, out, residual=None):
                                    rp, ldr, m, n, k, _stream())
     elif a.dtype == torch.bfloat16 and m <= SKINNY_ROWS and _skinny_ok(a, w):
         code = lib().cisr_gemm_skinny_bf16(a.data_ptr(), a.stride(0), w.data_ptr(), w.stride(0), out.data_ptr(),
-                                           out.stride(0), rp, ldr, m, n, k, _storage(out, "out"), 0, _stream())
+                                           out.stride(0), rp, ldr, m, n, k, _storage(out, "out"), 0, None, 0.0, None,
+                                           _stream())
     elif a.dtype == torch.bfloat16:
         code = lib().cisr_gemm_bf16(a.data_ptr(), a.stride(0), w.data_ptr(), w.stride(0), out.data_ptr(), out.stride(0),
                                     rp, ldr, m, n, k, _storage(out, "out"), _stream())
@@ -265,19 +267,59 @@ def _skinny_ok(a, w):
             and w.data_ptr() % 16 == 0)
 
 
-def gemm_swiglu(a, w_gate_up, out, scratch=None):
+def _norm_args(x, norm, k):
+    """(weight pointer, eps, rows pointer, number of output rows) for a fused RMSNorm prologue."""
+    weight, eps, rows = norm
+    _dev(x, "x", torch.float32)
+    if x.shape[1] != k or x.stride(0) % 8 or x.data_ptr() % 16:
+        raise KernelError("fused norm: the residual rows must be 32-byte aligned floats of the product's inner size")
+    wp = _dev(weight, "norm weight", torch.float32, (k,))
+    rp = None if rows is None else _dev(rows, "rows", torch.int32)
+    return wp, float(eps), rp, (x.shape[0] if rows is None else rows.shape[0])
+
+
+def fused_norm_ok(x, w, rows_out):
+    """Whether the weight-streaming kernel can take RMSNorm(x) . w^T with the norm fused."""
+    return (w.dtype == torch.bfloat16 and rows_out <= SKINNY_ROWS and x.dtype == torch.float32 and x.shape[1] % 8 == 0
+            and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w.stride(0) % 8 == 0 and w.data_ptr() % 16 == 0)
+
+
+def gemm_normed(x, norm, w, out):
+    """out[R, N] = RMSNorm(x[rows]) . w^T with the norm applied inside the product's kernel.
+    x float [T, K]; norm = (weight float [K], eps, rows int32 [R] or None); w bf16 [N, K]; out float or bf16."""
+    n, k = w.shape
+    wp, eps, rp, m = _norm_args(x, norm, k)
+    if not fused_norm_ok(x, w, m) or tuple(out.shape) != (m, n) or out.stride(1) != 1:
+        raise KernelError("gemm_normed: shape not supported by the fused kernel")
+    _check(lib().cisr_gemm_skinny_bf16(x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), out.data_ptr(), out.stride(0),
+                                       None, 0, m, n, k, _storage(out, "out"), 0, wp, eps, rp, _stream()), "gemm_normed")
+    return out
+
+
+def gemm_swiglu(a, w_gate_up, out, scratch=None, norm=None):
     """out[M, I] = silu(a . Wg^T) * (a . Wu^T) with w_gate_up = [Wg; Wu] ([2I, K]).
-    Few rows of bf16 run one fused weight-streaming kernel; otherwise the product
-    goes to `scratch` [M, 2I] and the activation is a second kernel."""
+    Few rows of bf16 run one fused weight-streaming kernel (with `norm` = (weight, eps, None), `a` is the float
+    residual and RMSNorm is fused too); otherwise the product goes to `scratch` [M, 2I] and the activation is
+    a second kernel."""
     m, k = a.shape
     two_i, k2 = w_gate_up.shape
     inter = two_i // 2
-    if k != k2 or two_i % 2 or tuple(out.shape) != (m, inter) or out.dtype != a.dtype or a.dtype != w_gate_up.dtype:
-        raise KernelError("gemm_swiglu: shapes or dtypes do not fit")
-    if a.dtype == torch.bfloat16 and m <= SKINNY_ROWS and _skinny_ok(a, w_gate_up) and a.is_cuda and out.is_contiguous():
+    if k != k2 or two_i % 2 or tuple(out.shape) != (m, inter) or not out.is_contiguous():
+        raise KernelError("gemm_swiglu: shapes do not fit")
+    if norm is not None:
+        wp, eps, rp, _ = _norm_args(a, norm, k)
+        if not fused_norm_ok(a, w_gate_up, m) or out.dtype != torch.bfloat16:
+            raise KernelError("gemm_swiglu: shape not supported by the fused kernel")
         _check(lib().cisr_gemm_skinny_bf16(a.data_ptr(), a.stride(0), w_gate_up.data_ptr(), w_gate_up.stride(0),
-                                           out.data_ptr(), out.stride(0), None, 0, m, inter, k, BF16, inter, _stream()),
-               "gemm_swiglu")
+                                           out.data_ptr(), out.stride(0), None, 0, m, inter, k, BF16, inter, wp, eps, rp,
+                                           _stream()), "gemm_swiglu")
+        return out
+    if out.dtype != a.dtype or a.dtype != w_gate_up.dtype:
+        raise KernelError("gemm_swiglu: dtypes differ")
+    if a.dtype == torch.bfloat16 and m <= SKINNY_ROWS and _skinny_ok(a, w_gate_up) and a.is_cuda:
+        _check(lib().cisr_gemm_skinny_bf16(a.data_ptr(), a.stride(0), w_gate_up.data_ptr(), w_gate_up.stride(0),
+                                           out.data_ptr(), out.stride(0), None, 0, m, inter, k, BF16, inter, None, 0.0,
+                                           None, _stream()), "gemm_swiglu")
         return out
     if scratch is None:
         raise KernelError("gemm_swiglu: this shape needs a scratch buffer [M, 2I]")
@@ -285,10 +327,48 @@ def gemm_swiglu(a, w_gate_up, out, scratch=None):
     return swiglu(scratch, out)
 
 
+def qkv_rope_fused_ok(a, w, head_dim, cos, normed):
+    """Whether the fused projection + rotary + scatter kernel takes this shape."""
+    m, k = a.shape
+    return (w.dtype == torch.bfloat16 and m <= SKINNY_ROWS and k % 8 == 0 and head_dim % 16 == 0
+            and 2 * cos.shape[1] == head_dim and a.stride(0) % 8 == 0 and a.data_ptr() % 16 == 0
+            and w.stride(0) % 8 == 0 and w.data_ptr() % 16 == 0
+            and a.dtype == (torch.float32 if normed else torch.bfloat16))
+
+
+def qkv_rope(a, w, q_out, positions, slots, cos, sin, kcache, vcache, heads, kv_heads, dim, page_size, norm=None):
+    """One kernel for a decode step's projections: (RMSNorm of the float residual `a` if `norm` = (weight, eps),
+    else `a` is bf16 and normed), product with w = [Wq; Wk; Wv], rotary embedding of q and k, q into
+    q_out [M, heads*dim], k and v into the cache at `slots`.  kcache None: w = Wq only (a layer reading
+    another layer's cache)."""
+    m, k = a.shape
+    has_kv = kcache is not None
+    n_kv = kv_heads if has_kv else 0
+    if not qkv_rope_fused_ok(a, w, dim, cos, norm is not None) or tuple(w.shape) != ((heads + 2 * n_kv) * dim, k):
+        raise KernelError("qkv_rope: shape not supported by the fused kernel")
+    wp, eps = (None, 0.0)
+    if norm is not None:
+        wp, eps = _dev(norm[0], "norm weight", torch.float32, (k,)), float(norm[1])
+    kp = vp = sp = None
+    if has_kv:
+        pages = kcache.shape[0]
+        kp = _dev(kcache, "kcache", torch.bfloat16, (pages, kv_heads, page_size, dim))
+        vp = _dev(vcache, "vcache", torch.bfloat16, (pages, kv_heads, dim, page_size))
+        sp = _dev(slots, "slots", torch.int32, (m,))
+    max_pos = cos.shape[0]
+    _check(lib().cisr_qkv_rope_skinny(a.data_ptr(), a.stride(0), w.data_ptr(), w.stride(0),
+                                      _dev(q_out, "q_out", torch.bfloat16, (m, heads * dim)), heads * dim, m, k, wp, eps,
+                                      _dev(positions, "positions", torch.int32, (m,)), sp,
+                                      _dev(cos, "cos", torch.float32), _dev(sin, "sin", torch.float32, (max_pos, dim // 2)),
+                                      kp, vp, heads, n_kv, dim, page_size, max_pos, _stream()), "qkv_rope")
+    return q_out
+
+
 def attention_mfma(q, q_row_stride, kcache, vcache, tables, seg_of_row, positions, out, heads, kv_heads, dim,
-                   page_size, window, scale, tasks=None, splits=1, workspace=None):
+                   page_size, window, scale, tasks=None, splits=1, workspace=None, waves=4):
     """Matrix-core attention (bf16).  tasks int32 [n, 4] = (segment, first row, rows, 0) runs tiles of
-    prompt rows; tasks None runs one block per row (decode) with `splits` blocks along the keys."""
+    prompt rows; tasks None runs one block per row (decode) of `waves` wavefronts (4 or 16) with `splits`
+    blocks along the keys; splits > 1 needs workspace = (partials float, statistics float) and a merge."""
     rows = out.shape[0]
     if not mfma_attention_supported(out.dtype, dim, page_size):
         raise KernelError(f"attention_mfma: head size {dim} / page size {page_size} / dtype {out.dtype} not supported")
@@ -318,10 +398,10 @@ def attention_mfma(q, q_row_stride, kcache, vcache, tables, seg_of_row, position
               _dev(vcache, "vcache", None, (pages, kv_heads, dim, page_size)), _dev(tables, "tables", torch.int32),
               tables.shape[1], tp, n_tasks, _dev(seg_of_row, "seg_of_row", torch.int32, (rows,)),
               _dev(positions, "positions", torch.int32, (rows,)), _dev(out, "out", None, (rows, heads * dim)), po, pm,
-              heads, kv_heads, dim, page_size.bit_length() - 1, int(window or 0), float(scale), int(splits), mode, _stream()),
-           "attention_mfma")
+              heads, kv_heads, dim, page_size.bit_length() - 1, int(window or 0), float(scale), int(splits), mode, int(waves),
+              _stream()), "attention_mfma")
     if mode == 1 and splits > 1:
-        _check(lib().cisr_attn_merge(po, pm, out.data_ptr(), rows, heads, dim, int(splits), BF16, _stream()), "attention_merge")
+        _check(lib().cisr_attn_merge(po, pm, out.data_ptr(), rows, heads, dim, int(splits), _stream()), "attention_merge")
     return out
 
 

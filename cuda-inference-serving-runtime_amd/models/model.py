@@ -92,5 +92,7 @@ class Model:
             x = self.layers[entry.layer].forward(x, ctx, self.site_of(index))
         if ctx.logit_rows.shape[0] == 0:
             return None
+        if self.head.fuses_norm(self.final_norm, x, ctx.logit_rows):
+            return self.head.forward(None, ctx, norm=self.final_norm, residual=x)
         h = self.final_norm.forward(x, ctx, rows=ctx.logit_rows, tag="final_norm")
         return self.head.forward(h, ctx)

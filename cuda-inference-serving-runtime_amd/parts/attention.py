@@ -17,6 +17,7 @@ import torch
 from ..cache.pages import KVNeed
 from ..kernels import ops
 from .base import Mixer, TensorSpec, matrix_operand, register_part
+from .norm import RMSNorm
 
 
 class PagedAttention(Mixer):
@@ -50,21 +51,36 @@ class PagedAttention(Mixer):
     def prepare(self, device, dtype):
         self.position.prepare(device, dtype)
 
-    def forward(self, h, residual, ctx, site):
-        T = h.shape[0]
+    def _fused_projection_ok(self, a, normed):
+        cos, _ = self.position.tables()
+        return ops.qkv_rope_fused_ok(a, self.w_in, self.head_dim, cos, normed)
+
+    def fuses_norm(self, norm, residual, ctx):
+        return isinstance(norm, RMSNorm) and self._fused_projection_ok(residual, True)
+
+    def forward(self, h, residual, ctx, site, norm=None):
+        T = residual.shape[0]
         D, nh, nkv = self.head_dim, self.heads, self.kv_heads
-        width = (nh + (2 * nkv if self.own_kv else 0)) * D
-        qkv = ctx.buffer("attn.qkv", (T, width), ctx.dtype)
-        ops.gemm(h, self.w_in, qkv)
         gid, kcache, vcache = ctx.cache.kv_of_site(site)
         view = ctx.kv[gid]
         cos, sin = self.position.tables()
-        if self.own_kv:
-            ops.rope_scatter(qkv, ctx.positions, view.slots, cos, sin, kcache, vcache, nh, nkv, D, view.page_size)
+        if not self.own_kv:
+            kcache_w = vcache_w = slots = None
         else:
-            ops.rope_scatter(qkv, ctx.positions, None, cos, sin, None, None, nh, nkv, D, view.page_size)
+            kcache_w, vcache_w, slots = kcache, vcache, view.slots
+        if norm is not None or self._fused_projection_ok(h, False):
+            # few rows: norm, projections, rotary embedding and the cache write are one kernel
+            q, q_stride = ctx.buffer("attn.q", (T, nh * D), ctx.dtype), nh * D
+            ops.qkv_rope(residual if norm is not None else h, self.w_in, q, ctx.positions, slots, cos, sin,
+                         kcache_w, vcache_w, nh, nkv, D, view.page_size,
+                         norm=(norm.weight, norm.eps) if norm is not None else None)
+        else:
+            q_stride = (nh + (2 * nkv if self.own_kv else 0)) * D
+            q = ctx.buffer("attn.qkv", (T, q_stride), ctx.dtype)
+            ops.gemm(h, self.w_in, q)
+            ops.rope_scatter(q, ctx.positions, slots, cos, sin, kcache_w, vcache_w, nh, nkv, D, view.page_size)
         out = ctx.buffer("attn.out", (T, nh * D), ctx.dtype)
-        ctx.attend(qkv, width, kcache, vcache, view, out, nh, nkv, D, self.window, self.scale)
+        ctx.attend(q, q_stride, kcache, vcache, view, out, nh, nkv, D, self.window, self.scale)
         return ops.gemm(out, self.w_out, residual, residual=residual)
 
 

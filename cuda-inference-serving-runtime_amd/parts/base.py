@@ -6,12 +6,15 @@ which model it is in.  Kinds of part:
 
   norm      forward(x_float[T, H], ctx, rows=None) -> activations [T or R, H]
   position  tables(device) -> (cos, sin) float [max_pos, rot/2] used by mixers
-  mixer     forward(h[T, H], residual[T, H] float, ctx, site) -> residual
-  ffn       forward(h[T, H], residual[T, H] float, ctx) -> residual
+  mixer     forward(h[T, H], residual[T, H] float, ctx, site, norm=None) -> residual
+  ffn       forward(h[T, H], residual[T, H] float, ctx, norm=None) -> residual
   block     forward(residual, ctx, site) -> residual  (the arrangement of the four)
 
 Mixers and feed-forwards add their result to the float residual stream
 themselves (their last matrix product does it in its epilogue) and return it.
+A mixer or feed-forward may take over the norm in front of it: if its
+`fuses_norm(norm, residual, ctx)` says so for a step, the block passes h=None
+and the norm part, and the part applies the norm inside its first kernel.
 A mixer states what it keeps between steps: `cache_need()` (pages of keys and
 values) and/or `state_need()` (a fixed-size state per request), or neither.
 """
@@ -65,12 +68,18 @@ class Mixer(Part):
     def state_need(self):
         return None
 
-    def forward(self, h, residual, ctx, site):
+    def fuses_norm(self, norm, residual, ctx):
+        return False
+
+    def forward(self, h, residual, ctx, site, norm=None):
         raise NotImplementedError
 
 
 class FeedForward(Part):
-    def forward(self, h, residual, ctx):
+    def fuses_norm(self, norm, residual, ctx):
+        return False
+
+    def forward(self, h, residual, ctx, norm=None):
         raise NotImplementedError
 
 

@@ -23,10 +23,13 @@ class PreNormBlock(Part):
             p.prepare(device, dtype)
 
     def forward(self, residual, ctx, site):
-        h = self.mixer_norm.forward(residual, ctx)
-        residual = self.mixer.forward(h, residual, ctx, site)
-        h = self.ffn_norm.forward(residual, ctx)
-        return self.ffn.forward(h, residual, ctx)
+        if self.mixer.fuses_norm(self.mixer_norm, residual, ctx):
+            residual = self.mixer.forward(None, residual, ctx, site, norm=self.mixer_norm)
+        else:
+            residual = self.mixer.forward(self.mixer_norm.forward(residual, ctx), residual, ctx, site)
+        if self.ffn.fuses_norm(self.ffn_norm, residual, ctx):
+            return self.ffn.forward(None, residual, ctx, norm=self.ffn_norm)
+        return self.ffn.forward(self.ffn_norm.forward(residual, ctx), residual, ctx)
 
 
 register_part("block", "prenorm", PreNormBlock)

@@ -8,6 +8,7 @@ import torch
 
 from ..kernels import ops
 from .base import Part, TensorSpec, matrix_operand
+from .norm import RMSNorm
 
 
 class TokenEmbedding(Part):
@@ -37,6 +38,13 @@ class LMHead(Part):
     def bind(self, tensors, dtype):
         self.weight = self.tied_to.weight if self.tied_to is not None else matrix_operand(tensors[self.name + ".weight"], dtype)
 
-    def forward(self, h, ctx):
-        logits = ctx.buffer("logits", (h.shape[0], self.vocab), torch.float32)
+    def fuses_norm(self, norm, residual, rows):
+        return isinstance(norm, RMSNorm) and ops.fused_norm_ok(residual, self.weight, rows.shape[0])
+
+    def forward(self, h, ctx, norm=None, residual=None):
+        """Logits of the normed rows h; or, with `norm`, of RMSNorm(residual[ctx.logit_rows]) in one kernel."""
+        n = ctx.logit_rows.shape[0] if norm is not None else h.shape[0]
+        logits = ctx.buffer("logits", (n, self.vocab), torch.float32)
+        if norm is not None:
+            return ops.gemm_normed(residual, (norm.weight, norm.eps, ctx.logit_rows), self.weight, logits)
         return ops.gemm(h, self.weight, logits)

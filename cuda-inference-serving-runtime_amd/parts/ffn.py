@@ -5,6 +5,7 @@ import torch
 
 from ..kernels import ops
 from .base import FeedForward, TensorSpec, matrix_operand, register_part
+from .norm import RMSNorm
 
 
 class GatedMLP(FeedForward):
@@ -25,10 +26,15 @@ class GatedMLP(FeedForward):
         self.w_gate_up = torch.cat([gate, up], dim=0).contiguous()
         self.w_down = matrix_operand(tensors[f"{self.name}.down_proj.weight"], dtype)
 
-    def forward(self, h, residual, ctx):
-        T = h.shape[0]
+    def fuses_norm(self, norm, residual, ctx):
+        return isinstance(norm, RMSNorm) and ops.fused_norm_ok(residual, self.w_gate_up, residual.shape[0])
+
+    def forward(self, h, residual, ctx, norm=None):
+        T = residual.shape[0]
         act = ctx.buffer("ffn.act", (T, self.intermediate), ctx.dtype)
-        if ctx.dtype == torch.bfloat16 and T <= ops.SKINNY_ROWS:
+        if norm is not None:
+            ops.gemm_swiglu(residual, self.w_gate_up, act, norm=(norm.weight, norm.eps, None))
+        elif ctx.dtype == torch.bfloat16 and T <= ops.SKINNY_ROWS:
             ops.gemm_swiglu(h, self.w_gate_up, act)   # fused when the fast kernel takes the shape
         else:
             ops.gemm_swiglu(h, self.w_gate_up, act, scratch=ctx.buffer("ffn.gate_up", (T, 2 * self.intermediate), ctx.dtype))

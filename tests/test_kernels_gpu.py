@@ -265,7 +265,7 @@ def test_attention_equal_large_scores_give_the_mean(ops):
     np.testing.assert_allclose(f64(out).reshape(heads, dim)[3], f64(vc)[0, 1, :, :n].mean(-1), rtol=1e-6)
 
 
-def run_mfma(ops, qt, kt, vt, tables, rows, page_size, mode, splits=1, window=None, scale=None, rows_per_tile=None):
+def run_mfma(ops, qt, kt, vt, tables, rows, page_size, mode, splits=1, window=None, scale=None, rows_per_tile=None, waves=4):
     """mode "tiles": rows are grouped into tiles of consecutive rows of one segment;
     mode "rows": one block per row with `splits` blocks along the keys."""
     T, heads, dim = qt.shape
@@ -286,7 +286,7 @@ def run_mfma(ops, qt, kt, vt, tables, rows, page_size, mode, splits=1, window=No
             items.append((rows[i][0], i, n, 0)); i += n
         tasks = torch.tensor(items, dtype=torch.int32, device=DEV)
     ops.attention_mfma(qt.reshape(T, heads * dim), heads * dim, kt, vt, tables, seg, pos, out, heads, kv_heads, dim,
-                       page_size, window, scale if scale is not None else 1 / math.sqrt(dim), tasks, splits, ws)
+                       page_size, window, scale if scale is not None else 1 / math.sqrt(dim), tasks, splits, ws, waves)
     return f64(out).reshape(T, heads, dim)
 
 
@@ -300,12 +300,17 @@ def test_attention_mfma_rows(ops, heads, kv_heads, dim, page_size):
     qt, kt, vt, tables, rows = paged_case(heads, kv_heads, dim, page_size, [17, 7, 1, 130, 333], torch.bfloat16, seed=dim + heads)
     want = reference_attention(qt, kt, vt, tables, rows, page_size)
     for splits in (1, 2, 3, 16):
-        got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, "rows", splits)
-        np.testing.assert_allclose(got, want, **MFMA_TOL, err_msg=f"splits={splits}")
+        for waves in (4, 16):
+            if waves == 16 and min(heads // kv_heads, 16) * (-(-dim // 32) * 32 + 2) * 64 > 128 * 1024:
+                continue
+            got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, "rows", splits, waves=waves)
+            np.testing.assert_allclose(got, want, **MFMA_TOL, err_msg=f"splits={splits} waves={waves}")
     rows2 = list(rows); rows2[0] = (-1, 0)            # a padding row gives zeros
     got = run_mfma(ops, qt, kt, vt, tables, rows2, page_size, "rows", 2)
     assert (got[0] == 0).all()
     np.testing.assert_allclose(got[1:], want[1:], **MFMA_TOL)
+    again = [run_mfma(ops, qt, kt, vt, tables, rows, page_size, "rows", 16) for _ in range(3)]
+    assert all((a == again[0]).all() for a in again)  # the merge order is fixed: repeated runs agree bit for bit
 
 
 def portion_case(heads, kv_heads, dim, page_size, plan, seed):
@@ -378,6 +383,74 @@ def test_gemm_skinny_and_fused_swiglu(ops):
     full = ops.gemm(a, w, torch.empty(64, 300, device=DEV))
     for m in (1, 5, 16, 17, 48):
         assert torch.equal(ops.gemm(a[:m].contiguous(), w, torch.empty(m, 300, device=DEV)), full[:m])
+
+
+def test_fused_norm_products(ops):
+    """RMSNorm inside the product's kernel (plain, row-gathered, SwiGLU) against norm then product."""
+    for M, N, K, eps in [(1, 48, 64, 1e-5), (8, 1728, 576, 1e-5), (33, 130, 200, 1e-6), (64, 100, 144, 1e-2)]:
+        x = rnd(M + 3, K, seed=1, scale=2.0)
+        nw = 1 + 0.1 * rnd(K, seed=2)
+        w = rnd(N, K, dtype=torch.bfloat16, seed=3, scale=0.1)
+        h = P.rmsnorm(f64(x), f64(nw), eps)
+        want = h @ f64(w).T
+        scale = np.abs(want).max()
+        got = ops.gemm_normed(x[:M], (nw, eps, None), w, torch.empty(M, N, device=DEV))
+        assert np.abs(f64(got) - want[:M]).max() < 6e-3 * scale      # operands rounded to bf16 as in the two-kernel path
+        rows = torch.tensor([M + 2, 0, M // 2], dtype=torch.int32, device=DEV)
+        got = ops.gemm_normed(x, (nw, eps, rows), w, torch.empty(3, N, dtype=torch.bfloat16, device=DEV))
+        assert np.abs(f64(got) - want[[M + 2, 0, M // 2]]).max() < 1.2e-2 * scale
+        # against the engine's own two-kernel path: same roundings up to the place of the row factor
+        hb = ops.rmsnorm(x[:M].contiguous(), nw, torch.empty(M, K, dtype=torch.bfloat16, device=DEV), eps)
+        two = ops.gemm(hb, w, torch.empty(M, N, device=DEV))
+        one = ops.gemm_normed(x[:M], (nw, eps, None), w, torch.empty(M, N, device=DEV))
+        assert np.abs(f64(one) - f64(two)).max() < 6e-3 * scale
+    M, I, K = 8, 172, 64
+    x, nw = rnd(M, K, seed=4), 1 + 0.1 * rnd(K, seed=5)
+    w = rnd(2 * I, K, dtype=torch.bfloat16, seed=6, scale=0.3)
+    gu = P.rmsnorm(f64(x), f64(nw), 1e-5) @ f64(w).T
+    want = P.swiglu(gu[:, :I], gu[:, I:])
+    got = ops.gemm_swiglu(x, w, torch.empty(M, I, dtype=torch.bfloat16, device=DEV), norm=(nw, 1e-5, None))
+    assert np.abs(f64(got) - want).max() < 2e-2 * np.abs(want).max()
+
+
+@pytest.mark.parametrize("heads, kv_heads, dim, theta, normed", [(4, 2, 16, 1e4, True), (9, 3, 64, 1e5, True), (2, 1, 128, 5e5, False), (3, 3, 48, 1e4, True)])
+def test_fused_projection_rotary_scatter(ops, heads, kv_heads, dim, theta, normed):
+    from runtime.parts import RotaryEmbedding
+    rope = RotaryEmbedding(dim, theta, 700); rope.prepare(DEV, torch.bfloat16)
+    cos, sin = rope.tables()
+    M, K, P_, pages = 5, 72, 4, 8
+    pos = [0, 17, 500, 699, 3]
+    slots = [5, 0, 22, -1, 9]
+    x = rnd(M, K, seed=1, scale=1.5)
+    nw = 1 + 0.1 * rnd(K, seed=2)
+    w = rnd((heads + 2 * kv_heads) * dim, K, dtype=torch.bfloat16, seed=3, scale=0.2)
+    h = P.rmsnorm(f64(x), f64(nw), 1e-5) if normed else f64(x.bfloat16())
+    ref = h @ f64(w).T
+    q_ref = P.rope(ref[:, :heads * dim].reshape(M, heads, dim), pos, theta)
+    k_ref = P.rope(ref[:, heads * dim:(heads + kv_heads) * dim].reshape(M, kv_heads, dim), pos, theta)
+    v_ref = ref[:, (heads + kv_heads) * dim:].reshape(M, kv_heads, dim)
+    kc = torch.full((pages, kv_heads, P_, dim), 7.0, dtype=torch.bfloat16, device=DEV)
+    vc = torch.full((pages, kv_heads, dim, P_), 7.0, dtype=torch.bfloat16, device=DEV)
+    q = torch.empty(M, heads * dim, dtype=torch.bfloat16, device=DEV)
+    a = x if normed else x.bfloat16()
+    ops.qkv_rope(a, w, q, torch.tensor(pos, dtype=torch.int32, device=DEV), torch.tensor(slots, dtype=torch.int32, device=DEV),
+                 cos, sin, kc, vc, heads, kv_heads, dim, P_, norm=(nw, 1e-5) if normed else None)
+    tol = dict(rtol=2e-2, atol=2e-2 * np.abs(ref).max())
+    np.testing.assert_allclose(f64(q).reshape(M, heads, dim), q_ref, **tol)
+    kc64, vc64 = f64(kc), f64(vc)
+    for t, s_ in enumerate(slots):
+        if s_ < 0:
+            continue
+        np.testing.assert_allclose(kc64[s_ // P_, :, s_ % P_], k_ref[t], **tol)
+        np.testing.assert_allclose(vc64[s_ // P_, :, :, s_ % P_], v_ref[t], **tol)
+    untouched = [s_ for s_ in range(pages * P_) if s_ not in slots]
+    assert all((kc64[s_ // P_, :, s_ % P_] == 7).all() and (vc64[s_ // P_, :, :, s_ % P_] == 7).all() for s_ in untouched)
+    # q only (a layer that reads another layer's cache)
+    wq = w[:heads * dim].contiguous()
+    q2 = torch.empty_like(q)
+    ops.qkv_rope(a, wq, q2, torch.tensor(pos, dtype=torch.int32, device=DEV), None, cos, sin, None, None, heads, kv_heads, dim, P_,
+                 norm=(nw, 1e-5) if normed else None)
+    assert torch.equal(q, q2)
 
 
 GEMM_SHAPES = [(1, 1, 1), (5, 7, 9), (64, 64, 32), (130, 200, 172), (33, 513, 144), (17, 130, 1000), (300, 129, 72), (8, 1536, 576)]

@@ -154,8 +154,12 @@ def test_logits_do_not_depend_on_the_cut_or_the_company(folders, tmp_path, dtype
     run(folders[name], dtype, cut, tmp_path / "cut", page_size=8)
     x = np.fromfile(tmp_path / "whole" / "0.f32", "<f4").reshape(90, V)
     y = np.concatenate([np.fromfile(tmp_path / "cut" / f"{s}.f32", "<f4").reshape(-1, V) for s in sorted(cut.expect)])
-    bound = 2e-5 if dtype == "float32" else 2e-2
-    assert np.abs(x - y).max() / np.abs(x).max() < bound
+    if dtype == "float32":
+        assert np.abs(x - y).max() / np.abs(x).max() < 2e-5
+    else:   # the two runs round at different places (other kernels for portions and single tokens);
+        # the bound is the one that holds against the plain implementation
+        from conftest import BF16_RMSE
+        assert np.linalg.norm(x - y) / np.linalg.norm(x) < BF16_RMSE
 
 
 def test_out_of_pages_and_bad_input_fail_loudly(folders, tmp_path):

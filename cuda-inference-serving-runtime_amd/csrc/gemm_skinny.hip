@@ -1,10 +1,10 @@
 // Skinny matrix products for decode steps:  C[M,N] = A[M,K] . W[N,K]^T  with
 // M <= 64 rows.  The product is bound by reading W once from HBM, so the kernel
 // is laid out around streaming W: a block owns 16 rows of W (16 output columns),
-// its four waves split K in interleaved 32-wide steps, every lane loads 16
-// contiguous bytes of a W row straight into a matrix-core operand
+// its waves (4, or 16 for a short K) split K in interleaved 32-wide steps, every
+// lane loads 16 contiguous bytes of a W row straight into a matrix-core operand
 // (v_mfma_f32_16x16x32_bf16, A as the first operand, W as the second), and the
-// four partial tiles are summed through LDS in a fixed order, so a row's result
+// waves' partial tiles are summed through LDS in a fixed order, so a row's result
 // does not depend on how many rows are beside it.
 //
 // Prologue (NORM): A is the float residual stream and the kernel applies RMSNorm
@@ -50,12 +50,17 @@ __device__ __forceinline__ uint32_t pack2(float a, float b) {
     return (uint32_t)f32_to_bf16(a) | ((uint32_t)f32_to_bf16(b) << 16);
 }
 
-template <int MT, bool NORM, int EPI, typename TC>
-__global__ void __launch_bounds__(256)
+// NW: wavefronts a block (4 or 16).  A short K is split over 16 waves so that every wave
+// issues all its loads at once (one trip to memory); a long K over 4 waves that keep
+// several steps of loads in flight.
+template <int MT, bool NORM, int EPI, typename TC, int NW>
+__global__ void __launch_bounds__(NW * 64)
 gemm_skinny_kernel(SkinnyArgs p) {
     constexpr int NB = EPI == EPI_SWIGLU ? 2 : 1;
-    __shared__ float red[4][NB][MT][WAVE][4];
-    __shared__ float ssq[4][MT][16];
+    constexpr int UNROLL = MT == 1 ? 8 : (MT == 2 ? 4 : 2);
+    extern __shared__ float smem[];
+    float (*red)[NB][MT][WAVE][4] = reinterpret_cast<float (*)[NB][MT][WAVE][4]>(smem);
+    float (*ssq)[MT][16] = reinterpret_cast<float (*)[MT][16]>(smem + NW * NB * MT * WAVE * 4);
     const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
     const int r = lane % 16, g = lane / 16;
     const int M = p.M, N = p.N, K = p.K;
@@ -97,8 +102,8 @@ gemm_skinny_kernel(SkinnyArgs p) {
     }
 
     // this wave's k-steps: wave, wave + 4, ...; K % 8 == 0, so a 16-byte chunk is inside K or outside
-#pragma unroll 2
-    for (int k0 = wave * 32; k0 < K; k0 += 4 * 32) {
+#pragma unroll UNROLL
+    for (int k0 = wave * 32; k0 < K; k0 += NW * 32) {
         const bool ok = k0 + g * 8 < K;
         const bf16x8 wf0 = ld16(wrow0 + k0, ok);
         bf16x8 wf1;
@@ -143,21 +148,29 @@ gemm_skinny_kernel(SkinnyArgs p) {
     }
     __syncthreads();
     // thread -> (l2 = tid % 64, e2 = tid / 64): element (m = 16 t + 4 (l2 / 16) + e2, column c = l2 % 16)
+    if (tid >= 256) return;
     const int l2 = tid % WAVE, e2 = tid / WAVE, c = l2 % 16;
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
         const int ml = (l2 / 16) * 4 + e2;              // row inside the 16-row tile
         const int m = t * 16 + ml;
         if (m >= M) continue;
-        float v = red[0][0][t][l2][e2] + red[1][0][t][l2][e2] + red[2][0][t][l2][e2] + red[3][0][t][l2][e2];
+        float v = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) v += red[w][0][t][l2][e2];
         float scale = 1.f;
         if (NORM) {
-            const float total = ssq[0][t][ml] + ssq[1][t][ml] + ssq[2][t][ml] + ssq[3][t][ml];
+            float total = 0.f;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) total += ssq[w][t][ml];
             scale = 1.0f / sqrtf(total / (float)K + p.eps);
             v *= scale;
         }
         if (EPI == EPI_SWIGLU) {
-            float u = (red[0][NB - 1][t][l2][e2] + red[1][NB - 1][t][l2][e2] + red[2][NB - 1][t][l2][e2] + red[3][NB - 1][t][l2][e2]) * scale;
+            float u = 0.f;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) u += red[w][NB - 1][t][l2][e2];
+            u *= scale;
             // the two-kernel path rounds gate and up to bf16 before the activation; do the same
             const float gq = bf16_to_f32(f32_to_bf16(v)), uq = bf16_to_f32(f32_to_bf16(u));
             v = gq / (1.0f + expf(-gq)) * uq;
@@ -165,7 +178,10 @@ gemm_skinny_kernel(SkinnyArgs p) {
         if (EPI == EPI_ROPE) {
             // partner column (the other half of the rotary pair) sits 8 lanes away
             const int lp = l2 ^ 8;
-            const float pv = (red[0][0][t][lp][e2] + red[1][0][t][lp][e2] + red[2][0][t][lp][e2] + red[3][0][t][lp][e2]) * scale;
+            float pv = 0.f;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) pv += red[w][0][t][lp][e2];
+            pv *= scale;
             const int D = p.head_dim, half = D / 2;
             const int i = j0 + (c & 7);
             const int col = c < 8 ? i : half + i;
@@ -199,18 +215,27 @@ gemm_skinny_kernel(SkinnyArgs p) {
     }
 }
 
-template <int MT, bool NORM, int EPI, typename TC>
+template <int MT, bool NORM, int EPI, typename TC, int NW>
 static int launch_one(const SkinnyArgs& a, int blocks, hipStream_t stream) {
-    gemm_skinny_kernel<MT, NORM, EPI, TC><<<blocks, 256, 0, stream>>>(a);
+    constexpr int NB = EPI == EPI_SWIGLU ? 2 : 1;
+    const size_t shmem = ((size_t)NW * NB * MT * WAVE * 4 + (size_t)NW * MT * 16) * sizeof(float);
+    if (shmem > 65536) {
+        hipError_t e = hipFuncSetAttribute((const void*)gemm_skinny_kernel<MT, NORM, EPI, TC, NW>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+        if (e != hipSuccess) return (int)e;
+    }
+    gemm_skinny_kernel<MT, NORM, EPI, TC, NW><<<blocks, NW * 64, shmem, stream>>>(a);
     return CISR_LAUNCH_CHECK();
 }
 
 template <bool NORM, int EPI, typename TC>
 static int launch_mt(const SkinnyArgs& a, int blocks, hipStream_t stream) {
-    if (a.M <= 16) return launch_one<1, NORM, EPI, TC>(a, blocks, stream);
-    if (a.M <= 32) return launch_one<2, NORM, EPI, TC>(a, blocks, stream);
-    if (a.M <= 48) return launch_one<3, NORM, EPI, TC>(a, blocks, stream);
-    return launch_one<4, NORM, EPI, TC>(a, blocks, stream);
+    // a short inner size is split over 16 waves: at most 8 steps of 32 each, all loads issued at once
+    const bool wide = a.K <= 16 * 32 * 8;
+    if (a.M <= 16) return wide ? launch_one<1, NORM, EPI, TC, 16>(a, blocks, stream) : launch_one<1, NORM, EPI, TC, 4>(a, blocks, stream);
+    if (a.M <= 32) return wide ? launch_one<2, NORM, EPI, TC, 16>(a, blocks, stream) : launch_one<2, NORM, EPI, TC, 4>(a, blocks, stream);
+    if (a.M <= 48) return wide ? launch_one<3, NORM, EPI, TC, 16>(a, blocks, stream) : launch_one<3, NORM, EPI, TC, 4>(a, blocks, stream);
+    return wide ? launch_one<4, NORM, EPI, TC, 16>(a, blocks, stream) : launch_one<4, NORM, EPI, TC, 4>(a, blocks, stream);
 }
 
 static bool aligned16(const void* p) { return ((uintptr_t)p) % 16 == 0; }

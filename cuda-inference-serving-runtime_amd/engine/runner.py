@@ -306,16 +306,11 @@ class ModelRunner:
     @staticmethod
     def _rows_launch(blocks, span, heads_per_chunk, head_dim):
         """Matrix-core decode kernel: (wavefronts a block, blocks along the keys).  Few rows:
-        sixteen waves share a row's keys inside one block, so no second kernel has to merge
-        partials; only when even that leaves the GPU idle and the context is long are the keys
-        also split over blocks.  Many rows: four waves a block, one block a row and head group."""
+        eight waves share a row's keys inside one block; when that still leaves the GPU idle
+        and the context is long, the keys are also split over blocks (a merge kernel follows).
+        Many rows: four waves a block, one block a row and head group."""
         steps = -(-span // 32)
-        dpad = -(-head_dim // 32) * 32
-        wide_fits = 16 * heads_per_chunk * (dpad + 2) * 4 <= 128 * 1024
-        if blocks >= 512 or not wide_fits:
-            waves = 4
-        else:
-            waves = 16
+        waves = 8 if blocks < 512 and head_dim <= 128 else 4
         per_block = 4 * waves            # at least four 32-key steps a wave
         splits = int(max(1, min(steps // per_block, -(-512 // blocks), 64)))
         return waves, splits

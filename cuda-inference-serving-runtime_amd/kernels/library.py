@@ -47,7 +47,7 @@ def sources():
 def _digest():
     h = hashlib.sha256()
     h.update(" ".join(HIPCC_FLAGS).encode())
-    for path in sorted(CSRC.glob("*.hip")) + sorted(CSRC.glob("*.h")):
+    for path in sorted(p for p in CSRC.iterdir() if p.suffix in (".hip", ".h", ".inc")):
         h.update(path.name.encode())
         h.update(path.read_bytes())
     return h.hexdigest()[:16]

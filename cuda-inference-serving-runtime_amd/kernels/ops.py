@@ -367,7 +367,7 @@ def qkv_rope(a, w, q_out, positions, slots, cos, sin, kcache, vcache, heads, kv_
 def attention_mfma(q, q_row_stride, kcache, vcache, tables, seg_of_row, positions, out, heads, kv_heads, dim,
                    page_size, window, scale, tasks=None, splits=1, workspace=None, waves=4):
     """Matrix-core attention (bf16).  tasks int32 [n, 4] = (segment, first row, rows, 0) runs tiles of
-    prompt rows; tasks None runs one block per row (decode) of `waves` wavefronts (4 or 16) with `splits`
+    prompt rows; tasks None runs one block per row (decode) of `waves` wavefronts (4 or 8) with `splits`
     blocks along the keys; splits > 1 needs workspace = (partials float, statistics float) and a merge."""
     rows = out.shape[0]
     if not mfma_attention_supported(out.dtype, dim, page_size):

@@ -300,9 +300,7 @@ def test_attention_mfma_rows(ops, heads, kv_heads, dim, page_size):
     qt, kt, vt, tables, rows = paged_case(heads, kv_heads, dim, page_size, [17, 7, 1, 130, 333], torch.bfloat16, seed=dim + heads)
     want = reference_attention(qt, kt, vt, tables, rows, page_size)
     for splits in (1, 2, 3, 16):
-        for waves in (4, 16):
-            if waves == 16 and min(heads // kv_heads, 16) * (-(-dim // 32) * 32 + 2) * 64 > 128 * 1024:
-                continue
+        for waves in (4, 8):
             got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, "rows", splits, waves=waves)
             np.testing.assert_allclose(got, want, **MFMA_TOL, err_msg=f"splits={splits} waves={waves}")
     rows2 = list(rows); rows2[0] = (-1, 0)            # a padding row gives zeros

@@ -230,8 +230,9 @@ static int launch_one(const SkinnyArgs& a, int blocks, hipStream_t stream) {
 
 template <bool NORM, int EPI, typename TC>
 static int launch_mt(const SkinnyArgs& a, int blocks, hipStream_t stream) {
-    // a short inner size is split over 16 waves: at most 8 steps of 32 each, all loads issued at once
-    const bool wide = a.K <= 16 * 32 * 8;
+    // a short inner size with few blocks is split over 16 waves: at most 8 steps of 32 each, all loads
+    // issued at once; with many blocks (a vocabulary) four waves a block fill the GPU without that
+    const bool wide = a.K <= 16 * 32 * 8 && blocks <= 1024;
     if (a.M <= 16) return wide ? launch_one<1, NORM, EPI, TC, 16>(a, blocks, stream) : launch_one<1, NORM, EPI, TC, 4>(a, blocks, stream);
     if (a.M <= 32) return wide ? launch_one<2, NORM, EPI, TC, 16>(a, blocks, stream) : launch_one<2, NORM, EPI, TC, 4>(a, blocks, stream);
     if (a.M <= 48) return wide ? launch_one<3, NORM, EPI, TC, 16>(a, blocks, stream) : launch_one<3, NORM, EPI, TC, 4>(a, blocks, stream);

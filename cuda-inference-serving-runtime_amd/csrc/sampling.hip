@@ -42,19 +42,47 @@ __device__ __forceinline__ void argmax_block(const float* __restrict__ x, int n,
     __syncthreads();
 }
 
+// Greedy pick in two passes so that a few rows still fill the GPU: the vocabulary is cut
+// into `chunks` slices, one block each; a second pass picks among the slice winners
+// (lower slice first, so the lowest index still wins a tie).
 __global__ void __launch_bounds__(256)
-argmax_kernel(const float* __restrict__ logits, int* __restrict__ out, int vocab) {
+argmax_partial_kernel(const float* __restrict__ logits, float* __restrict__ pval, int* __restrict__ pidx,
+                      int vocab, int chunks) {
     __shared__ float smax[256];
     __shared__ int sidx[256];
-    const float* x = logits + (size_t)blockIdx.x * vocab;
+    const int row = blockIdx.x, chunk = blockIdx.y;
+    const int per = (vocab + chunks - 1) / chunks;
+    const int lo = chunk * per, n = max(0, min(vocab, lo + per) - lo);
     float best; int idx;
-    argmax_block(x, vocab, smax, sidx, best, idx);
-    if (threadIdx.x == 0) out[blockIdx.x] = idx == 0x7fffffff ? 0 : idx;
+    argmax_block(logits + (size_t)row * vocab + lo, n, smax, sidx, best, idx);
+    if (threadIdx.x == 0) {
+        pval[row * chunks + chunk] = best;
+        pidx[row * chunks + chunk] = idx == 0x7fffffff ? 0x7fffffff : lo + idx;
+    }
 }
 
-extern "C" int cisr_argmax(const float* logits, int* out, int rows, int vocab, hipStream_t stream) {
+__global__ void __launch_bounds__(64)
+argmax_final_kernel(const float* __restrict__ pval, const int* __restrict__ pidx, int* __restrict__ out, int chunks) {
+    const int row = blockIdx.x;
+    if (threadIdx.x != 0) return;
+    float bv = -INFINITY; int bi = 0x7fffffff;
+    for (int c = 0; c < chunks; ++c) {
+        const float v = pval[row * chunks + c]; const int i = pidx[row * chunks + c];
+        if (i != 0x7fffffff && (bi == 0x7fffffff || v > bv)) { bv = v; bi = i; }
+    }
+    out[row] = bi == 0x7fffffff ? 0 : bi;
+}
+
+#define ARGMAX_CHUNKS 32
+
+// scratch: float [rows * 32] and int [rows * 32]
+extern "C" int cisr_argmax(const float* logits, int* out, float* scratch_val, int* scratch_idx, int rows, int vocab,
+                           hipStream_t stream) {
     if (rows <= 0) return 0;
-    argmax_kernel<<<rows, 256, 0, stream>>>(logits, out, vocab);
+    argmax_partial_kernel<<<dim3(rows, ARGMAX_CHUNKS), 256, 0, stream>>>(logits, scratch_val, scratch_idx, vocab, ARGMAX_CHUNKS);
+    int err = CISR_LAUNCH_CHECK();
+    if (err) return err;
+    argmax_final_kernel<<<rows, 64, 0, stream>>>(scratch_val, scratch_idx, out, ARGMAX_CHUNKS);
     return CISR_LAUNCH_CHECK();
 }
 

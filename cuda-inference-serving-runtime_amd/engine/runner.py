@@ -311,6 +311,7 @@ class ModelRunner:
         Many rows: four waves a block, one block a row and head group."""
         steps = -(-span // 32)
         waves = 8 if blocks < 512 and head_dim <= 128 else 4
-        per_block = 4 * waves            # at least four 32-key steps a wave
-        splits = int(max(1, min(steps // per_block, -(-512 // blocks), 64)))
+        # as many blocks along the keys as keep about a thousand blocks in flight (the loads of a
+        # whole layer's cache are then outstanding at once), each wave with at least one 32-key step
+        splits = int(max(1, min(steps // waves, -(-1024 // blocks), 64)))
         return waves, splits

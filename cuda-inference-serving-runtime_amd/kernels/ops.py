@@ -51,7 +51,7 @@ def _declare(h):
         "cisr_gemm_skinny_bf16": [p, i, p, i, p, i, p, i, i, i, i, i, i, p, f, p, p],
         "cisr_qkv_rope_skinny": [p, i, p, i, p, i, i, i, p, f, p, p, p, p, p, p, i, i, i, i, i, p],
         "cisr_attn_merge": [p, p, p, i, i, i, i, p],
-        "cisr_argmax": [p, p, i, i, p],
+        "cisr_argmax": [p, p, p, p, i, i, p],
         "cisr_sample": [p, p, p, p, p, i, i, p],
     }
     for d in MFMA_HEAD_PADS:
@@ -410,10 +410,19 @@ def mfma_attention_supported(dtype, dim, page_size):
             and page_size & (page_size - 1) == 0)
 
 
+_argmax_scratch = {}
+
+
 def argmax(logits, out):
+    """out[r] = index of the largest logit of row r (the lowest index wins a tie)."""
     rows, vocab = logits.shape
-    _check(lib().cisr_argmax(_dev(logits, "logits", torch.float32), _dev(out, "out", torch.int32, (rows,)), rows, vocab,
-                             _stream()), "argmax")
+    key = (logits.device, rows)
+    if key not in _argmax_scratch:
+        _argmax_scratch[key] = (torch.empty(rows * 32, dtype=torch.float32, device=logits.device),
+                                torch.empty(rows * 32, dtype=torch.int32, device=logits.device))
+    val, idx = _argmax_scratch[key]
+    _check(lib().cisr_argmax(_dev(logits, "logits", torch.float32), _dev(out, "out", torch.int32, (rows,)),
+                             val.data_ptr(), idx.data_ptr(), rows, vocab, _stream()), "argmax")
     return out
 
 

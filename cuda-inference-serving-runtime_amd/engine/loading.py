@@ -33,7 +33,7 @@ def load_model(folder, dtype="bfloat16", device="cuda:0"):
     dtype = parse_dtype(dtype)
     raw = read_config_json(folder)
     _, _, model = build_from_config_dict(raw)
-    tensors = load_folder(folder, model.tensor_specs(), dtype, torch.device(device))
+    tensors = load_folder(folder, model.tensor_specs(), dtype, torch.device(device), ignored=model.ignored_tensors())
     model.bind(tensors, dtype, torch.device(device))
     return model
 

@@ -31,7 +31,7 @@ def replay(model_dir, dtype, out_dir, max_tokens, lines, page_size=PAGE_SIZE, ec
     out_dir.mkdir(parents=True, exist_ok=True)
     model = load_model(model_dir, dtype=dtype)
     pages = max(1, -(-int(max_tokens) // page_size))
-    runner = ModelRunner(model, n_pages=pages, page_size=page_size, max_requests=max(MAX_LIVE, 8))
+    runner = ModelRunner(model, n_pages=pages, page_size=page_size, max_requests=4 * MAX_LIVE)
     for line in lines:
         line = line.strip()
         if not line:

@@ -48,6 +48,12 @@ class Model:
                 specs.append(spec)
         return specs
 
+    def ignored_tensors(self):
+        """Names a checkpoint may hold that the model does not read: the copy of a tied head
+        (the reference overwrites it with the embedding, runtime/checkpoint.py:38-39)."""
+        tied = getattr(self.head, "tied_to", None)
+        return (self.head.name + ".weight",) if tied is not None else ()
+
     def bind(self, tensors, dtype, device):
         self.dtype, self.device = dtype, device
         for part in self.parts():

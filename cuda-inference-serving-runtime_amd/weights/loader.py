@@ -51,11 +51,12 @@ def open_folder(folder):
     return index
 
 
-def check_against(specs, index):
-    """Raise one WeightError naming every missing, unexpected and mis-shaped tensor."""
+def check_against(specs, index, ignored=()):
+    """Raise one WeightError naming every missing, unexpected and mis-shaped tensor.
+    `ignored` names tensors a checkpoint may carry without the model using them."""
     expected = {s.name: s for s in specs}
     missing = sorted(n for n in expected if n not in index)
-    unexpected = sorted(n for n in index if n not in expected)
+    unexpected = sorted(n for n in index if n not in expected and n not in ignored)
     wrong = []
     for name, spec in expected.items():
         if name in index:
@@ -83,10 +84,10 @@ def _kept_dtype(stored, integer, dtype):
     return torch.float32  # stored in 32 bits (or float16/float64): kept in 32 bits
 
 
-def load_folder(folder, specs, dtype, device):
+def load_folder(folder, specs, dtype, device, ignored=()):
     """{name: tensor on `device`} for every spec, after the whole-set check."""
     index = open_folder(folder)
-    check_against(specs, index)
+    check_against(specs, index, ignored)
     out = {}
     for spec in specs:
         t = index[spec.name].tensor(spec.name)

@@ -125,16 +125,19 @@ def test_loader_lists_everything_wrong_in_one_error(tmp_path):
     del tensors["model.layers.1.mlp.up_proj.weight"]
     del tensors["model.norm.weight"]
     tensors["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.zeros(8)
-    tensors["lm_head.weight"] = torch.zeros(c["vocab_size"], c["hidden_size"])  # tied model: not expected
+    tensors["lm_head.weight"] = torch.zeros(c["vocab_size"], c["hidden_size"])  # tied model: its copy of the head is ignored
     tensors["model.layers.0.self_attn.k_proj.weight"] = torch.zeros(64, 64)
     save_file(tensors, str(folder / "model.safetensors"))
     _, _, model = build_from_config_dict(raw("a"))
     with pytest.raises(WeightError) as info:
-        check_against(model.tensor_specs(), open_folder(folder))
+        check_against(model.tensor_specs(), open_folder(folder), model.ignored_tensors())
     text = str(info.value)
-    for needle in ("missing (2)", "model.layers.1.mlp.up_proj.weight", "model.norm.weight", "unexpected (2)",
-                   "rotary_emb.inv_freq", "lm_head.weight", "wrong shape (1)", "k_proj.weight: file has [64, 64], model expects [32, 64]"):
+    for needle in ("missing (2)", "model.layers.1.mlp.up_proj.weight", "model.norm.weight", "unexpected (1)",
+                   "rotary_emb.inv_freq", "wrong shape (1)", "k_proj.weight: file has [64, 64], model expects [32, 64]"):
         assert needle in text, needle
+    assert "lm_head.weight" not in text
+    _, _, untied = build_from_config_dict(raw("b"))
+    assert untied.ignored_tensors() == ()
 
 
 def test_loader_duplicate_across_shards_and_empty_folder(tmp_path):

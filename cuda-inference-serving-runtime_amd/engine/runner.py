@@ -43,6 +43,8 @@ class ModelRunner:
         self.model = model
         self.execution = execution
         self.programs, self.program_capacity = {}, 16
+        self.block_tiles = False   # attention of long portions through LDS-shared tiles (measured slower so far)
+        self.tile_waves = 4        # wavefronts that share one 16-item tile's keys
         self.device = torch.device(device)
         self.page_size = page_size
         self.max_requests = max_requests
@@ -283,9 +285,13 @@ class ModelRunner:
                 ops.attention_mfma(q, q_row_stride, kcache, vcache, view.tables, ctx.seg_of_row, ctx.positions, out,
                                    heads, kv_heads, head_dim, view.page_size, window, scale, None, splits, workspace, waves)
             else:
-                tasks = ctx.attention_tasks(16 // heads_per_chunk)
+                # long portions: one block per 64/GC rows with keys and values shared through LDS;
+                # batches of short portions and single tokens: four independent 16/GC-row tiles a block
+                block_tiles = self.block_tiles and rows >= 16 * ctx.n_segments
+                tasks = ctx.attention_tasks((64 if block_tiles else 16) // heads_per_chunk)
                 ops.attention_mfma(q, q_row_stride, kcache, vcache, view.tables, ctx.seg_of_row, ctx.positions, out,
-                                   heads, kv_heads, head_dim, view.page_size, window, scale, tasks)
+                                   heads, kv_heads, head_dim, view.page_size, window, scale, tasks, waves=self.tile_waves,
+                                   block_tiles=block_tiles)
             return
         splits = self._splits(rows * heads, span)
         workspace = None
@@ -310,7 +316,7 @@ class ModelRunner:
         and the context is long, the keys are also split over blocks (a merge kernel follows).
         Many rows: four waves a block, one block a row and head group."""
         steps = -(-span // 32)
-        waves = 8 if blocks < 512 and head_dim <= 128 else 4
+        waves = 8 if blocks < 512 and head_dim <= 64 else 4
         # as many blocks along the keys as keep about a thousand blocks in flight (the loads of a
         # whole layer's cache are then outstanding at once), each wave with at least one 32-key step
         splits = int(max(1, min(steps // waves, -(-1024 // blocks), 64)))

@@ -275,9 +275,9 @@ def run_mfma(ops, qt, kt, vt, tables, rows, page_size, mode, splits=1, window=No
     out = torch.full((T, heads * dim), 9.0, dtype=qt.dtype, device=DEV)
     tasks = None
     ws = (torch.empty(T * heads * splits * dim, device=DEV), torch.empty(T * heads * splits * 2, device=DEV))
-    if mode == "tiles":
+    if mode in ("tiles", "block"):
         group = heads // kv_heads
-        rpt = rows_per_tile or 16 // min(group, 16)
+        rpt = rows_per_tile or (64 if mode == "block" else 16) // min(group, 16)
         items, i = [], 0
         while i < T:   # consecutive rows of one segment with consecutive positions form a tile
             n = 1
@@ -286,7 +286,8 @@ def run_mfma(ops, qt, kt, vt, tables, rows, page_size, mode, splits=1, window=No
             items.append((rows[i][0], i, n, 0)); i += n
         tasks = torch.tensor(items, dtype=torch.int32, device=DEV)
     ops.attention_mfma(qt.reshape(T, heads * dim), heads * dim, kt, vt, tables, seg, pos, out, heads, kv_heads, dim,
-                       page_size, window, scale if scale is not None else 1 / math.sqrt(dim), tasks, splits, ws, waves)
+                       page_size, window, scale if scale is not None else 1 / math.sqrt(dim), tasks, splits, ws, waves,
+                       block_tiles=(mode == "block"))
     return f64(out).reshape(T, heads, dim)
 
 
@@ -331,7 +332,13 @@ def test_attention_mfma_tiles(ops, heads, kv_heads, dim, page_size):
     want = reference_attention(qt, kt, vt, tables, rows, page_size)
     got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, "tiles")
     np.testing.assert_allclose(got, want, **MFMA_TOL)
+    got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, "tiles", waves=8)
+    np.testing.assert_allclose(got, want, **MFMA_TOL)
     got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, "tiles", rows_per_tile=1)   # tiles need not be full
+    np.testing.assert_allclose(got, want, **MFMA_TOL)
+    got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, "block")                    # 64-item tiles through LDS
+    np.testing.assert_allclose(got, want, **MFMA_TOL)
+    got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, "block", rows_per_tile=3)
     np.testing.assert_allclose(got, want, **MFMA_TOL)
 
 
@@ -340,6 +347,7 @@ def test_attention_mfma_window_and_far_key(ops):
     for window in (1, 8, 9, 33, 64):
         want = reference_attention(qt, kt, vt, tables, rows, 8, window=window)
         np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables, rows, 8, "tiles", window=window), want, **MFMA_TOL)
+        np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables, rows, 8, "block", window=window), want, **MFMA_TOL)
         np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables, rows, 8, "rows", 2, window=window), want, **MFMA_TOL)
     want = reference_attention(qt, kt, vt, tables, rows, 8, scale=0.3)
     np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables, rows, 8, "tiles", scale=0.3), want, **MFMA_TOL)
@@ -347,11 +355,12 @@ def test_attention_mfma_window_and_far_key(ops):
     tables2 = tables.clone(); tables2[0, :4] = -1          # keys 0..31 of request 0; window 8 from position 40 starts at 33
     want = reference_attention(qt, kt, vt, tables, rows, 8, window=8)
     np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables2, rows, 8, "tiles", window=8), want, **MFMA_TOL)
+    np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables2, rows, 8, "block", window=8), want, **MFMA_TOL)
     np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables2, rows, 8, "rows", 3, window=8), want, **MFMA_TOL)
     # one far key among hundreds stands out
     qt, kt, vt, tables, rows = paged_case(4, 2, 64, 16, [700, 40], torch.bfloat16, seed=5, sharpen=(0, 3))
     want = reference_attention(qt, kt, vt, tables, rows, 16)
-    for mode, splits in (("rows", 1), ("rows", 8), ("tiles", 1)):
+    for mode, splits in (("rows", 1), ("rows", 8), ("tiles", 1), ("block", 1)):
         np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables, rows, 16, mode, splits), want, **MFMA_TOL)
 
 

@@ -84,12 +84,23 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 
 // 16 bytes = 8 bf16 from row-major global memory, zero-filled outside the matrix.
-// `vec` says rows are 16-byte aligned (ld % 8 == 0 and base aligned).
-__device__ __forceinline__ u32x4 load_chunk(const bf16_t* base, int ld, int row, int nrows, int k, int K, bool vec) {
+// VEC: rows are 16-byte aligned and K % 8 == 0, so a chunk lies wholly inside or outside; the load
+// is unconditional from a clamped address (no branch between the loads of a tile, so they are all
+// in flight together) and the result is zeroed by a select.  Otherwise element by element.
+template <bool VEC>
+__device__ __forceinline__ u32x4 load_chunk(const bf16_t* base, int ld, int row, int nrows, int k, int K) {
+    if (VEC) {
+        // no branch and nothing that touches the loaded value (it would wait for the load): rows
+        // past the end read the last row (their products land in output rows or columns that are
+        // never stored); a chunk past K reads the last chunk and is zeroed by a mask when the tile
+        // is written to LDS, so that nothing is added to valid outputs
+        const int rr = row < nrows ? row : nrows - 1;
+        const int kk = k < K ? k : K - 8;
+        return *(const u32x4*)(base + (size_t)rr * ld + kk);   // the caller masks chunks past K when it uses them
+    }
     u32x4 v = {0u, 0u, 0u, 0u};
     if (row >= nrows || k >= K) return v;
     const bf16_t* p = base + (size_t)row * ld + k;
-    if (vec && k + 8 <= K) return *(const u32x4*)p;
     uint32_t w[4] = {0u, 0u, 0u, 0u};
 #pragma unroll
     for (int e = 0; e < 8; ++e)
@@ -99,20 +110,25 @@ __device__ __forceinline__ u32x4 load_chunk(const bf16_t* base, int ld, int row,
 }
 
 // Block tile (32 TM) x (32 TN), BK deep; four waves as 2 x 2, each wave TM x TN tiles of 16 x 16.
-// Operands are staged through LDS (rows padded by 8 elements, so rows stay 16-byte aligned and the
-// 16-byte operand reads of a wave spread over the banks); the next tile's global loads are in
-// flight while the current one is multiplied.
-template <int TM, int TN, int BK, typename TC>
+// Operands go global memory -> registers -> LDS -> matrix-core operands.  Rows in LDS are padded by 8
+// elements (rows stay 16-byte aligned, a wave's 16-byte operand reads spread over the banks).
+// The pipeline hides the global-memory latency inside one block, because small problems leave a
+// compute unit with a single block: PF tiles of global loads are in flight in a ring of registers,
+// and two LDS buffers let the next tile be written while the current one is multiplied, with one
+// barrier per tile.
+template <int TM, int TN, int BK, typename TC, bool VEC>
 __global__ void __launch_bounds__(256)
 gemm_bf16_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, int ldw,
-                 TC* C, int ldc, const float* R, int ldr, int M, int N, int K, int vecA, int vecW) {
+                 TC* C, int ldc, const float* R, int ldr, int M, int N, int K) {
     constexpr int BM = 2 * TM * 16, BN = 2 * TN * 16;
     constexpr int STRIDE = BK + 8;
     constexpr int CPR = BK / 8;                            // 16-byte chunks per tile row
-    constexpr int A_PER_THREAD = (BM * CPR + 255) / 256;
-    constexpr int W_PER_THREAD = (BN * CPR + 255) / 256;
-    __shared__ __attribute__((aligned(16))) bf16_t As[BM * STRIDE];
-    __shared__ __attribute__((aligned(16))) bf16_t Ws[BN * STRIDE];
+    static_assert((BM * CPR) % 256 == 0 && (BN * CPR) % 256 == 0, "a tile is a whole number of 16-byte chunks per thread");
+    constexpr int A_PER_THREAD = BM * CPR / 256;
+    constexpr int W_PER_THREAD = BN * CPR / 256;
+    constexpr int PF = 3;                                  // tiles of global loads in flight
+    __shared__ __attribute__((aligned(16))) bf16_t As[2][BM * STRIDE];
+    __shared__ __attribute__((aligned(16))) bf16_t Ws[2][BN * STRIDE];
 
     const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
     const int wm = wave / 2, wn = wave % 2;
@@ -125,51 +141,83 @@ gemm_bf16_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict
 #pragma unroll
         for (int j = 0; j < TN; ++j) acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
-    u32x4 ra[A_PER_THREAD], rw[W_PER_THREAD];
-    auto fetch = [&](int k0) {
+    u32x4 ra[PF][A_PER_THREAD], rw[PF][W_PER_THREAD];
+    auto fetch = [&](int k0, u32x4 (&fa)[A_PER_THREAD], u32x4 (&fw)[W_PER_THREAD]) {
 #pragma unroll
         for (int i = 0; i < A_PER_THREAD; ++i) {
             const int c = tid + i * 256;
-            if (c < BM * CPR) ra[i] = load_chunk(A, lda, m0 + c / CPR, M, k0 + (c % CPR) * 8, K, vecA);
+            fa[i] = load_chunk<VEC>(A, lda, m0 + c / CPR, M, k0 + (c % CPR) * 8, K);
         }
 #pragma unroll
         for (int i = 0; i < W_PER_THREAD; ++i) {
             const int c = tid + i * 256;
-            if (c < BN * CPR) rw[i] = load_chunk(W, ldw, n0 + c / CPR, N, k0 + (c % CPR) * 8, K, vecW);
+            fw[i] = load_chunk<VEC>(W, ldw, n0 + c / CPR, N, k0 + (c % CPR) * 8, K);
         }
     };
-    fetch(0);
-    for (int k0 = 0; k0 < K; k0 += BK) {
 #pragma unroll
-        for (int i = 0; i < A_PER_THREAD; ++i) {
-            const int c = tid + i * 256;
-            if (c < BM * CPR) *(u32x4*)(As + (c / CPR) * STRIDE + (c % CPR) * 8) = ra[i];
+    for (int s = 0; s < PF; ++s) fetch(s * BK, ra[s], rw[s]);   // beyond K: zeros, never used
+
+    int it = 0;
+    for (int k0 = 0; k0 < K; k0 += PF * BK) {
+#pragma unroll
+        for (int s = 0; s < PF; ++s) {
+            const int kk0 = k0 + s * BK;
+            if (kk0 < K) {
+                const int buf = it & 1;
+                ++it;
+#pragma unroll
+                for (int i = 0; i < A_PER_THREAD; ++i) {
+                    const int c = tid + i * 256;
+                    const uint32_t keep = (VEC && kk0 + (c % CPR) * 8 >= K) ? 0u : 0xffffffffu;
+                    u32x4 v = ra[s][i];
+                    v.x &= keep; v.y &= keep; v.z &= keep; v.w &= keep;
+                    *(u32x4*)(&As[buf][(c / CPR) * STRIDE + (c % CPR) * 8]) = v;
+                }
+#pragma unroll
+                for (int i = 0; i < W_PER_THREAD; ++i) {
+                    const int c = tid + i * 256;
+                    *(u32x4*)(&Ws[buf][(c / CPR) * STRIDE + (c % CPR) * 8]) = rw[s][i];   // A is zero there: enough
+                }
+                // one barrier a tile: whoever writes this buffer again (two tiles on) has passed
+                // the next tile's barrier, which every wave reaches only after reading this one
+                __syncthreads();
+                if (kk0 + PF * BK < K) fetch(kk0 + PF * BK, ra[s], rw[s]);
+#pragma unroll
+                for (int kk = 0; kk < BK; kk += 32) {
+                    bf16x8 fa[TM], fw[TN];
+#pragma unroll
+                    for (int i = 0; i < TM; ++i)
+                        fa[i] = *(const bf16x8*)(&As[buf][(wm * TM * 16 + i * 16 + r) * STRIDE + kk + g * 8]);
+#pragma unroll
+                    for (int j = 0; j < TN; ++j)
+                        fw[j] = *(const bf16x8*)(&Ws[buf][(wn * TN * 16 + j * 16 + r) * STRIDE + kk + g * 8]);
+#pragma unroll
+                    for (int i = 0; i < TM; ++i)
+#pragma unroll
+                        for (int j = 0; j < TN; ++j)
+                            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[i], fw[j], acc[i][j], 0, 0, 0);
+                }
+            }
         }
-#pragma unroll
-        for (int i = 0; i < W_PER_THREAD; ++i) {
-            const int c = tid + i * 256;
-            if (c < BN * CPR) *(u32x4*)(Ws + (c / CPR) * STRIDE + (c % CPR) * 8) = rw[i];
-        }
-        __syncthreads();
-        if (k0 + BK < K) fetch(k0 + BK);
-#pragma unroll
-        for (int kk = 0; kk < BK; kk += 32) {
-            bf16x8 fa[TM], fw[TN];
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-                fa[i] = *(const bf16x8*)(As + (wm * TM * 16 + i * 16 + r) * STRIDE + kk + g * 8);
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-                fw[j] = *(const bf16x8*)(Ws + (wn * TN * 16 + j * 16 + r) * STRIDE + kk + g * 8);
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int j = 0; j < TN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[i], fw[j], acc[i][j], 0, 0, 0);
-        }
-        __syncthreads();
     }
-    // lane holds rows 4g..4g+3 of column r in every 16 x 16 tile
+    // lane holds rows 4g..4g+3 of column r in every 16 x 16 tile.  The residual is read with
+    // unconditional loads from clamped addresses, all issued before the first is used.
+    if (R) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                const int n = min(n0 + wn * TN * 16 + j * 16 + r, N - 1);
+                float rv[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int m = min(m0 + wm * TM * 16 + i * 16 + g * 4 + e, M - 1);
+                    rv[e] = R[(size_t)m * ldr + n];
+                }
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc[i][j][e] += rv[e];
+            }
+    }
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
 #pragma unroll
@@ -179,10 +227,7 @@ gemm_bf16_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const int m = m0 + wm * TM * 16 + i * 16 + g * 4 + e;
-                if (m >= M) continue;
-                float v = acc[i][j][e];
-                if (R) v += R[(size_t)m * ldr + n];
-                store_f32(C + (size_t)m * ldc + n, v);
+                if (m < M) store_f32(C + (size_t)m * ldc + n, acc[i][j][e]);
             }
         }
     }
@@ -194,12 +239,14 @@ static int launch_bf16(const bf16_t* A, int lda, const bf16_t* W, int ldw, void*
     constexpr int BM = 2 * TM * 16, BN = 2 * TN * 16;
     dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM);
     if (grid.y > 65535) return (int)hipErrorInvalidValue;
-    const int vecA = (lda % 8 == 0) && (((uintptr_t)A) % 16 == 0);
-    const int vecW = (ldw % 8 == 0) && (((uintptr_t)W) % 16 == 0);
-    if (out_dtype == DT_F32)
-        gemm_bf16_kernel<TM, TN, BK, float><<<grid, 256, 0, stream>>>(A, lda, W, ldw, (float*)C, ldc, R, ldr, M, N, K, vecA, vecW);
-    else
-        gemm_bf16_kernel<TM, TN, BK, bf16_t><<<grid, 256, 0, stream>>>(A, lda, W, ldw, (bf16_t*)C, ldc, R, ldr, M, N, K, vecA, vecW);
+    const bool vec = lda % 8 == 0 && ldw % 8 == 0 && K % 8 == 0 && ((uintptr_t)A) % 16 == 0 && ((uintptr_t)W) % 16 == 0;
+    if (out_dtype == DT_F32) {
+        if (vec) gemm_bf16_kernel<TM, TN, BK, float, true><<<grid, 256, 0, stream>>>(A, lda, W, ldw, (float*)C, ldc, R, ldr, M, N, K);
+        else gemm_bf16_kernel<TM, TN, BK, float, false><<<grid, 256, 0, stream>>>(A, lda, W, ldw, (float*)C, ldc, R, ldr, M, N, K);
+    } else {
+        if (vec) gemm_bf16_kernel<TM, TN, BK, bf16_t, true><<<grid, 256, 0, stream>>>(A, lda, W, ldw, (bf16_t*)C, ldc, R, ldr, M, N, K);
+        else gemm_bf16_kernel<TM, TN, BK, bf16_t, false><<<grid, 256, 0, stream>>>(A, lda, W, ldw, (bf16_t*)C, ldc, R, ldr, M, N, K);
+    }
     return CISR_LAUNCH_CHECK();
 }
 

@@ -1,0 +1,28 @@
+// Arguments of the skinny (M <= 64) bf16 matrix-product kernels and the entry points that the
+// per-row-count translation units export (one unit per number of 16-row tiles, so that they
+// compile in parallel).
+#pragma once
+#include "common.h"
+
+enum { EPI_STORE = 0, EPI_SWIGLU = 1, EPI_ROPE = 2 };
+
+struct SkinnyArgs {
+    const void* A; int lda;            // bf16 activations, or float residual with NORM
+    const bf16_t* W; int ldw;
+    void* C; int ldc;                  // EPI_ROPE: q output, bf16 [M, heads*D]
+    const float* R; int ldr;           // residual (EPI_STORE, float C only)
+    int M, N, K;
+    int dual_off;                      // EPI_SWIGLU
+    // NORM
+    const float* norm_w; float eps; const int* rows;
+    // EPI_ROPE
+    const int* positions; const int* slots; const float* cos_tab; const float* sin_tab;
+    bf16_t* kcache; bf16_t* vcache; int heads, kv_heads, head_dim, page_size, max_pos;
+};
+
+
+// one function per MT = number of 16-row tiles of A (M <= 16 MT)
+int cisr_skinny_launch_m1(const SkinnyArgs& a, int blocks, bool norm, int epi, int out_dtype, hipStream_t stream);
+int cisr_skinny_launch_m2(const SkinnyArgs& a, int blocks, bool norm, int epi, int out_dtype, hipStream_t stream);
+int cisr_skinny_launch_m3(const SkinnyArgs& a, int blocks, bool norm, int epi, int out_dtype, hipStream_t stream);
+int cisr_skinny_launch_m4(const SkinnyArgs& a, int blocks, bool norm, int epi, int out_dtype, hipStream_t stream);

@@ -316,8 +316,11 @@ class ModelRunner:
         and the context is long, the keys are also split over blocks (a merge kernel follows).
         Many rows: four waves a block, one block a row and head group."""
         steps = -(-span // 32)
-        waves = 8 if blocks < 512 and head_dim <= 64 else 4
-        # as many blocks along the keys as keep about a thousand blocks in flight (the loads of a
-        # whole layer's cache are then outstanding at once), each wave with at least one 32-key step
-        splits = int(max(1, min(steps // waves, -(-1024 // blocks), 64)))
+        few = blocks < 128
+        waves = 8 if few and head_dim <= 64 else 4
+        # few rows: enough blocks along the keys to keep about a thousand blocks in flight (the loads
+        # of a whole layer's cache are then outstanding at once); many rows fill the GPU by themselves
+        # and split only a little.  A wave keeps at least two 32-key steps (one computing, one loading).
+        target = 1024 if few else 256
+        splits = int(max(1, min(steps // (waves * 2), -(-target // blocks), 64)))
         return waves, splits

@@ -125,7 +125,7 @@ def main():
     peak = PEAK_TFLOPS["bf16" if args.dtype == "bfloat16" else "fp32"] * 1e12
     points = {f"decode_b{b}": round(b * steps / results[b][0], 1) for b in batches if b != args.batch}
     line = {
-        "metric": "decode tokens/s, SmolLM2-135M layer sizes, batch 8, 2048-token prompts in a 4096 context",
+        "metric": f"decode tokens/s, {args.model} layer sizes, batch {args.batch}, {args.prompt}-token prompts in a {args.context} context",
         "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic (random weights N(0,0.02), uniform-random token ids)",

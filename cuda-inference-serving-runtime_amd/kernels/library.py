@@ -115,6 +115,12 @@ def build(force=False):
         if proc.returncode != 0:
             raise KernelLibraryError(f"link failed:\n{proc.stdout}\n{proc.stderr}")
         os.replace(tmp, target)  # atomic: a concurrent loader sees the whole file or none
+        for old in target.parent.glob("libcisr_kernels_*.so"):   # builds of other source states
+            if old != target:
+                try:
+                    old.unlink()
+                except OSError:
+                    pass
     finally:
         shutil.rmtree(work, ignore_errors=True)
     return target

@@ -284,6 +284,12 @@ def fused_norm_ok(x, w, rows_out):
             and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w.stride(0) % 8 == 0 and w.data_ptr() % 16 == 0)
 
 
+def swiglu_fused_ok(a, w_gate_up):
+    """Whether gemm_swiglu runs as one kernel for these operands (no scratch buffer needed)."""
+    return (a.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16 and a.shape[0] <= SKINNY_ROWS
+            and _skinny_ok(a, w_gate_up))
+
+
 def gemm_normed(x, norm, w, out):
     """out[R, N] = RMSNorm(x[rows]) . w^T with the norm applied inside the product's kernel.
     x float [T, K]; norm = (weight float [K], eps, rows int32 [R] or None); w bf16 [N, K]; out float or bf16."""
@@ -316,7 +322,7 @@ def gemm_swiglu(a, w_gate_up, out, scratch=None, norm=None):
         return out
     if out.dtype != a.dtype or a.dtype != w_gate_up.dtype:
         raise KernelError("gemm_swiglu: dtypes differ")
-    if a.dtype == torch.bfloat16 and m <= SKINNY_ROWS and _skinny_ok(a, w_gate_up) and a.is_cuda:
+    if swiglu_fused_ok(a, w_gate_up) and a.is_cuda:
         _check(lib().cisr_gemm_skinny_bf16(a.data_ptr(), a.stride(0), w_gate_up.data_ptr(), w_gate_up.stride(0),
                                            out.data_ptr(), out.stride(0), None, 0, m, inter, k, BF16, inter, None, 0.0,
                                            None, _stream()), "gemm_swiglu")

@@ -34,8 +34,8 @@ class GatedMLP(FeedForward):
         act = ctx.buffer("ffn.act", (T, self.intermediate), ctx.dtype)
         if norm is not None:
             ops.gemm_swiglu(residual, self.w_gate_up, act, norm=(norm.weight, norm.eps, None))
-        elif ctx.dtype == torch.bfloat16 and T <= ops.SKINNY_ROWS:
-            ops.gemm_swiglu(h, self.w_gate_up, act)   # fused when the fast kernel takes the shape
+        elif ops.swiglu_fused_ok(h, self.w_gate_up):
+            ops.gemm_swiglu(h, self.w_gate_up, act)   # one kernel: product and activation
         else:
             ops.gemm_swiglu(h, self.w_gate_up, act, scratch=ctx.buffer("ffn.gate_up", (T, 2 * self.intermediate), ctx.dtype))
         return ops.gemm(act, self.w_down, residual, residual=residual)

@@ -19,7 +19,7 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs an MI355X (run with -m gpu)")
 
 
-# Three tiny configurations that differ in every size and option: head counts and
+# Four tiny configurations that differ in every size and option: head counts and
 # grouping, head size (16 / 24 / 64, the last not hidden/heads), widths and
 # vocabularies that are no power of two, number of layers, eps, theta, tied head.
 TINY = {
@@ -32,8 +32,12 @@ TINY = {
     "c": dict(num_hidden_layers=2, hidden_size=200, num_attention_heads=6, num_key_value_heads=2, head_dim=64,
               intermediate_size=264, vocab_size=1003, rope_theta=100000.0, rms_norm_eps=1e-5,
               tie_word_embeddings=False, max_position_embeddings=640),
+    # sizes that fit none of the fast paths: width and head size that are no multiples of 8
+    "d": dict(num_hidden_layers=2, hidden_size=100, num_attention_heads=5, num_key_value_heads=1, head_dim=20,
+              intermediate_size=90, vocab_size=257, rope_theta=20000.0, rms_norm_eps=1e-4,
+              tie_word_embeddings=True, max_position_embeddings=384),
 }
-SEEDS = {"a": 0, "b": 1, "c": 2}
+SEEDS = {"a": 0, "b": 1, "c": 2, "d": 3}
 
 
 def tensor_shapes(c):

@@ -28,7 +28,7 @@ def run(folder, dtype, trace, out_dir, max_tokens=None, page_size=None):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", ["a", "b", "c"])
+@pytest.mark.parametrize("name", ["a", "b", "c", "d"])
 def test_whole_requests_alone(folders, tmp_path, name, dtype):
     V = TINY[name]["vocab_size"]
     seqs = {f"r{i}": random_tokens(10 * i + 1, n, V) for i, n in enumerate([1, 5, 64, 65, 150])}
@@ -41,7 +41,7 @@ def test_whole_requests_alone(folders, tmp_path, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", ["a", "b", "c"])
+@pytest.mark.parametrize("name", ["a", "b", "c", "d"])
 def test_prefix_then_last_32_one_by_one(folders, tmp_path, name, dtype):
     V = TINY[name]["vocab_size"]
     toks = random_tokens(77, 131, V)
@@ -54,7 +54,7 @@ def test_prefix_then_last_32_one_by_one(folders, tmp_path, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", ["a", "b", "c"])
+@pytest.mark.parametrize("name", ["a", "b", "c", "d"])
 def test_portions_of_changing_size(folders, tmp_path, name, dtype):
     V = TINY[name]["vocab_size"]
     toks = random_tokens(5, 140, V)
@@ -110,7 +110,7 @@ def mixed_trace(V, seed):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", ["a", "b", "c"])
+@pytest.mark.parametrize("name", ["a", "b", "c", "d"])
 def test_mixed_requests_reuse_pages(folders, tmp_path, name, dtype):
     V = TINY[name]["vocab_size"]
     trace, seqs = mixed_trace(V, seed=3)

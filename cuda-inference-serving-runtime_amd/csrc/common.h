@@ -16,12 +16,18 @@ __device__ __forceinline__ float bf16_to_f32(bf16_t v) {
     return __uint_as_float(((uint32_t)v) << 16);
 }
 
-// round to nearest even; NaN stays a quiet NaN with its sign
-// (same rule as the reference's kernels/precision.cuh:13-20)
+// round to nearest even, NaN stays NaN (the rule of the reference's kernels/precision.cuh:13-20),
+// done by the hardware conversion of gfx950 (v_cvt_pk_bf16_f32)
 __device__ __forceinline__ bf16_t f32_to_bf16(float f) {
-    uint32_t bits = __float_as_uint(f);
-    if ((bits & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((bits >> 16) | 0x40u);
-    return (bf16_t)((bits + 0x7fffu + ((bits >> 16) & 1u)) >> 16);
+    return __builtin_bit_cast(bf16_t, (__bf16)f);
+}
+
+// two floats to a pair of bf16 in one register (low half first)
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
+    typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+    typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+    const f32x2_t v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
 
 __device__ __forceinline__ float load_f32(const float* p) { return *p; }

@@ -12,6 +12,7 @@ context limit, token range, page preflight, then execution
 (runtime/model.py:93-102).
 """
 import gc
+import os
 from dataclasses import dataclass, field
 from typing import List, Sequence
 
@@ -44,7 +45,8 @@ class ModelRunner:
         self.execution = execution
         self.programs, self.program_capacity = {}, 16
         self.block_tiles = False   # attention of long portions through LDS-shared tiles (measured slower so far)
-        self.tile_waves = 4        # wavefronts that share one 16-item tile's keys
+        self.tile_waves = int(os.environ.get("CISR_TILE_WAVES", "4"))   # wavefronts that share one tile's keys
+        self.item_tiles = int(os.environ.get("CISR_ITEM_TILES", "1"))   # 16-item tiles a wave (2: measured slower)
         self.device = torch.device(device)
         self.page_size = page_size
         self.max_requests = max_requests
@@ -285,13 +287,16 @@ class ModelRunner:
                 ops.attention_mfma(q, q_row_stride, kcache, vcache, view.tables, ctx.seg_of_row, ctx.positions, out,
                                    heads, kv_heads, head_dim, view.page_size, window, scale, None, splits, workspace, waves)
             else:
-                # long portions: one block per 64/GC rows with keys and values shared through LDS;
-                # batches of short portions and single tokens: four independent 16/GC-row tiles a block
-                block_tiles = self.block_tiles and rows >= 16 * ctx.n_segments
-                tasks = ctx.attention_tasks((64 if block_tiles else 16) // heads_per_chunk)
+                # long portions with small heads: 32/GC rows a block, every wave owns two 16-item tiles
+                # (keys and values are loaded once for both); otherwise 16/GC rows a block.  The
+                # LDS-shared 64/GC-row variant exists but measured slower and is off.
+                long_portions = rows >= 16 * ctx.n_segments
+                block_tiles = self.block_tiles and long_portions
+                item_tiles = 2 if self.item_tiles == 2 and long_portions and head_dim <= 64 and not block_tiles else 1
+                tasks = ctx.attention_tasks((64 if block_tiles else 16 * item_tiles) // heads_per_chunk)
                 ops.attention_mfma(q, q_row_stride, kcache, vcache, view.tables, ctx.seg_of_row, ctx.positions, out,
                                    heads, kv_heads, head_dim, view.page_size, window, scale, tasks, waves=self.tile_waves,
-                                   block_tiles=block_tiles)
+                                   block_tiles=block_tiles, item_tiles=item_tiles)
             return
         splits = self._splits(rows * heads, span)
         workspace = None

@@ -371,10 +371,12 @@ def qkv_rope(a, w, q_out, positions, slots, cos, sin, kcache, vcache, heads, kv_
 
 
 def attention_mfma(q, q_row_stride, kcache, vcache, tables, seg_of_row, positions, out, heads, kv_heads, dim,
-                   page_size, window, scale, tasks=None, splits=1, workspace=None, waves=4, block_tiles=False):
+                   page_size, window, scale, tasks=None, splits=1, workspace=None, waves=4, block_tiles=False,
+                   item_tiles=1):
     """Matrix-core attention (bf16).  tasks int32 [n, 4] = (segment, first row, rows, 0) runs tiles of
-    prompt rows, four tiles of 16/GC rows a block, or with `block_tiles` one tile of 64/GC rows a block with
-    keys and values shared through LDS (GC = query heads per key head, at most 16); tasks None runs one block
+    prompt rows: one tile of 16/GC rows a block whose waves share the keys (with item_tiles=2, head sizes up to
+    64: 32/GC rows, two item tiles a wave), or with `block_tiles` one tile of 64/GC rows a block with keys and
+    values shared through LDS (GC = query heads per key head, at most 16); tasks None runs one block
     per row (decode) of `waves` wavefronts (4 or 8) with `splits` blocks along the keys; splits > 1 needs
     workspace = (partials float, statistics float) and a merge."""
     rows = out.shape[0]
@@ -391,7 +393,9 @@ def attention_mfma(q, q_row_stride, kcache, vcache, tables, seg_of_row, position
     fn = getattr(lib(), f"cisr_attn_mfma_d{dpad}")
     po = pm = tp = None
     if tasks is not None:
-        n_tasks, mode, splits = tasks.shape[0], (2 if block_tiles else 0), 1
+        if item_tiles not in (1, 2) or (item_tiles == 2 and (dim > 64 or block_tiles)):
+            raise KernelError("attention_mfma: two item tiles a wave need a head size of at most 64")
+        n_tasks, mode, splits = tasks.shape[0], (2 if block_tiles else 3 if item_tiles == 2 else 0), 1
         tp = _dev(tasks, "tasks", torch.int32, (n_tasks, 4))
     else:
         n_tasks, mode = rows, 1

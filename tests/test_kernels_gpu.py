@@ -275,9 +275,9 @@ def run_mfma(ops, qt, kt, vt, tables, rows, page_size, mode, splits=1, window=No
     out = torch.full((T, heads * dim), 9.0, dtype=qt.dtype, device=DEV)
     tasks = None
     ws = (torch.empty(T * heads * splits * dim, device=DEV), torch.empty(T * heads * splits * 2, device=DEV))
-    if mode in ("tiles", "block"):
+    if mode in ("tiles", "tiles2", "block"):
         group = heads // kv_heads
-        rpt = rows_per_tile or (64 if mode == "block" else 16) // min(group, 16)
+        rpt = rows_per_tile or {"tiles": 16, "tiles2": 32, "block": 64}[mode] // min(group, 16)
         items, i = [], 0
         while i < T:   # consecutive rows of one segment with consecutive positions form a tile
             n = 1
@@ -287,7 +287,7 @@ def run_mfma(ops, qt, kt, vt, tables, rows, page_size, mode, splits=1, window=No
         tasks = torch.tensor(items, dtype=torch.int32, device=DEV)
     ops.attention_mfma(qt.reshape(T, heads * dim), heads * dim, kt, vt, tables, seg, pos, out, heads, kv_heads, dim,
                        page_size, window, scale if scale is not None else 1 / math.sqrt(dim), tasks, splits, ws, waves,
-                       block_tiles=(mode == "block"))
+                       block_tiles=(mode == "block"), item_tiles=(2 if mode == "tiles2" else 1))
     return f64(out).reshape(T, heads, dim)
 
 
@@ -336,6 +336,11 @@ def test_attention_mfma_tiles(ops, heads, kv_heads, dim, page_size):
     np.testing.assert_allclose(got, want, **MFMA_TOL)
     got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, "tiles", rows_per_tile=1)   # tiles need not be full
     np.testing.assert_allclose(got, want, **MFMA_TOL)
+    if dim <= 64:
+        got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, "tiles2")               # two item tiles a wave
+        np.testing.assert_allclose(got, want, **MFMA_TOL)
+        got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, "tiles2", rows_per_tile=2)
+        np.testing.assert_allclose(got, want, **MFMA_TOL)
     got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, "block")                    # 64-item tiles through LDS
     np.testing.assert_allclose(got, want, **MFMA_TOL)
     got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, "block", rows_per_tile=3)
@@ -348,6 +353,7 @@ def test_attention_mfma_window_and_far_key(ops):
         want = reference_attention(qt, kt, vt, tables, rows, 8, window=window)
         np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables, rows, 8, "tiles", window=window), want, **MFMA_TOL)
         np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables, rows, 8, "block", window=window), want, **MFMA_TOL)
+        np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables, rows, 8, "tiles2", window=window), want, **MFMA_TOL)
         np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables, rows, 8, "rows", 2, window=window), want, **MFMA_TOL)
     want = reference_attention(qt, kt, vt, tables, rows, 8, scale=0.3)
     np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables, rows, 8, "tiles", scale=0.3), want, **MFMA_TOL)

@@ -133,7 +133,14 @@ gemm_bf16_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict
     const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
     const int wm = wave / 2, wn = wave % 2;
     const int r = lane % 16, g = lane / 16;
-    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    // The hardware deals consecutive workgroups round-robin to the 8 XCDs, each with an L2 of its
+    // own.  Renumber so that an XCD gets a contiguous run of tiles (column tiles fastest): it then
+    // touches one band of A rows instead of all of A, and W stays in its L2 across the band.
+    const int tiles_n = (N + BN - 1) / BN, tiles = tiles_n * ((M + BM - 1) / BM);
+    const int per_xcd = (tiles + 7) / 8;
+    const int tile = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    if (tile >= tiles) return;   // the grid is rounded up to a multiple of 8
+    const int m0 = (tile / tiles_n) * BM, n0 = (tile % tiles_n) * BN;
 
     f32x4 acc[TM][TN];
 #pragma unroll
@@ -237,8 +244,9 @@ template <int TM, int TN, int BK>
 static int launch_bf16(const bf16_t* A, int lda, const bf16_t* W, int ldw, void* C, int ldc, const float* R,
                        int ldr, int M, int N, int K, int out_dtype, hipStream_t stream) {
     constexpr int BM = 2 * TM * 16, BN = 2 * TN * 16;
-    dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM);
-    if (grid.y > 65535) return (int)hipErrorInvalidValue;
+    const long long tiles = (long long)((N + BN - 1) / BN) * ((M + BM - 1) / BM);
+    if (tiles > (1ll << 30)) return (int)hipErrorInvalidValue;
+    dim3 grid((unsigned)((tiles + 7) / 8 * 8));
     const bool vec = lda % 8 == 0 && ldw % 8 == 0 && K % 8 == 0 && ((uintptr_t)A) % 16 == 0 && ((uintptr_t)W) % 16 == 0;
     if (out_dtype == DT_F32) {
         if (vec) gemm_bf16_kernel<TM, TN, BK, float, true><<<grid, 256, 0, stream>>>(A, lda, W, ldw, (float*)C, ldc, R, ldr, M, N, K);

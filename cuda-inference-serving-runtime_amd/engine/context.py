@@ -7,6 +7,7 @@ never look at request identities.
 """
 from dataclasses import dataclass
 
+import numpy as np
 import torch
 
 from ..kernels import ops
@@ -19,6 +20,22 @@ class GroupView:
     tables: torch.Tensor      # int32 [S, W]: block table of each segment's request
     page_size: int
     width: int
+
+
+def fill_tasks(tasks, counts, rows_per_tile):
+    """Write (segment, first row, rows, 0) for tiles of at most `rows_per_tile` consecutive
+    rows of one segment into the int32 array tasks[n, 4]; returns how many were written."""
+    n = row = 0
+    for seg, count in enumerate(counts):
+        tiles = -(-count // rows_per_tile)
+        firsts = np.arange(tiles, dtype=np.int64) * rows_per_tile
+        tasks[n:n + tiles, 0] = seg
+        tasks[n:n + tiles, 1] = row + firsts
+        tasks[n:n + tiles, 2] = np.minimum(rows_per_tile, count - firsts)
+        tasks[n:n + tiles, 3] = 0
+        n += tiles
+        row += count
+    return n
 
 
 class StepContext:
@@ -35,23 +52,28 @@ class StepContext:
         self.max_context = 0      # host: largest position + 1 among the rows
         self.decode_only = False  # host: every segment brings exactly one token
         self.span_hint = 0        # host: context length that sizes attention launches (a bucket under capture)
-        self._tasks = {}
+        self.tasks = {}           # rows per tile -> int32 [n, 4] task list on the device
+        self.capturing = False    # the step is being recorded into a graph: launches only
 
     def buffer(self, name, shape, dtype):
         return self.runner.workspace.get(name, shape, dtype)
 
     def attention_tasks(self, rows_per_tile):
         """int32 [n, 4] on the device: (segment, first row, rows, 0) for tiles of at most
-        `rows_per_tile` consecutive rows of one segment."""
-        tasks = self._tasks.get(rows_per_tile)
+        `rows_per_tile` consecutive rows of one segment; entries with segment -1 are no tile.
+        The step's metadata holds the list for every tiling asked for before; a new tiling
+        is built and uploaded here once and travels with the metadata from the next step on."""
+        tasks = self.tasks.get(rows_per_tile)
         if tasks is None:
-            items, row = [], 0
-            for seg, (_, _, count) in enumerate(self.segments):
-                for first in range(0, count, rows_per_tile):
-                    items.append((seg, row + first, min(rows_per_tile, count - first), 0))
-                row += count
-            tasks = torch.tensor(items, dtype=torch.int32).to(self.device, non_blocking=False)
-            self._tasks[rows_per_tile] = tasks
+            if self.capturing:
+                raise RuntimeError(f"a task list of {rows_per_tile} rows a tile was first asked for under graph capture")
+            counts = [count for _, _, count in self.segments]
+            host = np.full((sum(-(-c // rows_per_tile) for c in counts), 4), -1, dtype=np.int32)
+            fill_tasks(host, counts, rows_per_tile)
+            tasks = torch.from_numpy(host).to(self.device, non_blocking=False)
+            self.tasks[rows_per_tile] = tasks
+            if rows_per_tile not in self.runner.task_tilings:
+                self.runner.task_tilings.append(rows_per_tile)
         return tasks
 
     def attend(self, q, q_row_stride, kcache, vcache, view, out, heads, kv_heads, head_dim, window, scale):

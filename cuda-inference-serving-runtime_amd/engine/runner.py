@@ -21,7 +21,7 @@ import torch
 
 from ..cache import CacheManager, OutOfPages
 from ..kernels import ops
-from .context import GroupView, StepContext, Workspace
+from .context import GroupView, StepContext, Workspace, fill_tasks
 
 
 @dataclass
@@ -32,6 +32,13 @@ class StepEntry:
 
 
 _TORCH_OF = {"float32": torch.float32, "bfloat16": torch.bfloat16, "int32": torch.int32}
+
+
+def _bucket(n):
+    """Sizes that captured programs are padded to: powers of two up to 64, then multiples of 64."""
+    if n <= 0:
+        return 0
+    return 1 << (n - 1).bit_length() if n <= 64 else -(-n // 64) * 64
 
 
 class ModelRunner:
@@ -68,6 +75,7 @@ class ModelRunner:
         self.table_width = -(-self.max_context // page_size)
         self._staging = []
         self._staging_next = 0
+        self.task_tilings = []   # rows-per-tile values that mixers have asked task lists for
         self.steps = 0
 
     # -- requests -------------------------------------------------------------
@@ -115,9 +123,8 @@ class ModelRunner:
         self.check(entries)
         done = self.cache.append_many([(e.request, len(e.tokens)) for e in entries])  # OutOfPages changes nothing
         self.steps += 1
-        key = self._program_key(entries, done) if self.execution == "graph" else None
-        if key is not None:
-            return self._run_program(key, entries, done)
+        if self.execution == "graph":
+            return self._run_program(self._program_key(entries, done), entries, done)
         ctx = self._context(entries, done)
         logits = self.model.forward(ctx)
         if logits is None:
@@ -126,9 +133,10 @@ class ModelRunner:
 
     def _layout(self, T, S, R):
         """Offsets of the packed int32 metadata: tokens, positions, seg_of_row, seg_start, seg_first_pos,
-        state_slots, logit_rows, then per group slots and tables."""
+        state_slots, logit_rows, then per group slots and tables, then one attention task list per
+        known tiling (its length is the most tiles that T rows in S segments can make)."""
         W, G = self.table_width, len(self.cache.groups)
-        sizes = [T, T, T, S + 1, S, S, R] + [T, S * W] * G
+        sizes = [T, T, T, S + 1, S, S, R] + [T, S * W] * G + [4 * (-(-T // r) + S) for r in self.task_tilings]
         return np.concatenate(([0], np.cumsum(sizes))).astype(np.int64)
 
     def _context(self, entries, done, pad=None, device_buffer=None):
@@ -178,6 +186,11 @@ class ModelRunner:
             row += n
             max_context = max(max_context, d.start + n)
         seg_start[len(entries):] = n_rows
+        tilings = list(self.task_tilings)
+        for i, rows_per_tile in enumerate(tilings):
+            tasks = arr[offsets[7 + 2 * G + i]:offsets[8 + 2 * G + i]].reshape(-1, 4)
+            n = fill_tasks(tasks, [d.count for d in done], rows_per_tile)
+            tasks[n:] = (-1, 0, 0, 0)   # tiles of no segment do nothing
         dev = self._upload(host, total, device_buffer)
 
         def view(i, shape=None):
@@ -189,6 +202,7 @@ class ModelRunner:
         ctx.tokens, ctx.positions, ctx.seg_of_row = view(0), view(1), view(2)
         ctx.seg_start, ctx.seg_first_pos, ctx.state_slots, ctx.logit_rows = view(3), view(4), view(5), view(6)
         ctx.kv = [GroupView(view(7 + 2 * g), view(8 + 2 * g, (S, W)), self.page_size, W) for g in range(G)]
+        ctx.tasks = {r: view(7 + 2 * G + i, (-1, 4)) for i, r in enumerate(tilings)}
         ctx.segments = [(d.request, d.start, d.count) for d in done]
         ctx.max_context = ctx.span_hint = max_context
         ctx.decode_only = all(d.count == 1 for d in done)
@@ -219,23 +233,23 @@ class ModelRunner:
         entry[2].record()
         return target
 
-    # -- captured programs (decode steps) -------------------------------------------
+    # -- captured programs ------------------------------------------------------------
     def _program_key(self, entries, done):
-        """Decode-only steps that want every row's logits run as a captured graph,
-        keyed by the padded batch size and the context length rounded up to a power
-        of two (it decides how attention splits the keys)."""
-        if not all(d.count == 1 and list(e.want) == [0] for e, d in zip(entries, done)):
-            return None
-        batch = 1 << (len(entries) - 1).bit_length()
-        context = 1 << (max(d.start + 1 for d in done) - 1).bit_length()
-        return (batch, max(context, 256))
+        """What the launches of a step depend on: the padded numbers of rows, segments and
+        wanted rows, whether every segment brings one token, and the context length rounded up
+        to a power of two (it decides how attention splits the keys).  Steps with the same key
+        replay one captured graph; only the metadata they read differs."""
+        rows = sum(d.count for d in done)
+        wanted = sum(len(e.want) for e in entries)
+        decode_only = all(d.count == 1 for d in done)
+        context = 1 << (max(d.start + d.count for d in done) - 1).bit_length()
+        return (_bucket(rows), _bucket(len(entries)), _bucket(wanted), decode_only, max(context, 256))
 
     def _run_program(self, key, entries, done):
-        batch, context = key
+        T, S, R, decode_only, context = key
         program = self.programs.get(key)
         if program is None:
-            total = int(self._layout(batch, batch, batch)[-1])
-            program = {"meta": torch.zeros(total, dtype=torch.int32, device=self.device), "graph": None, "runs": 0}
+            program = {"meta": None, "graph": None, "runs": 0, "tilings": None}
             self.programs[key] = program
             while len(self.programs) > self.program_capacity:
                 oldest = next(iter(self.programs))
@@ -243,15 +257,22 @@ class ModelRunner:
                 del self.programs[oldest]
         else:
             self.programs[key] = self.programs.pop(key)  # most recently used last
-        ctx = self._context(entries, done, pad=(batch, batch, batch), device_buffer=program["meta"])
+        if program["tilings"] != self.task_tilings:
+            # a mixer asked for a task list that the metadata did not hold yet: lay it out again
+            torch.cuda.synchronize()
+            program.update(meta=torch.zeros(int(self._layout(T, S, R)[-1]), dtype=torch.int32, device=self.device),
+                           graph=None, runs=0, tilings=list(self.task_tilings))
+        ctx = self._context(entries, done, pad=(T, S, R), device_buffer=program["meta"])
         ctx.span_hint = context   # launch shapes inside a captured program depend on the key only
-        if program["graph"] is None and program["runs"] >= 1:
+        ctx.decode_only = decode_only
+        if program["graph"] is None and program["runs"] >= 1 and program["tilings"] == self.task_tilings:
             # the first run was eager and allocated every buffer; capture launches nothing
             # nothing but kernel launches may happen while the stream records: keep the garbage
             # collector from freeing device objects (other graphs, events) in the middle of it
             graph = torch.cuda.CUDAGraph()
             collecting = gc.isenabled()
             gc.disable()
+            ctx.capturing = True
             try:
                 with torch.cuda.graph(graph, capture_error_mode="thread_local"):
                     program["logits"] = self.model.forward(ctx)
@@ -265,7 +286,10 @@ class ModelRunner:
         else:
             logits = self.model.forward(ctx)
         program["runs"] += 1
-        return logits[:len(entries)]
+        wanted = sum(len(e.want) for e in entries)
+        if logits is None:
+            return torch.empty((0, self.model.vocab_size), dtype=torch.float32, device=self.device)
+        return logits[:wanted]
 
     # -- attention dispatch -------------------------------------------------------
     def attention(self, ctx, q, q_row_stride, kcache, vcache, view, out, heads, kv_heads, head_dim, window, scale):

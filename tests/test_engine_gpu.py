@@ -96,8 +96,51 @@ def test_graph_replays_match_eager_logits(folders):
         for k in keys:
             fed[k] += 1
     graph_runner = runners[1]
-    assert sum(p["graph"] is not None for p in graph_runner.programs.values()) >= 2
-    assert all(p["runs"] >= 3 for p in graph_runner.programs.values() if p["graph"] is not None)
+    decode_programs = [p for key, p in graph_runner.programs.items() if key[3] and p["graph"] is not None]
+    assert len(decode_programs) >= 2 and all(p["runs"] >= 3 for p in decode_programs)
+
+
+@pytest.mark.parametrize("name,dtype", [("d", "float32"), ("d", "bfloat16"), ("a", "bfloat16"), ("c", "bfloat16")])
+def test_captured_prompt_and_mixed_steps_match_the_plain_model(folders, name, dtype):
+    """In graph mode every step shape becomes a captured program: portions of prompts, alone and
+    beside decoded tokens, padded to the program's sizes.  The same shapes come again and again
+    with other requests, positions and pages; every replay is compared with the plain model."""
+    from runtime.engine import load_model, ModelRunner, StepEntry
+    from conftest import plain_logits, assert_close
+    V = TINY[name]["vocab_size"]
+    model = load_model(folders[name], dtype=dtype)
+    runner = ModelRunner(model, n_pages=24, page_size=8, max_requests=4, execution="graph")
+    for round_ in range(5):
+        seqs = {k: random_tokens(300 + 10 * round_ + i, 45, V) for i, k in enumerate("xyz")}
+        refs = {k: plain_logits(folders[name], seqs[k]) for k in seqs}
+        for k in seqs:
+            runner.create(k)
+        fed = {k: 0 for k in seqs}
+
+        def feed(*parts):
+            entries, places = [], []
+            for k, n in parts:
+                entries.append(StepEntry(k, seqs[k][fed[k]:fed[k] + n], [0, n - 1] if n > 1 else [0]))
+                places += [(k, fed[k]), (k, fed[k] + n - 1)] if n > 1 else [(k, fed[k])]
+                fed[k] += n
+            logits = runner.step(entries).float().cpu().numpy()
+            assert logits.shape[0] == len(places)
+            for row, (k, pos) in zip(logits, places):
+                assert_close(row[None], refs[k][pos][None], dtype, f"round {round_} request {k} position {pos}")
+
+        feed(("x", 19))                        # a portion alone
+        feed(("y", 19))                        # the same shape, another request
+        feed(("x", 1), ("y", 1), ("z", 11))    # decoded tokens beside a portion
+        feed(("x", 1), ("y", 1), ("z", 11))
+        feed(("z", 19))
+        feed(("x", 1), ("y", 1), ("z", 1))
+        feed(("x", 1), ("y", 1), ("z", 1))
+        for k in seqs:
+            runner.release(k)
+    captured = [p for p in runner.programs.values() if p["graph"] is not None]
+    assert len(captured) >= 3 and all(p["runs"] >= 3 for p in captured)
+    assert any(not key[3] for key, p in runner.programs.items() if p["graph"] is not None), "no prompt step was captured"
+    runner.cache.check()
 
 
 def test_temperature_sampling_is_seeded_and_independent_of_the_batch(folders):

@@ -1,0 +1,29 @@
+"""Host-side metadata of a step: the attention task lists and the sizes that captured programs pad to."""
+import numpy as np
+
+from runtime.engine.context import fill_tasks
+from runtime.engine.runner import _bucket
+
+
+def test_task_lists_cover_every_row_once_and_never_cross_a_segment():
+    rng = np.random.default_rng(0)
+    for _ in range(50):
+        counts = rng.integers(1, 40, size=rng.integers(1, 6)).tolist()
+        rows_per_tile = int(rng.choice([1, 2, 4, 5, 16, 64]))
+        most = -(-sum(counts) // rows_per_tile) + len(counts)
+        tasks = np.full((most, 4), -7, dtype=np.int32)
+        n = fill_tasks(tasks, counts, rows_per_tile)
+        assert n == sum(-(-c // rows_per_tile) for c in counts) <= most
+        assert (tasks[n:] == -7).all()
+        starts = np.concatenate(([0], np.cumsum(counts)))
+        seen = []
+        for seg, first, rows, zero in tasks[:n]:
+            assert zero == 0 and 1 <= rows <= rows_per_tile
+            assert starts[seg] <= first and first + rows <= starts[seg + 1]
+            seen += list(range(first, first + rows))
+        assert seen == list(range(sum(counts)))
+
+
+def test_program_sizes_are_powers_of_two_then_multiples_of_64():
+    assert [_bucket(n) for n in (0, 1, 2, 3, 5, 33, 64, 65, 128, 129, 2048)] == [0, 1, 2, 4, 8, 64, 64, 128, 128, 192, 2048]
+    assert all(_bucket(n) >= n for n in range(1, 500))

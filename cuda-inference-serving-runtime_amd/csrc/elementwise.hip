@@ -46,14 +46,68 @@ __global__ void rmsnorm_kernel(const float* __restrict__ x, const float* __restr
     for (int d = threadIdx.x; d < dim; d += 256) store_f32(dst + d, src[d] * scale * w[d]);
 }
 
+// The same for rows of a multiple of four floats, 16-byte aligned: one wavefront a row, the row stays
+// in registers (R float4 a lane: dim <= 256 R), loads and stores of 16 bytes.  The sum of squares of a
+// row is made by its own wave in a fixed order, whatever else is in the batch.
+template <typename T, int R>
+__global__ void __launch_bounds__(256)
+rmsnorm_wave_kernel(const float* __restrict__ x, const float* __restrict__ w, T* __restrict__ y,
+                    const int* __restrict__ rows, int n_out, int dim, float eps) {
+    const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+    const int orow = blockIdx.x * 4 + wave;
+    if (orow >= n_out) return;
+    const int irow = rows ? rows[orow] : orow;
+    const int n4 = dim / 4;
+    const float4* src = (const float4*)(x + (size_t)irow * dim);
+    const float4* w4 = (const float4*)w;
+    float4 v[R], g[R];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+        const int c = min(lane + WAVE * i, n4 - 1);   // past the row: a copy of its last chunk, not counted
+        v[i] = src[c];
+        g[i] = w4[c];
+    }
+#pragma unroll
+    for (int i = 0; i < R; ++i)
+        if (lane + WAVE * i < n4) ss += v[i].x * v[i].x + v[i].y * v[i].y + v[i].z * v[i].z + v[i].w * v[i].w;
+    const float scale = 1.0f / sqrtf(wave_sum(ss) / (float)dim + eps);
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+        const int c = lane + WAVE * i;
+        if (c >= n4) continue;
+        const float a = v[i].x * scale * g[i].x, b = v[i].y * scale * g[i].y;
+        const float cc = v[i].z * scale * g[i].z, d = v[i].w * scale * g[i].w;
+        if (sizeof(T) == 4) {
+            ((float4*)((float*)y + (size_t)orow * dim))[c] = make_float4(a, b, cc, d);
+        } else {
+            ((uint2*)((bf16_t*)y + (size_t)orow * dim))[c] = make_uint2(pack_bf16x2(a, b), pack_bf16x2(cc, d));
+        }
+    }
+}
+
+template <typename T>
+static int launch_rmsnorm(const float* x, const float* w, T* y, const int* rows, int n_out, int dim, float eps,
+                          hipStream_t stream) {
+    const bool vec = dim % 4 == 0 && dim <= 8192 && ((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0) &&
+                     ((uintptr_t)y % 16 == 0);
+    const int blocks = (n_out + 3) / 4, chunks = (dim / 4 + WAVE - 1) / WAVE;
+    if (!vec) rmsnorm_kernel<T><<<n_out, 256, 0, stream>>>(x, w, y, rows, dim, eps);
+    else if (chunks <= 1) rmsnorm_wave_kernel<T, 1><<<blocks, 256, 0, stream>>>(x, w, y, rows, n_out, dim, eps);
+    else if (chunks <= 2) rmsnorm_wave_kernel<T, 2><<<blocks, 256, 0, stream>>>(x, w, y, rows, n_out, dim, eps);
+    else if (chunks <= 3) rmsnorm_wave_kernel<T, 3><<<blocks, 256, 0, stream>>>(x, w, y, rows, n_out, dim, eps);
+    else if (chunks <= 4) rmsnorm_wave_kernel<T, 4><<<blocks, 256, 0, stream>>>(x, w, y, rows, n_out, dim, eps);
+    else if (chunks <= 8) rmsnorm_wave_kernel<T, 8><<<blocks, 256, 0, stream>>>(x, w, y, rows, n_out, dim, eps);
+    else if (chunks <= 16) rmsnorm_wave_kernel<T, 16><<<blocks, 256, 0, stream>>>(x, w, y, rows, n_out, dim, eps);
+    else rmsnorm_wave_kernel<T, 32><<<blocks, 256, 0, stream>>>(x, w, y, rows, n_out, dim, eps);
+    return CISR_LAUNCH_CHECK();
+}
+
 extern "C" int cisr_rmsnorm(const float* x, const float* w, void* y, const int* rows, int n_out,
                             int dim, float eps, int out_dtype, hipStream_t stream) {
     if (n_out <= 0) return 0;
-    if (out_dtype == DT_F32)
-        rmsnorm_kernel<float><<<n_out, 256, 0, stream>>>(x, w, (float*)y, rows, dim, eps);
-    else
-        rmsnorm_kernel<bf16_t><<<n_out, 256, 0, stream>>>(x, w, (bf16_t*)y, rows, dim, eps);
-    return CISR_LAUNCH_CHECK();
+    if (out_dtype == DT_F32) return launch_rmsnorm<float>(x, w, (float*)y, rows, n_out, dim, eps, stream);
+    return launch_rmsnorm<bf16_t>(x, w, (bf16_t*)y, rows, n_out, dim, eps, stream);
 }
 
 // x += delta, then y = rmsnorm(x) (reference: kernels/execution.cu:12-24; here
@@ -191,17 +245,79 @@ __global__ void rope_scatter_kernel(T* __restrict__ qkv, const int* __restrict__
     }
 }
 
+// The same for bf16 rows whose whole heads turn (rot == dim) with dim a multiple of 16: one wavefront a
+// row, every lane turns 8 pairs at a time with 16-byte loads and stores.
+__global__ void __launch_bounds__(256)
+rope_scatter_wave_kernel(bf16_t* __restrict__ qkv, const int* __restrict__ positions, const int* __restrict__ slots,
+                         const float* __restrict__ cos_tab, const float* __restrict__ sin_tab,
+                         bf16_t* __restrict__ kcache, bf16_t* __restrict__ vcache, int rows, int heads, int kv_heads,
+                         int dim, int page_size, int max_pos, int has_kv) {
+    typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+    const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+    const int row = blockIdx.x * 4 + wave;
+    if (row >= rows) return;
+    const int half = dim / 2, per_head = half / 8;   // 8-pair chunks of a head
+    int pos = positions[row];
+    pos = pos < 0 ? 0 : (pos >= max_pos ? max_pos - 1 : pos);
+    const float* cs = cos_tab + (size_t)pos * half;
+    const float* sn = sin_tab + (size_t)pos * half;
+    const int row_width = (heads + (has_kv ? 2 * kv_heads : 0)) * dim;
+    bf16_t* base = qkv + (size_t)row * row_width;
+    const int slot = (has_kv && slots) ? slots[row] : -1;
+    const int page = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot % page_size : 0;
+    const int turning = heads + (slot >= 0 ? kv_heads : 0);   // q heads, then k heads if they have a place to go
+    for (int i = lane; i < turning * per_head; i += WAVE) {
+        const int h = i / per_head, d = (i % per_head) * 8;
+        const bf16_t* p = base + h * dim + d;
+        const u32x4 av = *(const u32x4*)p, bv = *(const u32x4*)(p + half);
+        const float4 c0 = *(const float4*)(cs + d), c1 = *(const float4*)(cs + d + 4);
+        const float4 s0 = *(const float4*)(sn + d), s1 = *(const float4*)(sn + d + 4);
+        const float c[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
+        const float sv[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+        uint32_t lo[4], hi[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float a0 = __uint_as_float(av[j] << 16), a1 = __uint_as_float(av[j] & 0xffff0000u);
+            const float b0 = __uint_as_float(bv[j] << 16), b1 = __uint_as_float(bv[j] & 0xffff0000u);
+            lo[j] = pack_bf16x2(a0 * c[2 * j] - b0 * sv[2 * j], a1 * c[2 * j + 1] - b1 * sv[2 * j + 1]);
+            hi[j] = pack_bf16x2(b0 * c[2 * j] + a0 * sv[2 * j], b1 * c[2 * j + 1] + a1 * sv[2 * j + 1]);
+        }
+        bf16_t* dst = h < heads ? base + h * dim + d
+                                : kcache + (((size_t)page * kv_heads + (h - heads)) * page_size + off) * dim + d;
+        *(u32x4*)dst = (u32x4){lo[0], lo[1], lo[2], lo[3]};
+        *(u32x4*)(dst + half) = (u32x4){hi[0], hi[1], hi[2], hi[3]};
+    }
+    if (slot < 0) return;
+    // v heads: 8 coordinates a lane, written to the transposed page one by one
+    const bf16_t* vb = base + (heads + kv_heads) * dim;
+    for (int i = lane; i < kv_heads * (dim / 8); i += WAVE) {
+        const int h = i / (dim / 8), d = (i % (dim / 8)) * 8;
+        const u32x4 v = *(const u32x4*)(vb + h * dim + d);
+        bf16_t* dst = vcache + (((size_t)page * kv_heads + h) * dim + d) * page_size + off;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            dst[(size_t)(2 * j) * page_size] = (bf16_t)(v[j] & 0xffffu);
+            dst[(size_t)(2 * j + 1) * page_size] = (bf16_t)(v[j] >> 16);
+        }
+    }
+}
+
 extern "C" int cisr_rope_scatter(void* qkv, const int* positions, const int* slots, const float* cos_tab,
                                  const float* sin_tab, void* kcache, void* vcache, int rows, int heads,
                                  int kv_heads, int dim, int rot, int page_size, int max_pos, int has_kv,
                                  int dtype, hipStream_t stream) {
     if (rows <= 0) return 0;
-    if (dtype == DT_F32)
+    if (dtype == DT_F32) {
         rope_scatter_kernel<float><<<rows, 256, 0, stream>>>((float*)qkv, positions, slots, cos_tab, sin_tab,
             (float*)kcache, (float*)vcache, heads, kv_heads, dim, rot, page_size, max_pos, has_kv);
-    else
+    } else if (rot == dim && dim % 16 == 0 && (uintptr_t)qkv % 16 == 0 && (uintptr_t)cos_tab % 16 == 0 &&
+               (uintptr_t)sin_tab % 16 == 0 && (!has_kv || (uintptr_t)kcache % 16 == 0)) {
+        rope_scatter_wave_kernel<<<(rows + 3) / 4, 256, 0, stream>>>((bf16_t*)qkv, positions, slots, cos_tab, sin_tab,
+            (bf16_t*)kcache, (bf16_t*)vcache, rows, heads, kv_heads, dim, page_size, max_pos, has_kv);
+    } else {
         rope_scatter_kernel<bf16_t><<<rows, 256, 0, stream>>>((bf16_t*)qkv, positions, slots, cos_tab, sin_tab,
             (bf16_t*)kcache, (bf16_t*)vcache, heads, kv_heads, dim, rot, page_size, max_pos, has_kv);
+    }
     return CISR_LAUNCH_CHECK();
 }
 

@@ -116,11 +116,17 @@ __device__ __forceinline__ u32x4 load_chunk(const bf16_t* base, int ld, int row,
 // compute unit with a single block: PF tiles of global loads are in flight in a ring of registers,
 // and two LDS buffers let the next tile be written while the current one is multiplied, with one
 // barrier per tile.
-template <int TM, int TN, int BK, typename TC, bool VEC>
+// SWIGLU: W holds two blocks of N rows, `dual_off` rows apart (gate, then up).  A wave's first TN/2
+// column tiles take gate rows and its last TN/2 the up rows of the same output columns, so a lane ends
+// with gate and up of one output element in its registers and writes silu(gate) * up (both rounded to
+// bf16 first, as the two-kernel path does); a block then covers BN/2 output columns.
+template <int TM, int TN, int BK, typename TC, bool VEC, bool SWIGLU = false>
 __global__ void __launch_bounds__(256)
 gemm_bf16_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, int ldw,
-                 TC* C, int ldc, const float* R, int ldr, int M, int N, int K) {
+                 TC* C, int ldc, const float* R, int ldr, int M, int N, int K, int dual_off = 0) {
+    static_assert(!SWIGLU || (TN % 2 == 0 && VEC), "the activation pairs column tiles");
     constexpr int BM = 2 * TM * 16, BN = 2 * TN * 16;
+    constexpr int BN_OUT = SWIGLU ? BN / 2 : BN;           // output columns a block covers
     constexpr int STRIDE = BK + 8;
     constexpr int CPR = BK / 8;                            // 16-byte chunks per tile row
     static_assert((BM * CPR) % 256 == 0 && (BN * CPR) % 256 == 0, "a tile is a whole number of 16-byte chunks per thread");
@@ -136,11 +142,11 @@ gemm_bf16_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict
     // The hardware deals consecutive workgroups round-robin to the 8 XCDs, each with an L2 of its
     // own.  Renumber so that an XCD gets a contiguous run of tiles (column tiles fastest): it then
     // touches one band of A rows instead of all of A, and W stays in its L2 across the band.
-    const int tiles_n = (N + BN - 1) / BN, tiles = tiles_n * ((M + BM - 1) / BM);
+    const int tiles_n = (N + BN_OUT - 1) / BN_OUT, tiles = tiles_n * ((M + BM - 1) / BM);
     const int per_xcd = (tiles + 7) / 8;
     const int tile = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
     if (tile >= tiles) return;   // the grid is rounded up to a multiple of 8
-    const int m0 = (tile / tiles_n) * BM, n0 = (tile % tiles_n) * BN;
+    const int m0 = (tile / tiles_n) * BM, n0 = (tile % tiles_n) * BN_OUT;
 
     f32x4 acc[TM][TN];
 #pragma unroll
@@ -158,7 +164,14 @@ gemm_bf16_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict
 #pragma unroll
         for (int i = 0; i < W_PER_THREAD; ++i) {
             const int c = tid + i * 256;
-            fw[i] = load_chunk<VEC>(W, ldw, n0 + c / CPR, N, k0 + (c % CPR) * 8, K);
+            if (SWIGLU) {
+                // local column -> (wave, column tile, column): the W row of its output column, gate or up
+                const int lc = c / CPR, jj = (lc % (TN * 16)) / 16;
+                const int oc = min(n0 + (lc / (TN * 16)) * (TN / 2) * 16 + (jj % (TN / 2)) * 16 + lc % 16, N - 1);
+                fw[i] = load_chunk<VEC>(W, ldw, oc + (jj >= TN / 2 ? dual_off : 0), dual_off + N, k0 + (c % CPR) * 8, K);
+            } else {
+                fw[i] = load_chunk<VEC>(W, ldw, n0 + c / CPR, N, k0 + (c % CPR) * 8, K);
+            }
         }
     };
 #pragma unroll
@@ -206,6 +219,22 @@ gemm_bf16_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict
                 }
             }
         }
+    }
+    if (SWIGLU) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN / 2; ++j) {
+                const int n = n0 + wn * (TN / 2) * 16 + j * 16 + r;
+                if (n >= N) continue;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int m = m0 + wm * TM * 16 + i * 16 + g * 4 + e;
+                    const float gq = bf16_to_f32(f32_to_bf16(acc[i][j][e])), uq = bf16_to_f32(f32_to_bf16(acc[i][j + TN / 2][e]));
+                    if (m < M) store_f32(C + (size_t)m * ldc + n, gq / (1.0f + expf(-gq)) * uq);
+                }
+            }
+        return;
     }
     // lane holds rows 4g..4g+3 of column r in every 16 x 16 tile.  The residual is read with
     // unconditional loads from clamped addresses, all issued before the first is used.
@@ -256,6 +285,31 @@ static int launch_bf16(const bf16_t* A, int lda, const bf16_t* W, int ldw, void*
         else gemm_bf16_kernel<TM, TN, BK, bf16_t, false><<<grid, 256, 0, stream>>>(A, lda, W, ldw, (bf16_t*)C, ldc, R, ldr, M, N, K);
     }
     return CISR_LAUNCH_CHECK();
+}
+
+// C[M, N] = silu(A . Wg^T) * (A . Wu^T), W = [Wg; Wu] with `dual_off` rows between the blocks; bf16 in and out,
+// 16-byte aligned rows with K % 8 == 0.
+template <int TM, int TN, int BK>
+static int launch_bf16_swiglu(const bf16_t* A, int lda, const bf16_t* W, int ldw, bf16_t* C, int ldc, int M, int N, int K,
+                              int dual_off, hipStream_t stream) {
+    constexpr int BM = 2 * TM * 16, BN_OUT = TN * 16;
+    const long long tiles = (long long)((N + BN_OUT - 1) / BN_OUT) * ((M + BM - 1) / BM);
+    if (tiles > (1ll << 30)) return (int)hipErrorInvalidValue;
+    dim3 grid((unsigned)((tiles + 7) / 8 * 8));
+    gemm_bf16_kernel<TM, TN, BK, bf16_t, true, true><<<grid, 256, 0, stream>>>(A, lda, W, ldw, C, ldc, nullptr, 0, M, N, K, dual_off);
+    return CISR_LAUNCH_CHECK();
+}
+
+extern "C" int cisr_gemm_bf16_swiglu(const void* A, int lda, const void* W, int ldw, void* C, int ldc, int M, int N, int K,
+                                     int dual_off, hipStream_t stream) {
+    if (M <= 0 || N <= 0) return 0;
+    if (K <= 0 || K % 8 || lda % 8 || ldw % 8 || ((uintptr_t)A) % 16 || ((uintptr_t)W) % 16 || dual_off < N)
+        return (int)hipErrorInvalidValue;
+    const bf16_t* a = (const bf16_t*)A; const bf16_t* w = (const bf16_t*)W;
+    auto blocks = [&](int bm, int bn) { return (long long)((M + bm - 1) / bm) * ((2 * N + bn - 1) / bn); };
+    if (blocks(128, 128) >= 512) return launch_bf16_swiglu<4, 4, 32>(a, lda, w, ldw, (bf16_t*)C, ldc, M, N, K, dual_off, stream);
+    if (blocks(128, 64) >= 512) return launch_bf16_swiglu<4, 2, 64>(a, lda, w, ldw, (bf16_t*)C, ldc, M, N, K, dual_off, stream);
+    return launch_bf16_swiglu<2, 2, 64>(a, lda, w, ldw, (bf16_t*)C, ldc, M, N, K, dual_off, stream);
 }
 
 // Tile choice: the largest tile that still gives the 256 compute units a few blocks each.

@@ -22,9 +22,12 @@ class GroupView:
     width: int
 
 
-def fill_tasks(tasks, counts, rows_per_tile):
+def fill_tasks(tasks, counts, rows_per_tile, starts=None):
     """Write (segment, first row, rows, 0) for tiles of at most `rows_per_tile` consecutive
-    rows of one segment into the int32 array tasks[n, 4]; returns how many were written."""
+    rows of one segment into the int32 array tasks[n, 4]; returns how many were written.
+    With `starts` (the position of each segment's first row) the tiles are ordered by the
+    number of keys they attend to, most first: blocks are handed out in this order, and the
+    long ones must not be the last to start."""
     n = row = 0
     for seg, count in enumerate(counts):
         tiles = -(-count // rows_per_tile)
@@ -35,6 +38,10 @@ def fill_tasks(tasks, counts, rows_per_tile):
         tasks[n:n + tiles, 3] = 0
         n += tiles
         row += count
+    if starts is not None and n > 1:
+        first_row = np.concatenate(([0], np.cumsum(counts)))[tasks[:n, 0]]
+        keys = np.asarray(starts, dtype=np.int64)[tasks[:n, 0]] + (tasks[:n, 1] - first_row) + tasks[:n, 2]
+        tasks[:n] = tasks[:n][np.argsort(-keys, kind="stable")]
     return n
 
 
@@ -69,7 +76,7 @@ class StepContext:
                 raise RuntimeError(f"a task list of {rows_per_tile} rows a tile was first asked for under graph capture")
             counts = [count for _, _, count in self.segments]
             host = np.full((sum(-(-c // rows_per_tile) for c in counts), 4), -1, dtype=np.int32)
-            fill_tasks(host, counts, rows_per_tile)
+            fill_tasks(host, counts, rows_per_tile, [start for _, start, _ in self.segments])
             tasks = torch.from_numpy(host).to(self.device, non_blocking=False)
             self.tasks[rows_per_tile] = tasks
             if rows_per_tile not in self.runner.task_tilings:

@@ -189,7 +189,7 @@ class ModelRunner:
         tilings = list(self.task_tilings)
         for i, rows_per_tile in enumerate(tilings):
             tasks = arr[offsets[7 + 2 * G + i]:offsets[8 + 2 * G + i]].reshape(-1, 4)
-            n = fill_tasks(tasks, [d.count for d in done], rows_per_tile)
+            n = fill_tasks(tasks, [d.count for d in done], rows_per_tile, [d.start for d in done])
             tasks[n:] = (-1, 0, 0, 0)   # tiles of no segment do nothing
         dev = self._upload(host, total, device_buffer)
 

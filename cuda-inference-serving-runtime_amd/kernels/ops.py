@@ -48,6 +48,7 @@ def _declare(h):
         "cisr_attn_rowwise": [p, i, p, p, p, p, p, p, p, p, i, i, i, i, i, i, i, f, i, i, p],
         "cisr_gemm_f32": [p, i, p, i, p, i, p, i, i, i, i, p],
         "cisr_gemm_bf16": [p, i, p, i, p, i, p, i, i, i, i, i, p],
+        "cisr_gemm_bf16_swiglu": [p, i, p, i, p, i, i, i, i, i, p],
         "cisr_gemm_skinny_bf16": [p, i, p, i, p, i, p, i, i, i, i, i, i, p, f, p, p],
         "cisr_qkv_rope_skinny": [p, i, p, i, p, i, i, i, p, f, p, p, p, p, p, p, i, i, i, i, i, p],
         "cisr_attn_merge": [p, p, p, i, i, i, i, p],
@@ -285,9 +286,9 @@ def fused_norm_ok(x, w, rows_out):
 
 
 def swiglu_fused_ok(a, w_gate_up):
-    """Whether gemm_swiglu runs as one kernel for these operands (no scratch buffer needed)."""
-    return (a.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16 and a.shape[0] <= SKINNY_ROWS
-            and _skinny_ok(a, w_gate_up))
+    """Whether gemm_swiglu runs as one kernel for these operands (no scratch buffer needed): bf16 with
+    16-byte aligned rows; few rows take the weight-streaming kernel, more the tiled one."""
+    return a.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16 and a.is_cuda and _skinny_ok(a, w_gate_up)
 
 
 def gemm_normed(x, norm, w, out):
@@ -322,10 +323,14 @@ def gemm_swiglu(a, w_gate_up, out, scratch=None, norm=None):
         return out
     if out.dtype != a.dtype or a.dtype != w_gate_up.dtype:
         raise KernelError("gemm_swiglu: dtypes differ")
-    if swiglu_fused_ok(a, w_gate_up) and a.is_cuda:
-        _check(lib().cisr_gemm_skinny_bf16(a.data_ptr(), a.stride(0), w_gate_up.data_ptr(), w_gate_up.stride(0),
-                                           out.data_ptr(), out.stride(0), None, 0, m, inter, k, BF16, inter, None, 0.0,
-                                           None, _stream()), "gemm_swiglu")
+    if swiglu_fused_ok(a, w_gate_up):
+        if m <= SKINNY_ROWS:
+            _check(lib().cisr_gemm_skinny_bf16(a.data_ptr(), a.stride(0), w_gate_up.data_ptr(), w_gate_up.stride(0),
+                                               out.data_ptr(), out.stride(0), None, 0, m, inter, k, BF16, inter, None, 0.0,
+                                               None, _stream()), "gemm_swiglu")
+        else:   # many rows: the tiled product with the activation as its epilogue
+            _check(lib().cisr_gemm_bf16_swiglu(a.data_ptr(), a.stride(0), w_gate_up.data_ptr(), w_gate_up.stride(0),
+                                               out.data_ptr(), out.stride(0), m, inter, k, inter, _stream()), "gemm_swiglu")
         return out
     if scratch is None:
         raise KernelError("gemm_swiglu: this shape needs a scratch buffer [M, 2I]")

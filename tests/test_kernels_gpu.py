@@ -59,7 +59,7 @@ def test_embedding(ops, dtype):
     np.testing.assert_array_equal(f64(out), f64(table)[ids.cpu().numpy()])
 
 
-@pytest.mark.parametrize("dim", [10, 64, 130, 576, 4100])
+@pytest.mark.parametrize("dim", [10, 64, 130, 576, 2048, 4100, 8200])
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
 def test_rmsnorm(ops, dim, out_dtype):
     # reference tests/test_cuda.py:28-36 (dims 10/64/130/512)
@@ -388,9 +388,19 @@ def test_gemm_skinny_and_fused_swiglu(ops):
         want = P.swiglu(gq[:, :I], gq[:, I:])
         got = ops.gemm_swiglu(a, w, torch.empty(M, I, dtype=torch.bfloat16, device=DEV))
         np.testing.assert_allclose(f64(got), want, rtol=2e-2, atol=2e-2)
-        two = ops.gemm_swiglu(rnd(70, K, dtype=torch.bfloat16, seed=4, scale=0.5), w, torch.empty(70, I, dtype=torch.bfloat16, device=DEV),
-                              scratch=torch.empty(70, 2 * I, dtype=torch.bfloat16, device=DEV))   # more rows: product + activation
-        assert two.shape == (70, I)
+        for rows in (70, 300):   # more rows: the tiled product with the activation as its epilogue
+            big = rnd(rows, K, dtype=torch.bfloat16, seed=4, scale=0.5)
+            gq = torch.from_numpy(f64(big) @ f64(w).T).to(torch.bfloat16).double().numpy()
+            tiled = ops.gemm_swiglu(big, w, torch.empty(rows, I, dtype=torch.bfloat16, device=DEV))
+            np.testing.assert_allclose(f64(tiled), P.swiglu(gq[:, :I], gq[:, I:]), rtol=2e-2, atol=2e-2)
+    # rows that are not 16-byte aligned: product into a scratch buffer, then the activation kernel
+    a, w = rnd(70, 100, dtype=torch.bfloat16, seed=8, scale=0.5), rnd(2 * 90, 100, dtype=torch.bfloat16, seed=9, scale=0.2)
+    assert not ops.swiglu_fused_ok(a, w)
+    with pytest.raises(ops.KernelError):
+        ops.gemm_swiglu(a, w, torch.empty(70, 90, dtype=torch.bfloat16, device=DEV))
+    gq = torch.from_numpy(f64(a) @ f64(w).T).to(torch.bfloat16).double().numpy()
+    two = ops.gemm_swiglu(a, w, torch.empty(70, 90, dtype=torch.bfloat16, device=DEV), scratch=torch.empty(70, 180, dtype=torch.bfloat16, device=DEV))
+    np.testing.assert_allclose(f64(two), P.swiglu(gq[:, :90], gq[:, 90:]), rtol=2e-2, atol=2e-2)
     # a row's result does not depend on how many rows are beside it
     a, w = rnd(64, 576, dtype=torch.bfloat16, seed=6), rnd(300, 576, dtype=torch.bfloat16, seed=7)
     full = ops.gemm(a, w, torch.empty(64, 300, device=DEV))

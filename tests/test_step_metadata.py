@@ -22,6 +22,13 @@ def test_task_lists_cover_every_row_once_and_never_cross_a_segment():
             assert starts[seg] <= first and first + rows <= starts[seg + 1]
             seen += list(range(first, first + rows))
         assert seen == list(range(sum(counts)))
+        # with the segments' first positions: the same tiles, those with the most keys first
+        seg_starts = rng.integers(0, 100, size=len(counts)).tolist()
+        ordered = np.full((most, 4), -7, dtype=np.int32)
+        assert fill_tasks(ordered, counts, rows_per_tile, seg_starts) == n
+        assert sorted(map(tuple, ordered[:n])) == sorted(map(tuple, tasks[:n]))
+        keys = [seg_starts[seg] + first - starts[seg] + rows for seg, first, rows, _ in ordered[:n]]
+        assert keys == sorted(keys, reverse=True)
 
 
 def test_program_sizes_are_powers_of_two_then_multiples_of_64():

@@ -110,6 +110,32 @@ __global__ void attn_merge_kernel(const float* __restrict__ part_o, const float*
                                   T* __restrict__ out, int heads, int dim, int splits) {
     const int row = blockIdx.x, head = blockIdx.y;
     const size_t base = ((size_t)row * heads + head) * splits;
+    if (splits <= 16) {
+        // every load is issued before the first is used (one trip to memory instead of two); splits
+        // past the count read the last one again and are left out of the sums
+        for (int d = threadIdx.x; d < dim; d += blockDim.x) {
+            float ms[16], ls[16], os[16];
+#pragma unroll
+            for (int s = 0; s < 16; ++s) {
+                const size_t at = base + min(s, splits - 1);
+                ms[s] = part_ml[at * 2]; ls[s] = part_ml[at * 2 + 1]; os[s] = part_o[at * dim + d];
+            }
+            float m = -INFINITY;
+#pragma unroll
+            for (int s = 0; s < 16; ++s) if (s < splits) m = fmaxf(m, ms[s]);
+            float den = 0.f, num = 0.f;
+#pragma unroll
+            for (int s = 0; s < 16; ++s) {
+                if (s >= splits) continue;
+                const float dm = ms[s] - m;
+                const float w = ls[s] > 0.f ? (LOG2 ? exp2f(dm) : expf(dm)) * ls[s] : 0.f;
+                den += w;
+                num += w * os[s];
+            }
+            store_f32(out + ((size_t)row * heads + head) * dim + d, den > 0.f ? num / den : 0.f);
+        }
+        return;
+    }
     float m = -INFINITY;
     for (int s = 0; s < splits; ++s) m = fmaxf(m, part_ml[(base + s) * 2]);
     for (int d = threadIdx.x; d < dim; d += blockDim.x) {

@@ -51,9 +51,9 @@ class ModelRunner:
         self.model = model
         self.execution = execution
         self.programs, self.program_capacity = {}, 16
-        self.block_tiles = False   # attention of long portions through LDS-shared tiles (measured slower so far)
+        self.block_tiles = int(os.environ.get("CISR_BLOCK_TILES", "0"))   # long portions: LDS-shared tiles of 64 x this items
         self.tile_waves = int(os.environ.get("CISR_TILE_WAVES", "4"))   # wavefronts that share one tile's keys
-        self.item_tiles = int(os.environ.get("CISR_ITEM_TILES", "1"))   # 16-item tiles a wave (2: measured slower)
+        self.item_tiles = int(os.environ.get("CISR_ITEM_TILES", "2"))   # 16-item tiles a wave of long portions (small heads)
         self.device = torch.device(device)
         self.page_size = page_size
         self.max_requests = max_requests
@@ -311,16 +311,20 @@ class ModelRunner:
                 ops.attention_mfma(q, q_row_stride, kcache, vcache, view.tables, ctx.seg_of_row, ctx.positions, out,
                                    heads, kv_heads, head_dim, view.page_size, window, scale, None, splits, workspace, waves)
             else:
-                # long portions with small heads: 32/GC rows a block, every wave owns two 16-item tiles
-                # (keys and values are loaded once for both); otherwise 16/GC rows a block.  The
-                # LDS-shared 64/GC-row variant exists but measured slower and is off.
+                # long portions: the four waves of a block own different rows and share each step's keys and
+                # values through LDS (64 or 128 items a block); otherwise the waves of a block share one tile
+                # of 16 items (32 with small heads) and split its keys
                 long_portions = rows >= 16 * ctx.n_segments
-                block_tiles = self.block_tiles and long_portions
-                item_tiles = 2 if self.item_tiles == 2 and long_portions and head_dim <= 64 and not block_tiles else 1
-                tasks = ctx.attention_tasks((64 if block_tiles else 16 * item_tiles) // heads_per_chunk)
+                block_tiles = self.block_tiles if long_portions and head_dim <= 128 else 0
+                if block_tiles:
+                    item_tiles = block_tiles
+                    tasks = ctx.attention_tasks(64 * item_tiles // heads_per_chunk)
+                else:
+                    item_tiles = 2 if self.item_tiles == 2 and long_portions and head_dim <= 64 else 1
+                    tasks = ctx.attention_tasks(16 * item_tiles // heads_per_chunk)
                 ops.attention_mfma(q, q_row_stride, kcache, vcache, view.tables, ctx.seg_of_row, ctx.positions, out,
                                    heads, kv_heads, head_dim, view.page_size, window, scale, tasks, waves=self.tile_waves,
-                                   block_tiles=block_tiles, item_tiles=item_tiles)
+                                   block_tiles=bool(block_tiles), item_tiles=item_tiles)
             return
         splits = self._splits(rows * heads, span)
         workspace = None

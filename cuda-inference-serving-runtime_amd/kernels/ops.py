@@ -380,8 +380,9 @@ def attention_mfma(q, q_row_stride, kcache, vcache, tables, seg_of_row, position
                    item_tiles=1):
     """Matrix-core attention (bf16).  tasks int32 [n, 4] = (segment, first row, rows, 0) runs tiles of
     prompt rows: one tile of 16/GC rows a block whose waves share the keys (with item_tiles=2, head sizes up to
-    64: 32/GC rows, two item tiles a wave), or with `block_tiles` one tile of 64/GC rows a block with keys and
-    values shared through LDS (GC = query heads per key head, at most 16); tasks None runs one block
+    64: 32/GC rows, two item tiles a wave), or with `block_tiles` (head sizes up to 128) one tile of
+    64 item_tiles / GC rows a block whose four waves own different rows and share keys and values through LDS
+    (GC = query heads per key head, at most 16); tasks None runs one block
     per row (decode) of `waves` wavefronts (4 or 8) with `splits` blocks along the keys; splits > 1 needs
     workspace = (partials float, statistics float) and a merge."""
     rows = out.shape[0]
@@ -389,18 +390,25 @@ def attention_mfma(q, q_row_stride, kcache, vcache, tables, seg_of_row, position
         raise KernelError(f"attention_mfma: head size {dim} / page size {page_size} / dtype {out.dtype} not supported")
     if heads % kv_heads:
         raise KernelError(f"attention: {heads} query heads do not divide into {kv_heads} key heads")
+    if not scale > 0:
+        raise KernelError("attention_mfma: the score scale must be positive (the maximum is taken before scaling)")
     if q.dtype != out.dtype or kcache.dtype != out.dtype or q_row_stride % 8 or q.data_ptr() % 16:
         raise KernelError("attention_mfma: q, cache and out must be bfloat16 with 16-byte aligned rows")
     if q.numel() < (rows - 1) * q_row_stride + heads * dim:
         raise KernelError("attention: q buffer too small for its stride")
     pages = kcache.shape[0]
+    if kcache.numel() >= 2 ** 32 or vcache.numel() >= 2 ** 32:
+        raise KernelError("attention_mfma: a layer's keys (or values) must be fewer than 2^32 elements (32-bit offsets)")
     dpad = -(-dim // 32) * 32
     fn = getattr(lib(), f"cisr_attn_mfma_d{dpad}")
     po = pm = tp = None
     if tasks is not None:
-        if item_tiles not in (1, 2) or (item_tiles == 2 and (dim > 64 or block_tiles)):
+        if item_tiles not in (1, 2) or (item_tiles == 2 and dim > 64 and not block_tiles):
             raise KernelError("attention_mfma: two item tiles a wave need a head size of at most 64")
-        n_tasks, mode, splits = tasks.shape[0], (2 if block_tiles else 3 if item_tiles == 2 else 0), 1
+        if block_tiles and dpad > 128:
+            raise KernelError("attention_mfma: block tiles need a head size of at most 128")
+        n_tasks, splits = tasks.shape[0], 1
+        mode = (2 if item_tiles == 1 else 4) if block_tiles else (3 if item_tiles == 2 else 0)
         tp = _dev(tasks, "tasks", torch.int32, (n_tasks, 4))
     else:
         n_tasks, mode = rows, 1

@@ -275,9 +275,9 @@ def run_mfma(ops, qt, kt, vt, tables, rows, page_size, mode, splits=1, window=No
     out = torch.full((T, heads * dim), 9.0, dtype=qt.dtype, device=DEV)
     tasks = None
     ws = (torch.empty(T * heads * splits * dim, device=DEV), torch.empty(T * heads * splits * 2, device=DEV))
-    if mode in ("tiles", "tiles2", "block"):
+    if mode in ("tiles", "tiles2", "block", "block2"):
         group = heads // kv_heads
-        rpt = rows_per_tile or {"tiles": 16, "tiles2": 32, "block": 64}[mode] // min(group, 16)
+        rpt = rows_per_tile or {"tiles": 16, "tiles2": 32, "block": 64, "block2": 128}[mode] // min(group, 16)
         items, i = [], 0
         while i < T:   # consecutive rows of one segment with consecutive positions form a tile
             n = 1
@@ -287,7 +287,7 @@ def run_mfma(ops, qt, kt, vt, tables, rows, page_size, mode, splits=1, window=No
         tasks = torch.tensor(items, dtype=torch.int32, device=DEV)
     ops.attention_mfma(qt.reshape(T, heads * dim), heads * dim, kt, vt, tables, seg, pos, out, heads, kv_heads, dim,
                        page_size, window, scale if scale is not None else 1 / math.sqrt(dim), tasks, splits, ws, waves,
-                       block_tiles=(mode == "block"), item_tiles=(2 if mode == "tiles2" else 1))
+                       block_tiles=mode.startswith("block"), item_tiles=(2 if mode in ("tiles2", "block2") else 1))
     return f64(out).reshape(T, heads, dim)
 
 
@@ -341,10 +341,15 @@ def test_attention_mfma_tiles(ops, heads, kv_heads, dim, page_size):
         np.testing.assert_allclose(got, want, **MFMA_TOL)
         got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, "tiles2", rows_per_tile=2)
         np.testing.assert_allclose(got, want, **MFMA_TOL)
-    got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, "block")                    # 64-item tiles through LDS
-    np.testing.assert_allclose(got, want, **MFMA_TOL)
-    got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, "block", rows_per_tile=3)
-    np.testing.assert_allclose(got, want, **MFMA_TOL)
+    if dim > 128:                                                                        # block tiles: head sizes up to 128
+        with pytest.raises(ops.KernelError):
+            run_mfma(ops, qt, kt, vt, tables, rows, page_size, "block")
+        return
+    for mode in ("block", "block2"):                                                     # 64 / 128-item tiles through LDS
+        got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, mode)
+        np.testing.assert_allclose(got, want, **MFMA_TOL, err_msg=mode)
+        got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, mode, rows_per_tile=3)
+        np.testing.assert_allclose(got, want, **MFMA_TOL, err_msg=mode)
 
 
 def test_attention_mfma_window_and_far_key(ops):
@@ -353,6 +358,7 @@ def test_attention_mfma_window_and_far_key(ops):
         want = reference_attention(qt, kt, vt, tables, rows, 8, window=window)
         np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables, rows, 8, "tiles", window=window), want, **MFMA_TOL)
         np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables, rows, 8, "block", window=window), want, **MFMA_TOL)
+        np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables, rows, 8, "block2", window=window), want, **MFMA_TOL)
         np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables, rows, 8, "tiles2", window=window), want, **MFMA_TOL)
         np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables, rows, 8, "rows", 2, window=window), want, **MFMA_TOL)
     want = reference_attention(qt, kt, vt, tables, rows, 8, scale=0.3)
@@ -362,11 +368,12 @@ def test_attention_mfma_window_and_far_key(ops):
     want = reference_attention(qt, kt, vt, tables, rows, 8, window=8)
     np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables2, rows, 8, "tiles", window=8), want, **MFMA_TOL)
     np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables2, rows, 8, "block", window=8), want, **MFMA_TOL)
+    np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables2, rows, 8, "block2", window=8), want, **MFMA_TOL)
     np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables2, rows, 8, "rows", 3, window=8), want, **MFMA_TOL)
     # one far key among hundreds stands out
     qt, kt, vt, tables, rows = paged_case(4, 2, 64, 16, [700, 40], torch.bfloat16, seed=5, sharpen=(0, 3))
     want = reference_attention(qt, kt, vt, tables, rows, 16)
-    for mode, splits in (("rows", 1), ("rows", 8), ("tiles", 1), ("block", 1)):
+    for mode, splits in (("rows", 1), ("rows", 8), ("tiles", 1), ("block", 1), ("block2", 1)):
         np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables, rows, 16, mode, splits), want, **MFMA_TOL)
 
 

@@ -30,8 +30,18 @@ def main():
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--page-size", type=int, default=16)
     ap.add_argument("--points", default="1,64", help="other batch sizes to time (comma separated, empty for none)")
-    ap.add_argument("--execution", default="graph", choices=["graph", "eager"])
+    ap.add_argument("--execution", default=None, choices=["graph", "eager"],
+                    help="default: graph for the decode workload, eager for serving (its step shapes keep changing)")
+    ap.add_argument("--workload", default="decode", choices=["decode", "serving"],
+                    help="decode: fixed batch after whole prompts (the default, timed per step); serving: --requests "
+                         "requests with prompts of 128..--prompt tokens and --new-tokens each through the scheduler")
+    ap.add_argument("--requests", type=int, default=64)
+    ap.add_argument("--new-tokens", type=int, default=256)
+    ap.add_argument("--token-budget", type=int, default=1024)
+    ap.add_argument("--prefill-chunk", type=int, default=512)
     args = ap.parse_args()
+    if args.execution is None:
+        args.execution = "graph" if args.workload == "decode" else "eager"
     if args.gpus != 1:
         print(f"bench.py measures one GPU only; --gpus {args.gpus} is not run")
         return 2
@@ -56,6 +66,8 @@ def main():
     rng = np.random.default_rng(0)
     batches = [args.batch] + [int(b) for b in args.points.split(",") if b]
     need_tokens = max(batches) * args.context
+    if args.workload == "serving":
+        return serving(args, model, full_layers)
     runner = ModelRunner(model, n_pages=-(-need_tokens // args.page_size), page_size=args.page_size,
                          max_requests=max(batches), execution=args.execution)
 
@@ -140,6 +152,57 @@ def main():
                      "frac": round(achieved / HBM_GBPS, 5)},
         "points": points,
         "reference_b1_tokens_per_s": REFERENCE_B1_TOKS,
+    }
+    print(json.dumps(line))
+    return 0
+
+
+def serving(args, model, full_layers):
+    """Continuous batching: every request is submitted at once, the scheduler admits, cuts prompts into
+    portions under the token budget, decodes and frees.  One JSON line: generated tokens a second."""
+    import numpy as np
+    import torch
+    from runtime.engine import ModelRunner
+    from runtime.engine.scheduler import Engine, Request
+    c = model.config
+    rng = np.random.default_rng(0)
+    lengths = rng.integers(128, args.prompt + 1, size=args.requests).tolist()
+    pages = sum(-(-(n + args.new_tokens) // args.page_size) for n in lengths) + 8
+    runner = ModelRunner(model, n_pages=pages, page_size=args.page_size, max_requests=args.requests, execution=args.execution)
+    engine = Engine(runner, max_active=args.requests, token_budget=args.token_budget, prefill_chunk=args.prefill_chunk,
+                    policy="decode_first")
+    # warm-up: a short run of the same shape of work compiles nothing new but fills the workspace
+    for i in range(2):
+        engine.submit(Request(f"warm{i}", rng.integers(0, c.vocab_size, size=args.prefill_chunk + 3).tolist(), 4))
+    engine.run()
+    for i, n in enumerate(lengths):
+        engine.submit(Request(f"r{i}", rng.integers(0, c.vocab_size, size=n).tolist(), args.new_tokens))
+    torch.cuda.synchronize()
+    ticks0 = len(engine.trace)
+    t0 = time.perf_counter()
+    done = engine.run()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    reqs = [r for r in done if r.key.startswith("r")]
+    generated = sum(len(r.generated) for r in reqs)
+    assert all(r.status == "finished" and len(r.generated) == args.new_tokens for r in reqs)
+    ticks = len(engine.trace) - ticks0
+    ttft = sorted(r.first_token_at - t0 for r in reqs)
+    line = {
+        "metric": f"generated tokens/s, {args.model} layer sizes, {args.requests} requests at once, prompts of 128..{args.prompt} "
+                  f"tokens, {args.new_tokens} new tokens each, continuous batching",
+        "value": round(generated / elapsed, 1), "unit": "tokens/s", "n_gpus": 1, "steps": ticks, "warmup": 0,
+        "ms_per_step": round(elapsed / ticks * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic (random weights N(0,0.02), uniform-random token ids)",
+        "config": {"model": args.model, "global_batch": args.requests, "seq_len": args.prompt + args.new_tokens,
+                   "parallelism": "single-gpu", "layers": c.num_hidden_layers, "layers_of_configuration": full_layers,
+                   "hidden": c.hidden_size, "heads": c.num_attention_heads, "kv_heads": c.num_key_value_heads,
+                   "head_dim": c.head_dim, "intermediate": c.intermediate_size, "vocab": c.vocab_size,
+                   "token_budget": args.token_budget, "prefill_chunk": args.prefill_chunk, "page_size": args.page_size,
+                   "execution": args.execution},
+        "serving": {"seconds": round(elapsed, 3), "prompt_tokens": int(sum(lengths)), "generated_tokens": generated,
+                    "all_tokens_per_s": round((sum(lengths) + generated) / elapsed, 1),
+                    "ttft_median_ms": round(ttft[len(ttft) // 2] * 1e3, 1), "ttft_last_ms": round(ttft[-1] * 1e3, 1)},
     }
     print(json.dumps(line))
     return 0

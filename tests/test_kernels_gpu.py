@@ -413,6 +413,15 @@ def test_gemm_skinny_and_fused_swiglu(ops):
     full = ops.gemm(a, w, torch.empty(64, 300, device=DEV))
     for m in (1, 5, 16, 17, 48):
         assert torch.equal(ops.gemm(a[:m].contiguous(), w, torch.empty(m, 300, device=DEV)), full[:m])
+    # a wide output with more than 32 rows runs with eight waves a block instead of sixteen, which changes the
+    # order of the sum over K: bit for bit among such batches, and to rounding against the smaller ones
+    a, w = rnd(64, 200, dtype=torch.bfloat16, seed=8), rnd(6400, 200, dtype=torch.bfloat16, seed=9)
+    small = ops.gemm(a[:32].contiguous(), w, torch.empty(32, 6400, device=DEV))
+    large = ops.gemm(a, w, torch.empty(64, 6400, device=DEV))
+    assert torch.equal(ops.gemm(a[:7].contiguous(), w, torch.empty(7, 6400, device=DEV)), small[:7])
+    assert torch.equal(ops.gemm(a[:40].contiguous(), w, torch.empty(40, 6400, device=DEV)), large[:40])
+    torch.testing.assert_close(small, large[:32], rtol=1e-5, atol=1e-4)
+    np.testing.assert_allclose(f64(large), f64(a) @ f64(w).T, rtol=1e-4, atol=1e-4 * math.sqrt(200))
 
 
 def test_fused_norm_products(ops):

@@ -45,7 +45,8 @@ class ModelRunner:
     def __init__(self, model, n_pages, page_size=16, max_requests=64, device="cuda:0", execution="eager"):
         if not torch.cuda.is_available():
             raise RuntimeError("no GPU: the engine runs on an MI355X only and has no CPU path")
-        ops.lib()  # fail now if the kernel library is missing
+        # fail now if the kernels are missing; a first call builds what this model needs, all at once
+        ops.prepare([need.head_dim for need in model.cache_needs().values() if need is not None], model.dtype)
         if execution not in ("eager", "graph"):
             raise ValueError(f"execution {execution!r} is not eager or graph")
         self.model = model

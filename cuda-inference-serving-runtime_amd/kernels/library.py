@@ -1,9 +1,11 @@
 """Builds and loads the HIP kernel library (gfx950 only).
 
-The sources under ``csrc/`` are compiled with ``hipcc`` into one shared object
-whose file name carries a digest of the sources and flags, so a stale build is
-never loaded.  Loading looks for that file first and compiles only if it is
-missing; compilation prints a line per file so a first call is visibly alive.
+The sources under ``csrc/`` are compiled with ``hipcc`` into shared objects (the
+core, and one per head size of the matrix-core attention, so that a first call
+compiles only what its model needs) whose file names carry a digest of the
+sources and flags, so a stale build is never loaded.  Loading looks for that
+file first and compiles only if it is missing; compilation prints a line per
+file so a first call is visibly alive.
 There is no fallback: if the library cannot be built or loaded, or no GPU is
 present when a kernel is called, an error is raised.
 """
@@ -29,7 +31,10 @@ HIPCC_FLAGS = [
 ]
 
 _lock = threading.Lock()
-_lib = None
+_libs = {}
+
+CORE = "kernels"                                   # everything but the matrix-core attention
+ATTENTION_PADS = (32, 64, 96, 128, 160, 192, 224, 256)
 
 
 class KernelLibraryError(RuntimeError):
@@ -40,14 +45,30 @@ def _log(msg):
     print(f"[runtime.kernels] {msg}", file=sys.stderr, flush=True)
 
 
-def sources():
-    return sorted(CSRC.glob("*.hip"))
+def attention_unit(dpad):
+    return f"attn_d{dpad}"
 
 
-def _digest():
+def units():
+    """The shared objects the kernels are built into: the core, and one per padded head size of the
+    matrix-core attention (a model needs only its own, so a first call compiles only that one)."""
+    return [CORE] + [attention_unit(d) for d in ATTENTION_PADS]
+
+
+def sources(unit=CORE):
+    if unit == CORE:
+        return sorted(p for p in CSRC.glob("*.hip") if not p.name.startswith("attention_mfma_d"))
+    path = CSRC / f"attention_mfma_{unit[len('attn_'):]}.hip"
+    if not path.exists():
+        raise KernelLibraryError(f"no source for kernel unit {unit}")
+    return [path]
+
+
+def _digest(unit):
     h = hashlib.sha256()
     h.update(" ".join(HIPCC_FLAGS).encode())
-    for path in sorted(p for p in CSRC.iterdir() if p.suffix in (".hip", ".h", ".inc")):
+    included = sorted(p for p in CSRC.iterdir() if p.suffix in (".h", ".inc"))
+    for path in sources(unit) + included:
         h.update(path.name.encode())
         h.update(path.read_bytes())
     return h.hexdigest()[:16]
@@ -67,8 +88,8 @@ def _build_dirs():
     yield Path(tempfile.gettempdir()) / f"cisr_amd_build_{os.getuid()}"
 
 
-def library_path(create=False):
-    name = f"libcisr_kernels_{_digest()}.so"
+def library_path(unit=CORE, create=False):
+    name = f"libcisr_{unit}_{_digest(unit)}.so"
     for d in _build_dirs():
         if (d / name).exists():
             return d / name
@@ -97,15 +118,15 @@ def _compile_one(hipcc, src, obj):
     return obj
 
 
-def build(force=False):
-    """Compile every kernel source and link the shared library.  Returns its path."""
-    target = library_path(create=True)
+def build_unit(unit, force=False):
+    """Compile one unit's sources and link its shared object.  Returns its path."""
+    target = library_path(unit, create=True)
     if target.exists() and not force:
         return target
     hipcc = _hipcc()
     work = Path(tempfile.mkdtemp(prefix="obj_", dir=str(target.parent)))
     try:
-        srcs = sources()
+        srcs = sources(unit)
         with ThreadPoolExecutor(max_workers=min(8, len(srcs))) as pool:
             objs = list(pool.map(lambda s: _compile_one(hipcc, s, work / (s.stem + ".o")), srcs))
         tmp = work / target.name
@@ -115,7 +136,7 @@ def build(force=False):
         if proc.returncode != 0:
             raise KernelLibraryError(f"link failed:\n{proc.stdout}\n{proc.stderr}")
         os.replace(tmp, target)  # atomic: a concurrent loader sees the whole file or none
-        for old in target.parent.glob("libcisr_kernels_*.so"):   # builds of other source states
+        for old in target.parent.glob(f"libcisr_{unit}_*.so"):   # builds of other source states
             if old != target:
                 try:
                     old.unlink()
@@ -126,19 +147,42 @@ def build(force=False):
     return target
 
 
-def load():
-    """The loaded library (built at the first call if no current build exists)."""
-    global _lib
+def build(force=False):
+    """Compile every unit (the core and every attention head size).  Returns the core's path."""
+    with ThreadPoolExecutor(max_workers=4) as pool:
+        paths = list(pool.map(lambda u: build_unit(u, force), units()))
+    return paths[0]
+
+
+def ensure(wanted):
+    """Build the units of `wanted` that have no current build, side by side."""
+    missing = [u for u in dict.fromkeys(wanted) if library_path(u) is None]
+    if missing:
+        with ThreadPoolExecutor(max_workers=len(missing)) as pool:
+            list(pool.map(build_unit, missing))
+
+
+def load(unit=CORE):
+    """The loaded shared object of a unit (built at the first call if no current build exists)."""
     with _lock:
-        if _lib is None:
-            path = library_path() or build()
+        handle = _libs.get(unit)
+        if handle is None:
+            path = library_path(unit) or build_unit(unit)
             try:
-                _lib = ctypes.CDLL(str(path))
+                handle = ctypes.CDLL(str(path))
             except OSError as exc:
                 raise KernelLibraryError(f"cannot load {path}: {exc}") from exc
-            _lib._cisr_path = str(path)
-        return _lib
+            handle._cisr_path = str(path)
+            _libs[unit] = handle
+        return handle
 
 
-def loaded_path():
-    return None if _lib is None else _lib._cisr_path
+def load_attention(dpad):
+    if dpad not in ATTENTION_PADS:
+        raise KernelLibraryError(f"no matrix-core attention for a padded head size of {dpad}")
+    return load(attention_unit(dpad))
+
+
+def loaded_path(unit=CORE):
+    handle = _libs.get(unit)
+    return None if handle is None else handle._cisr_path

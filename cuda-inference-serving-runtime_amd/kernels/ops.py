@@ -13,7 +13,7 @@ import torch
 from . import library
 
 F32, BF16 = 0, 1
-MFMA_HEAD_PADS = (32, 64, 96, 128, 160, 192, 224, 256)
+MFMA_HEAD_PADS = library.ATTENTION_PADS
 SKINNY_ROWS = 64   # products with at most this many rows run the weight-streaming kernel
 _DT = {torch.float32: F32, torch.bfloat16: BF16}
 
@@ -55,12 +55,36 @@ def _declare(h):
         "cisr_argmax": [p, p, p, p, i, i, p],
         "cisr_sample": [p, p, p, p, p, i, i, p],
     }
-    for d in MFMA_HEAD_PADS:
-        sig[f"cisr_attn_mfma_d{d}"] = [p, i, p, p, p, i, p, i, p, p, p, p, p, i, i, i, i, i, f, i, i, i, p]
     for name, args in sig.items():
         fn = getattr(h, name)
         fn.argtypes = args
         fn.restype = C.c_int
+
+
+_attention_entries = {}
+
+
+def _attention_entry(dpad):
+    """The matrix-core attention entry point for a padded head size (its shared object is built and loaded
+    at the first use of that size)."""
+    fn = _attention_entries.get(dpad)
+    if fn is None:
+        p, i, f = C.c_void_p, C.c_int, C.c_float
+        fn = getattr(library.load_attention(dpad), f"cisr_attn_mfma_d{dpad}")
+        fn.argtypes = [p, i, p, p, p, i, p, i, p, p, p, p, p, i, i, i, i, i, f, i, i, i, p]
+        fn.restype = C.c_int
+        _attention_entries[dpad] = fn
+    return fn
+
+
+def prepare(head_dims=(), dtype=None):
+    """Build, side by side, whatever a model with these attention head sizes will load: the core, and for
+    bfloat16 the matrix-core attention of each head size that it supports."""
+    wanted = [library.CORE]
+    if dtype == torch.bfloat16:
+        wanted += [library.attention_unit(-(-d // 32) * 32) for d in head_dims if d % 8 == 0 and 0 < d <= 256]
+    library.ensure(wanted)
+    lib()
 
 
 def _stream():
@@ -400,7 +424,7 @@ def attention_mfma(q, q_row_stride, kcache, vcache, tables, seg_of_row, position
     if kcache.numel() >= 2 ** 32 or vcache.numel() >= 2 ** 32:
         raise KernelError("attention_mfma: a layer's keys (or values) must be fewer than 2^32 elements (32-bit offsets)")
     dpad = -(-dim // 32) * 32
-    fn = getattr(lib(), f"cisr_attn_mfma_d{dpad}")
+    fn = _attention_entry(dpad)
     po = pm = tp = None
     if tasks is not None:
         if item_tiles not in (1, 2) or (item_tiles == 2 and dim > 64 and not block_tiles):

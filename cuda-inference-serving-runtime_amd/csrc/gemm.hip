@@ -109,9 +109,16 @@ __device__ __forceinline__ u32x4 load_chunk(const bf16_t* base, int ld, int row,
     return v;
 }
 
-// Block tile (32 TM) x (32 TN), BK deep; four waves as 2 x 2, each wave TM x TN tiles of 16 x 16.
-// Operands go global memory -> registers -> LDS -> matrix-core operands.  Rows in LDS are padded by 8
-// elements (rows stay 16-byte aligned, a wave's 16-byte operand reads spread over the banks).
+// Side of the patches in which tiles are numbered: `tiles` cut into the fewest parts of at most 8, evenly.
+__host__ __device__ inline int patch_side(int tiles) {
+    const int parts = (tiles + 7) / 8;
+    return (tiles + parts - 1) / parts;
+}
+
+// Block tile (16 WM TM) x (32 TN), BK deep; WM x 2 waves (WM = 2 or 4), each wave TM x TN tiles of 16 x 16.
+// The larger the block tile, the fewer bytes come from L2 per product: 128 x 128 is bound by the L2 at about
+// a third of the matrix cores' peak, 256 x 128 moves a quarter less.
+// Operands go global memory -> registers -> LDS -> matrix-core operands.
 // The pipeline hides the global-memory latency inside one block, because small problems leave a
 // compute unit with a single block: PF tiles of global loads are in flight in a ring of registers,
 // and two LDS buffers let the next tile be written while the current one is multiplied, with one
@@ -120,33 +127,46 @@ __device__ __forceinline__ u32x4 load_chunk(const bf16_t* base, int ld, int row,
 // column tiles take gate rows and its last TN/2 the up rows of the same output columns, so a lane ends
 // with gate and up of one output element in its registers and writes silu(gate) * up (both rounded to
 // bf16 first, as the two-kernel path does); a block then covers BN/2 output columns.
-template <int TM, int TN, int BK, typename TC, bool VEC, bool SWIGLU = false>
-__global__ void __launch_bounds__(256)
+template <int TM, int TN, int BK, typename TC, bool VEC, bool SWIGLU = false, int WM = 2>
+__global__ void __launch_bounds__(WM * 128)
 gemm_bf16_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, int ldw,
                  TC* C, int ldc, const float* R, int ldr, int M, int N, int K, int dual_off = 0) {
     static_assert(!SWIGLU || (TN % 2 == 0 && VEC), "the activation pairs column tiles");
-    constexpr int BM = 2 * TM * 16, BN = 2 * TN * 16;
+    constexpr int BM = WM * TM * 16, BN = 2 * TN * 16, NT = WM * 128;   // WM x 2 waves
     constexpr int BN_OUT = SWIGLU ? BN / 2 : BN;           // output columns a block covers
-    constexpr int STRIDE = BK + 8;
     constexpr int CPR = BK / 8;                            // 16-byte chunks per tile row
-    static_assert((BM * CPR) % 256 == 0 && (BN * CPR) % 256 == 0, "a tile is a whole number of 16-byte chunks per thread");
-    constexpr int A_PER_THREAD = BM * CPR / 256;
-    constexpr int W_PER_THREAD = BN * CPR / 256;
+    // LDS rows are not padded; the 16-byte chunks of a row are permuted by a function of the row instead,
+    // so that neither the copies into LDS (consecutive chunks of a few rows) nor the operand reads (one
+    // chunk of 16 consecutive rows) meet in a bank
+    auto lds_at = [](int row, int chunk) {
+        const int turn = BK == 32 ? ((row >> 1) ^ (row >> 3)) : (row ^ (row >> 3));
+        return row * BK + ((chunk ^ turn) & (CPR - 1)) * 8;
+    };
+    static_assert((BM * CPR) % NT == 0 && (BN * CPR) % NT == 0, "a tile is a whole number of 16-byte chunks per thread");
+    constexpr int A_PER_THREAD = BM * CPR / NT;
+    constexpr int W_PER_THREAD = BN * CPR / NT;
     constexpr int PF = 3;                                  // tiles of global loads in flight
-    __shared__ __attribute__((aligned(16))) bf16_t As[2][BM * STRIDE];
-    __shared__ __attribute__((aligned(16))) bf16_t Ws[2][BN * STRIDE];
+    __shared__ __attribute__((aligned(16))) bf16_t As[2][BM * BK];
+    __shared__ __attribute__((aligned(16))) bf16_t Ws[2][BN * BK];
 
     const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
     const int wm = wave / 2, wn = wave % 2;
     const int r = lane % 16, g = lane / 16;
-    // The hardware deals consecutive workgroups round-robin to the 8 XCDs, each with an L2 of its
-    // own.  Renumber so that an XCD gets a contiguous run of tiles (column tiles fastest): it then
-    // touches one band of A rows instead of all of A, and W stays in its L2 across the band.
-    const int tiles_n = (N + BN_OUT - 1) / BN_OUT, tiles = tiles_n * ((M + BM - 1) / BM);
-    const int per_xcd = (tiles + 7) / 8;
-    const int tile = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
-    if (tile >= tiles) return;   // the grid is rounded up to a multiple of 8
-    const int m0 = (tile / tiles_n) * BM, n0 = (tile % tiles_n) * BN_OUT;
+    // The hardware deals consecutive workgroups round-robin to the 8 XCDs, each with an L2 of its own.
+    // Renumber so that an XCD gets a contiguous run of tiles, and order the tiles in patches of up to
+    // 8 x 8 (sides as even as the tile counts allow, so that few slots fall outside the matrix): the sixty-odd blocks that run on an XCD at one time then share 8 row bands of A and 8 of W
+    // (16 bands from memory for 64 tiles) instead of one band of A and 64 of W.
+    const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN_OUT - 1) / BN_OUT;
+    const int gm = patch_side(tiles_m), gn = patch_side(tiles_n);
+    const int patches_n = (tiles_n + gn - 1) / gn, patches = ((tiles_m + gm - 1) / gm) * patches_n;
+    const int slots = patches * gm * gn;                   // tile slots (those outside the matrix do nothing)
+    const int per_xcd = (slots + 7) / 8;
+    const int slot = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    if (slot >= slots) return;                             // the grid is rounded up to a multiple of 8
+    const int patch = slot / (gm * gn), in_patch = slot % (gm * gn);
+    const int tile_m = (patch / patches_n) * gm + in_patch % gm, tile_n = (patch % patches_n) * gn + in_patch / gm;
+    if (tile_m >= tiles_m || tile_n >= tiles_n) return;
+    const int m0 = tile_m * BM, n0 = tile_n * BN_OUT;
 
     f32x4 acc[TM][TN];
 #pragma unroll
@@ -158,12 +178,12 @@ gemm_bf16_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict
     auto fetch = [&](int k0, u32x4 (&fa)[A_PER_THREAD], u32x4 (&fw)[W_PER_THREAD]) {
 #pragma unroll
         for (int i = 0; i < A_PER_THREAD; ++i) {
-            const int c = tid + i * 256;
+            const int c = tid + i * NT;
             fa[i] = load_chunk<VEC>(A, lda, m0 + c / CPR, M, k0 + (c % CPR) * 8, K);
         }
 #pragma unroll
         for (int i = 0; i < W_PER_THREAD; ++i) {
-            const int c = tid + i * 256;
+            const int c = tid + i * NT;
             if (SWIGLU) {
                 // local column -> (wave, column tile, column): the W row of its output column, gate or up
                 const int lc = c / CPR, jj = (lc % (TN * 16)) / 16;
@@ -187,16 +207,16 @@ gemm_bf16_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict
                 ++it;
 #pragma unroll
                 for (int i = 0; i < A_PER_THREAD; ++i) {
-                    const int c = tid + i * 256;
+                    const int c = tid + i * NT;
                     const uint32_t keep = (VEC && kk0 + (c % CPR) * 8 >= K) ? 0u : 0xffffffffu;
                     u32x4 v = ra[s][i];
                     v.x &= keep; v.y &= keep; v.z &= keep; v.w &= keep;
-                    *(u32x4*)(&As[buf][(c / CPR) * STRIDE + (c % CPR) * 8]) = v;
+                    *(u32x4*)(&As[buf][lds_at(c / CPR, c % CPR)]) = v;
                 }
 #pragma unroll
                 for (int i = 0; i < W_PER_THREAD; ++i) {
-                    const int c = tid + i * 256;
-                    *(u32x4*)(&Ws[buf][(c / CPR) * STRIDE + (c % CPR) * 8]) = rw[s][i];   // A is zero there: enough
+                    const int c = tid + i * NT;
+                    *(u32x4*)(&Ws[buf][lds_at(c / CPR, c % CPR)]) = rw[s][i];   // A is zero there: enough
                 }
                 // one barrier a tile: whoever writes this buffer again (two tiles on) has passed
                 // the next tile's barrier, which every wave reaches only after reading this one
@@ -207,10 +227,10 @@ gemm_bf16_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict
                     bf16x8 fa[TM], fw[TN];
 #pragma unroll
                     for (int i = 0; i < TM; ++i)
-                        fa[i] = *(const bf16x8*)(&As[buf][(wm * TM * 16 + i * 16 + r) * STRIDE + kk + g * 8]);
+                        fa[i] = *(const bf16x8*)(&As[buf][lds_at(wm * TM * 16 + i * 16 + r, kk / 8 + g)]);
 #pragma unroll
                     for (int j = 0; j < TN; ++j)
-                        fw[j] = *(const bf16x8*)(&Ws[buf][(wn * TN * 16 + j * 16 + r) * STRIDE + kk + g * 8]);
+                        fw[j] = *(const bf16x8*)(&Ws[buf][lds_at(wn * TN * 16 + j * 16 + r, kk / 8 + g)]);
 #pragma unroll
                     for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -269,34 +289,40 @@ gemm_bf16_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict
     }
 }
 
-template <int TM, int TN, int BK>
+// tile slots of the kernel's patch numbering (whole patches)
+static long long tile_slots(long long tiles_m, long long tiles_n) {
+    const long long gm = patch_side((int)tiles_m), gn = patch_side((int)tiles_n);
+    return ((tiles_m + gm - 1) / gm) * ((tiles_n + gn - 1) / gn) * gm * gn;
+}
+
+template <int TM, int TN, int BK, int WM = 2>
 static int launch_bf16(const bf16_t* A, int lda, const bf16_t* W, int ldw, void* C, int ldc, const float* R,
                        int ldr, int M, int N, int K, int out_dtype, hipStream_t stream) {
-    constexpr int BM = 2 * TM * 16, BN = 2 * TN * 16;
-    const long long tiles = (long long)((N + BN - 1) / BN) * ((M + BM - 1) / BM);
-    if (tiles > (1ll << 30)) return (int)hipErrorInvalidValue;
-    dim3 grid((unsigned)((tiles + 7) / 8 * 8));
+    constexpr int BM = WM * TM * 16, BN = 2 * TN * 16, NT = WM * 128;
+    const long long slots = tile_slots((M + BM - 1) / BM, (N + BN - 1) / BN);
+    if (slots > (1ll << 30)) return (int)hipErrorInvalidValue;
+    dim3 grid((unsigned)((slots + 7) / 8 * 8));
     const bool vec = lda % 8 == 0 && ldw % 8 == 0 && K % 8 == 0 && ((uintptr_t)A) % 16 == 0 && ((uintptr_t)W) % 16 == 0;
     if (out_dtype == DT_F32) {
-        if (vec) gemm_bf16_kernel<TM, TN, BK, float, true><<<grid, 256, 0, stream>>>(A, lda, W, ldw, (float*)C, ldc, R, ldr, M, N, K);
-        else gemm_bf16_kernel<TM, TN, BK, float, false><<<grid, 256, 0, stream>>>(A, lda, W, ldw, (float*)C, ldc, R, ldr, M, N, K);
+        if (vec) gemm_bf16_kernel<TM, TN, BK, float, true, false, WM><<<grid, NT, 0, stream>>>(A, lda, W, ldw, (float*)C, ldc, R, ldr, M, N, K);
+        else gemm_bf16_kernel<TM, TN, BK, float, false, false, WM><<<grid, NT, 0, stream>>>(A, lda, W, ldw, (float*)C, ldc, R, ldr, M, N, K);
     } else {
-        if (vec) gemm_bf16_kernel<TM, TN, BK, bf16_t, true><<<grid, 256, 0, stream>>>(A, lda, W, ldw, (bf16_t*)C, ldc, R, ldr, M, N, K);
-        else gemm_bf16_kernel<TM, TN, BK, bf16_t, false><<<grid, 256, 0, stream>>>(A, lda, W, ldw, (bf16_t*)C, ldc, R, ldr, M, N, K);
+        if (vec) gemm_bf16_kernel<TM, TN, BK, bf16_t, true, false, WM><<<grid, NT, 0, stream>>>(A, lda, W, ldw, (bf16_t*)C, ldc, R, ldr, M, N, K);
+        else gemm_bf16_kernel<TM, TN, BK, bf16_t, false, false, WM><<<grid, NT, 0, stream>>>(A, lda, W, ldw, (bf16_t*)C, ldc, R, ldr, M, N, K);
     }
     return CISR_LAUNCH_CHECK();
 }
 
 // C[M, N] = silu(A . Wg^T) * (A . Wu^T), W = [Wg; Wu] with `dual_off` rows between the blocks; bf16 in and out,
 // 16-byte aligned rows with K % 8 == 0.
-template <int TM, int TN, int BK>
+template <int TM, int TN, int BK, int WM = 2>
 static int launch_bf16_swiglu(const bf16_t* A, int lda, const bf16_t* W, int ldw, bf16_t* C, int ldc, int M, int N, int K,
                               int dual_off, hipStream_t stream) {
-    constexpr int BM = 2 * TM * 16, BN_OUT = TN * 16;
-    const long long tiles = (long long)((N + BN_OUT - 1) / BN_OUT) * ((M + BM - 1) / BM);
-    if (tiles > (1ll << 30)) return (int)hipErrorInvalidValue;
-    dim3 grid((unsigned)((tiles + 7) / 8 * 8));
-    gemm_bf16_kernel<TM, TN, BK, bf16_t, true, true><<<grid, 256, 0, stream>>>(A, lda, W, ldw, C, ldc, nullptr, 0, M, N, K, dual_off);
+    constexpr int BM = WM * TM * 16, BN_OUT = TN * 16;
+    const long long slots = tile_slots((M + BM - 1) / BM, (N + BN_OUT - 1) / BN_OUT);
+    if (slots > (1ll << 30)) return (int)hipErrorInvalidValue;
+    dim3 grid((unsigned)((slots + 7) / 8 * 8));
+    gemm_bf16_kernel<TM, TN, BK, bf16_t, true, true, WM><<<grid, WM * 128, 0, stream>>>(A, lda, W, ldw, C, ldc, nullptr, 0, M, N, K, dual_off);
     return CISR_LAUNCH_CHECK();
 }
 
@@ -307,7 +333,7 @@ extern "C" int cisr_gemm_bf16_swiglu(const void* A, int lda, const void* W, int 
         return (int)hipErrorInvalidValue;
     const bf16_t* a = (const bf16_t*)A; const bf16_t* w = (const bf16_t*)W;
     auto blocks = [&](int bm, int bn) { return (long long)((M + bm - 1) / bm) * ((2 * N + bn - 1) / bn); };
-    if (blocks(128, 128) >= 512) return launch_bf16_swiglu<4, 4, 32>(a, lda, w, ldw, (bf16_t*)C, ldc, M, N, K, dual_off, stream);
+    if (blocks(128, 128) >= 512) return launch_bf16_swiglu<4, 4, 64>(a, lda, w, ldw, (bf16_t*)C, ldc, M, N, K, dual_off, stream);
     if (blocks(128, 64) >= 512) return launch_bf16_swiglu<4, 2, 64>(a, lda, w, ldw, (bf16_t*)C, ldc, M, N, K, dual_off, stream);
     return launch_bf16_swiglu<2, 2, 64>(a, lda, w, ldw, (bf16_t*)C, ldc, M, N, K, dual_off, stream);
 }
@@ -320,7 +346,7 @@ extern "C" int cisr_gemm_bf16(const void* A, int lda, const void* W, int ldw, vo
     const bf16_t* a = (const bf16_t*)A; const bf16_t* w = (const bf16_t*)W;
     auto blocks = [&](int bm, int bn) { return (long long)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
     if (M <= 32) return launch_bf16<1, 2, 64>(a, lda, w, ldw, C, ldc, R, ldr, M, N, K, out_dtype, stream);
-    if (blocks(128, 128) >= 512) return launch_bf16<4, 4, 32>(a, lda, w, ldw, C, ldc, R, ldr, M, N, K, out_dtype, stream);
+    if (blocks(128, 128) >= 512) return launch_bf16<4, 4, 64>(a, lda, w, ldw, C, ldc, R, ldr, M, N, K, out_dtype, stream);
     if (blocks(128, 64) >= 512) return launch_bf16<4, 2, 64>(a, lda, w, ldw, C, ldc, R, ldr, M, N, K, out_dtype, stream);
     return launch_bf16<2, 2, 64>(a, lda, w, ldw, C, ldc, R, ldr, M, N, K, out_dtype, stream);
 }

@@ -61,9 +61,12 @@ class StepContext:
         self.span_hint = 0        # host: context length that sizes attention launches (a bucket under capture)
         self.tasks = {}           # rows per tile -> int32 [n, 4] task list on the device
         self.capturing = False    # the step is being recorded into a graph: launches only
+        self.owner = None         # key of the captured program this step belongs to, if any
 
     def buffer(self, name, shape, dtype):
-        return self.runner.workspace.get(name, shape, dtype)
+        """A device buffer for an intermediate result of this step (stable across the replays of a
+        captured program; otherwise valid until the next step)."""
+        return self.runner.workspace.get(name, shape, dtype, owner=self.owner)
 
     def attention_tasks(self, rows_per_tile):
         """int32 [n, 4] on the device: (segment, first row, rows, 0) for tiles of at most
@@ -89,31 +92,48 @@ class StepContext:
 
 
 class Workspace:
-    """Named device buffers with stable addresses, one per (name, shape, dtype)."""
+    """Named device buffers for a step's intermediate results.
+
+    A captured program needs buffers whose addresses never change: it asks with its key as `owner` and gets
+    one buffer per (name, shape, dtype), shared with every other program that asks for the same; a buffer
+    lives until its last owner is released.  Steps that are not captured (owner None) share one buffer per
+    name that only grows, and get a view of its first rows."""
 
     def __init__(self, device):
         self.device = device
-        self.buffers = {}
+        self.owned = {}      # (name, shape, dtype) -> [tensor, set of owners]
+        self.growing = {}    # (name, trailing shape, dtype) -> tensor
 
-    def get(self, name, shape, dtype):
-        key = (name, tuple(shape), dtype)
-        buf = self.buffers.get(key)
-        if buf is None:
-            buf = torch.empty(tuple(shape), dtype=dtype, device=self.device)
-            self.buffers[key] = buf
-        return buf
+    def get(self, name, shape, dtype, owner=None, zeroed=False):
+        shape = tuple(int(d) for d in shape)
+        make = torch.zeros if zeroed else torch.empty
+        if owner is not None:
+            entry = self.owned.get((name, shape, dtype))
+            if entry is None:
+                entry = self.owned[(name, shape, dtype)] = [make(shape, dtype=dtype, device=self.device), set()]
+            entry[1].add(owner)
+            return entry[0]
+        key = (name, shape[1:], dtype)
+        buf = self.growing.get(key)
+        if buf is None or buf.shape[0] < shape[0]:
+            rows = shape[0] if buf is None else max(shape[0], buf.shape[0] * 3 // 2)
+            # the old buffer goes back to the allocator, which hands it out again only behind the work
+            # already queued on this stream
+            buf = self.growing[key] = make((rows, *shape[1:]), dtype=dtype, device=self.device)
+        return buf[:shape[0]]
 
-    def get_zeroed(self, name, shape, dtype):
-        """A buffer that is zero when first handed out; its users leave it zero."""
-        key = (name, tuple(shape), dtype)
-        buf = self.buffers.get(key)
-        if buf is None:
-            buf = torch.zeros(tuple(shape), dtype=dtype, device=self.device)
-            self.buffers[key] = buf
-        return buf
+    def release(self, owner):
+        """Forget a program: buffers that no other program uses are freed."""
+        for key in [k for k, (_, owners) in self.owned.items() if owner in owners]:
+            owners = self.owned[key][1]
+            owners.discard(owner)
+            if not owners:
+                del self.owned[key]
 
     def bytes(self):
-        return sum(b.numel() * b.element_size() for b in self.buffers.values())
+        tensors = [t for t, _ in self.owned.values()] + list(self.growing.values())
+        return sum(t.numel() * t.element_size() for t in tensors)
 
     def clear(self):
-        self.buffers.clear()
+        self.owned.clear()
+        self.growing.clear()

@@ -256,6 +256,7 @@ class ModelRunner:
                 oldest = next(iter(self.programs))
                 torch.cuda.synchronize()
                 del self.programs[oldest]
+                self.workspace.release(oldest)
         else:
             self.programs[key] = self.programs.pop(key)  # most recently used last
         if program["tilings"] != self.task_tilings:
@@ -264,6 +265,7 @@ class ModelRunner:
             program.update(meta=torch.zeros(int(self._layout(T, S, R)[-1]), dtype=torch.int32, device=self.device),
                            graph=None, runs=0, tilings=list(self.task_tilings))
         ctx = self._context(entries, done, pad=(T, S, R), device_buffer=program["meta"])
+        ctx.owner = key
         ctx.span_hint = context   # launch shapes inside a captured program depend on the key only
         ctx.decode_only = decode_only
         if program["graph"] is None and program["runs"] >= 1 and program["tilings"] == self.task_tilings:

@@ -34,3 +34,27 @@ def test_task_lists_cover_every_row_once_and_never_cross_a_segment():
 def test_program_sizes_are_powers_of_two_then_multiples_of_64():
     assert [_bucket(n) for n in (0, 1, 2, 3, 5, 33, 64, 65, 128, 129, 2048)] == [0, 1, 2, 4, 8, 64, 64, 128, 128, 192, 2048]
     assert all(_bucket(n) >= n for n in range(1, 500))
+
+
+def test_workspace_buffers_are_stable_for_programs_and_bounded_for_other_steps():
+    import torch
+    from runtime.engine.context import Workspace
+    ws = Workspace(torch.device("cpu"))
+    # captured programs: the same tensor for the same (name, shape, dtype), alive until its last owner goes
+    a = ws.get("x", (4, 8), torch.float32, owner="p1")
+    assert ws.get("x", (4, 8), torch.float32, owner="p1") is a
+    assert ws.get("x", (4, 8), torch.float32, owner="p2") is a
+    b = ws.get("x", (6, 8), torch.float32, owner="p2")
+    assert b is not a and b.shape == (6, 8)
+    ws.release("p1")
+    assert ws.get("x", (4, 8), torch.float32, owner="p2") is a
+    ws.release("p2")
+    assert ws.bytes() == 0
+    # other steps: one buffer per name that only grows; smaller requests are views of it
+    big = ws.get("y", (10, 3), torch.float32)
+    small = ws.get("y", (4, 3), torch.float32)
+    assert small.shape == (4, 3) and small.is_contiguous() and small.data_ptr() == big.data_ptr()
+    bigger = ws.get("y", (11, 3), torch.float32)
+    assert bigger.shape == (11, 3) and ws.bytes() == 15 * 3 * 4      # grown by half, the old one dropped
+    assert ws.get("y", (2, 5), torch.float32).shape == (2, 5)       # another trailing shape: another buffer
+    assert ws.get("z", (7,), torch.int32, zeroed=True).sum() == 0

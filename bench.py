@@ -30,8 +30,7 @@ def main():
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--page-size", type=int, default=16)
     ap.add_argument("--points", default="1,64", help="other batch sizes to time (comma separated, empty for none)")
-    ap.add_argument("--execution", default=None, choices=["graph", "eager"],
-                    help="default: graph for the decode workload, eager for serving (its step shapes keep changing)")
+    ap.add_argument("--execution", default="graph", choices=["graph", "eager"])
     ap.add_argument("--workload", default="decode", choices=["decode", "serving"],
                     help="decode: fixed batch after whole prompts (the default, timed per step); serving: --requests "
                          "requests with prompts of 128..--prompt tokens and --new-tokens each through the scheduler")
@@ -40,8 +39,6 @@ def main():
     ap.add_argument("--token-budget", type=int, default=1024)
     ap.add_argument("--prefill-chunk", type=int, default=512)
     args = ap.parse_args()
-    if args.execution is None:
-        args.execution = "graph" if args.workload == "decode" else "eager"
     if args.gpus != 1:
         print(f"bench.py measures one GPU only; --gpus {args.gpus} is not run")
         return 2

@@ -52,7 +52,7 @@ class ModelRunner:
         self.model = model
         self.execution = execution
         self.programs, self.program_capacity = {}, 16
-        self.block_tiles = int(os.environ.get("CISR_BLOCK_TILES", "0"))   # long portions: LDS-shared tiles of 64 x this items
+        self.block_tiles = None    # long portions through LDS-shared tiles of 64 x this items: None = by the number of blocks
         self.tile_waves = int(os.environ.get("CISR_TILE_WAVES", "4"))   # wavefronts that share one tile's keys
         self.item_tiles = int(os.environ.get("CISR_ITEM_TILES", "2"))   # 16-item tiles a wave of long portions (small heads)
         self.device = torch.device(device)
@@ -314,11 +314,15 @@ class ModelRunner:
                 ops.attention_mfma(q, q_row_stride, kcache, vcache, view.tables, ctx.seg_of_row, ctx.positions, out,
                                    heads, kv_heads, head_dim, view.page_size, window, scale, None, splits, workspace, waves)
             else:
-                # long portions: the four waves of a block own different rows and share each step's keys and
-                # values through LDS (64 or 128 items a block); otherwise the waves of a block share one tile
-                # of 16 items (32 with small heads) and split its keys
+                # long portions, enough of them to fill the GPU with blocks of 64 items (or 128): the four waves of
+                # a block own different rows and share each step's keys and values through LDS.  Otherwise (few
+                # heads, short portions) the waves of a block share one tile of 16 items (32 with small heads)
+                # and split its keys, which is what hides the latency of a step when blocks are scarce.
                 long_portions = rows >= 16 * ctx.n_segments
-                block_tiles = self.block_tiles if long_portions and head_dim <= 128 else 0
+                block_tiles = 0
+                if long_portions and head_dim <= 128:
+                    blocks = -(-rows // (64 // heads_per_chunk)) * kv_heads * -(-group // heads_per_chunk)
+                    block_tiles = (2 if blocks >= 2048 else 1 if blocks >= 512 else 0) if self.block_tiles is None else self.block_tiles
                 if block_tiles:
                     item_tiles = block_tiles
                     tasks = ctx.attention_tasks(64 * item_tiles // heads_per_chunk)

@@ -143,6 +143,29 @@ def test_captured_prompt_and_mixed_steps_match_the_plain_model(folders, name, dt
     runner.cache.check()
 
 
+@pytest.mark.parametrize("name", ["a", "c"])
+@pytest.mark.parametrize("item_tiles", [1, 2])
+def test_long_portions_through_block_tiles_match_the_plain_model(folders, name, item_tiles):
+    """With many heads and long portions the attention of a prompt step runs in blocks whose waves share keys
+    through LDS; forced here on small models: a whole prompt, then a second portion beside another request."""
+    from runtime.engine import load_model, ModelRunner, StepEntry
+    from conftest import plain_logits, assert_close
+    V = TINY[name]["vocab_size"]
+    model = load_model(folders[name], dtype="bfloat16")
+    runner = ModelRunner(model, n_pages=64, page_size=8, max_requests=4)
+    runner.block_tiles = item_tiles
+    seqs = {k: random_tokens(500 + i, 230, V) for i, k in enumerate("pq")}
+    refs = {k: plain_logits(folders[name], seqs[k]) for k in seqs}
+    for k in seqs:
+        runner.create(k)
+    got = runner.step([StepEntry("p", seqs["p"][:150], list(range(150)))]).float().cpu().numpy()
+    assert_close(got, refs["p"][:150], "bfloat16", "first portion")
+    got = runner.step([StepEntry("p", seqs["p"][150:], list(range(80))),
+                       StepEntry("q", seqs["q"][:97], list(range(97)))]).float().cpu().numpy()
+    assert_close(got[:80], refs["p"][150:], "bfloat16", "second portion on a cached prefix")
+    assert_close(got[80:], refs["q"][:97], "bfloat16", "another request in the same step")
+
+
 def test_temperature_sampling_is_seeded_and_independent_of_the_batch(folders):
     from runtime.engine.scheduler import Engine, Request
     V = TINY["b"]["vocab_size"]

@@ -81,6 +81,8 @@ class CacheGroup:
         self.page_size = page_size
         self.pool = PagePool(n_pages)
         self.tables = {}
+        self.versions = {}   # request -> stamp of the last change of its table (stamps are never reused)
+        self._stamp = 0
         self.storage = None  # device tensor [sites, 2, pages, kv_heads, page_size, head_dim], set by the owner
 
     # -- planning -------------------------------------------------------
@@ -107,12 +109,17 @@ class CacheGroup:
                    if table[j] >= 0 and self.pool.refs[table[j]] == 1)
 
     # -- mutation -------------------------------------------------------
+    def _touch(self, request):
+        self._stamp += 1
+        self.versions[request] = self._stamp
+
     def trim(self, request, length):
         table = self.tables[request]
         for j in range(min(self._dead_pages(request, length), len(table))):
             if table[j] >= 0:
                 self.pool.drop(table[j])
                 table[j] = -1
+                self._touch(request)
 
     def append(self, request, length, n_new):
         """Slots of the n_new tokens at logical positions length.. and the page
@@ -124,21 +131,26 @@ class CacheGroup:
             copies.append((old, new))
             self.pool.drop(old)
             table[-1] = new
+            self._touch(request)
         while len(table) * P < length + n_new:
             table.append(self.pool.allocate())
+            self._touch(request)
         slots = [table[(length + i) // P] * P + (length + i) % P for i in range(n_new)]
         return slots, copies
 
     def create(self, request):
         self.tables[request] = []
+        self._touch(request)
 
     def fork(self, source, target):
         self.tables[target] = list(self.tables[source])
+        self._touch(target)
         for page in self.tables[target]:
             if page >= 0:
                 self.pool.share(page)
 
     def release(self, request):
+        self.versions.pop(request, None)
         for page in self.tables.pop(request):
             if page >= 0:
                 self.pool.drop(page)

@@ -76,6 +76,10 @@ class ModelRunner:
         self.table_width = -(-self.max_context // page_size)
         self._staging = []
         self._staging_next = 0
+        self._layouts = {}
+        # host copies of the block tables by state slot, with the stamp of the table they were made from
+        self._table_mirror = [(np.full((max_requests, self.table_width), -1, dtype=np.int32), [None] * max_requests)
+                              for _ in self.cache.groups]
         self.task_tilings = []   # rows-per-tile values that mixers have asked task lists for
         self.steps = 0
 
@@ -140,62 +144,91 @@ class ModelRunner:
         sizes = [T, T, T, S + 1, S, S, R] + [T, S * W] * G + [4 * (-(-T // r) + S) for r in self.task_tilings]
         return np.concatenate(([0], np.cumsum(sizes))).astype(np.int64)
 
+    def _table_rows(self, g, done):
+        """int32 [len(done), W]: the block tables of the step's requests in group g.  A host copy of every
+        live request's table is kept by state slot and rewritten only when the table has changed (a new
+        page, a page the window has passed, a copy-on-write), so a step costs one gather."""
+        group = self.cache.groups[g]
+        mirror, stamps = self._table_mirror[g]
+        for d in done:
+            stamp = group.versions[d.request]
+            if stamps[d.state_slot] != stamp:
+                table = group.tables[d.request]
+                mirror[d.state_slot, :len(table)] = table
+                mirror[d.state_slot, len(table):] = -1
+                stamps[d.state_slot] = stamp
+        return mirror[[d.state_slot for d in done]]
+
     def _context(self, entries, done, pad=None, device_buffer=None):
         """Build the step's metadata on the host, upload it in one copy and wrap it.
         `pad` = (T, S, R) pads the batch with inert rows (for captured programs):
         token 0 at position 0, no segment, no cache slot."""
-        n_rows = sum(len(e.tokens) for e in entries)
+        counts = [d.count for d in done]
+        starts = [d.start for d in done]
+        n_rows, n_seg = sum(counts), len(entries)
         n_want = sum(len(e.want) for e in entries)
-        T, S, R = pad if pad is not None else (n_rows, len(entries), n_want)
+        T, S, R = pad if pad is not None else (n_rows, n_seg, n_want)
         W, G = self.table_width, len(self.cache.groups)
-        offsets = self._layout(T, S, R)
-        total = int(offsets[-1])
+        layout = (T, S, R, tuple(self.task_tilings))
+        offsets = self._layouts.get(layout)
+        if offsets is None:
+            offsets = self._layouts[layout] = [int(x) for x in self._layout(T, S, R)]
+        total = offsets[-1]
         host = self._stage(total)
         arr = host.numpy()
         tokens, positions, seg_of_row, seg_start, seg_first, state_slots, logit_rows = (
             arr[offsets[i]:offsets[i + 1]] for i in range(7))
-        if pad is not None:
-            tokens[:] = 0
-            positions[:] = 0
-            seg_of_row[:] = -1
-            seg_start[:] = n_rows
-            seg_first[:] = 0
-            state_slots[:] = 0
-            logit_rows[:] = 0
-            for g in range(G):
-                arr[offsets[7 + 2 * g]:offsets[8 + 2 * g]] = -1
-                arr[offsets[8 + 2 * g]:offsets[9 + 2 * g]] = -1
-        row = out_row = max_context = 0
-        for s, (e, d) in enumerate(zip(entries, done)):
-            n = len(e.tokens)
-            tokens[row:row + n] = e.tokens
-            positions[row:row + n] = np.arange(d.start, d.start + n)
-            seg_of_row[row:row + n] = s
-            seg_start[s] = row
-            seg_first[s] = d.start
-            state_slots[s] = d.state_slot
-            for w in e.want:
-                logit_rows[out_row] = row + int(w)
-                out_row += 1
-            for g in range(G):
-                base = 7 + 2 * g
-                arr[offsets[base] + row: offsets[base] + row + n] = d.slots[g]
-                table = self.cache.table(g, e.request)
-                trow = arr[offsets[base + 1] + s * W: offsets[base + 1] + (s + 1) * W]
-                trow[:len(table)] = table
-                trow[len(table):] = -1
-            row += n
-            max_context = max(max_context, d.start + n)
-        seg_start[len(entries):] = n_rows
+        decode_only = n_rows == n_seg
+        if decode_only:
+            first_row = np.arange(n_seg, dtype=np.int32)
+            tokens[:n_rows] = [e.tokens[0] for e in entries]
+            positions[:n_rows] = starts
+            seg_of_row[:n_rows] = first_row
+            wanted = [s for s, e in enumerate(entries) for _ in e.want]
+        else:
+            first_row = np.concatenate(([0], np.cumsum(counts[:-1]))).astype(np.int32)
+            tokens[:n_rows] = np.concatenate([np.asarray(e.tokens, dtype=np.int32) for e in entries])
+            seg_of_row[:n_rows] = np.repeat(np.arange(n_seg, dtype=np.int32), counts)
+            positions[:n_rows] = np.arange(n_rows, dtype=np.int32) + np.repeat(np.asarray(starts, dtype=np.int32) - first_row, counts)
+            wanted = [int(first_row[s]) + int(w) for s, e in enumerate(entries) for w in e.want]
+        seg_start[:n_seg] = first_row
+        seg_start[n_seg:] = n_rows
+        seg_first[:n_seg] = starts
+        state_slots[:n_seg] = [d.state_slot for d in done]
+        logit_rows[:n_want] = wanted
+        if pad is not None:      # the inert rest: token 0 at position 0, no segment, no slot, no table
+            tokens[n_rows:] = 0
+            positions[n_rows:] = 0
+            seg_of_row[n_rows:] = -1
+            seg_first[n_seg:] = 0
+            state_slots[n_seg:] = 0
+            logit_rows[n_want:] = 0
+        for g in range(G):
+            slots = arr[offsets[7 + 2 * g]:offsets[8 + 2 * g]]
+            tables = arr[offsets[8 + 2 * g]:offsets[9 + 2 * g]].reshape(S, W)
+            if decode_only:
+                slots[:n_rows] = [d.slots[g][0] for d in done]
+            else:
+                slots[:n_rows] = np.concatenate([np.asarray(d.slots[g], dtype=np.int32) for d in done])
+            tables[:n_seg] = self._table_rows(g, done)
+            if pad is not None:
+                slots[n_rows:] = -1
+                tables[n_seg:] = -1
         tilings = list(self.task_tilings)
         for i, rows_per_tile in enumerate(tilings):
             tasks = arr[offsets[7 + 2 * G + i]:offsets[8 + 2 * G + i]].reshape(-1, 4)
-            n = fill_tasks(tasks, [d.count for d in done], rows_per_tile, [d.start for d in done])
+            if decode_only:      # one tile of one row a segment
+                n = n_seg
+                tasks[:n, 0] = tasks[:n, 1] = first_row
+                tasks[:n, 2] = 1
+                tasks[:n, 3] = 0
+            else:
+                n = fill_tasks(tasks, counts, rows_per_tile, starts)
             tasks[n:] = (-1, 0, 0, 0)   # tiles of no segment do nothing
         dev = self._upload(host, total, device_buffer)
 
         def view(i, shape=None):
-            t = dev[int(offsets[i]):int(offsets[i + 1])]
+            t = dev[offsets[i]:offsets[i + 1]]
             return t if shape is None else t.view(shape)
 
         ctx = StepContext(self)
@@ -205,8 +238,8 @@ class ModelRunner:
         ctx.kv = [GroupView(view(7 + 2 * g), view(8 + 2 * g, (S, W)), self.page_size, W) for g in range(G)]
         ctx.tasks = {r: view(7 + 2 * G + i, (-1, 4)) for i, r in enumerate(tilings)}
         ctx.segments = [(d.request, d.start, d.count) for d in done]
-        ctx.max_context = ctx.span_hint = max_context
-        ctx.decode_only = all(d.count == 1 for d in done)
+        ctx.max_context = ctx.span_hint = max(s + c for s, c in zip(starts, counts))
+        ctx.decode_only = decode_only
         return ctx
 
     def _stage(self, n):

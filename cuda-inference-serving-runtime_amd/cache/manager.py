@@ -27,6 +27,8 @@ class Appended:
 
 
 class CacheManager:
+    fast_decode = True   # steps of one token a request take a short path (tests switch it off to compare)
+
     def __init__(self, site_needs, n_pages, page_size, max_requests, state_needs=None,
                  allocate_kv=None, allocate_state=None, copy_pages=None, zero_state=None, copy_state=None):
         """site_needs: {site id: KVNeed}; state_needs: {site id: StateNeed}.
@@ -120,6 +122,8 @@ class CacheManager:
             if n <= 0:
                 raise ValueError("a request must bring at least one token")
             seen.add(request)
+        if self.fast_decode and all(n == 1 for _, n in items) and all(g.need.window is None for g in self.groups):
+            return self._append_one_each(items)
         if not self.can_append(items):
             raise OutOfPages("not enough free KV pages for this step")
         result = []
@@ -133,6 +137,36 @@ class CacheManager:
                 if copies and self._copy_pages is not None:
                     self._copy_pages(group, copies)
             self.lengths[request] = length + n
+            result.append(done)
+        return result
+
+    def _append_one_each(self, items):
+        """append_many for the common step in which every request brings one token and no group has a
+        window: the same pages in the same order, with the counting and the placing done in line."""
+        P = self.page_size
+        lengths = self.lengths
+        for group in self.groups:
+            refs, tables, fresh = group.pool.refs, group.tables, 0
+            for request, _ in items:
+                if lengths[request] % P == 0 or refs[tables[request][-1]] > 1:
+                    fresh += 1
+            if fresh > len(group.pool.free):
+                raise OutOfPages("not enough free KV pages for this step")
+        result = []
+        for request, _ in items:
+            length = lengths[request]
+            done = Appended(request, length, 1, state_slot=self.slots.slot_of(request))
+            for gid, group in enumerate(self.groups):
+                table = group.tables[request]
+                if length % P == 0:
+                    table.append(group.pool.allocate())
+                    group._touch(request)
+                elif group.pool.refs[table[-1]] > 1:      # the shared, partly filled last page: copy on write
+                    slots, copies = group.append(request, length, 1)
+                    if copies and self._copy_pages is not None:
+                        self._copy_pages(group, copies)
+                done.slots[gid] = [table[-1] * P + length % P]
+            lengths[request] = length + 1
             result.append(done)
         return result
 

@@ -107,21 +107,26 @@ class ModelRunner:
         if not entries:
             raise ValueError("a step needs at least one entry")
         seen = set()
+        vocab, limit, lengths = self.model.vocab_size, self.max_context, self.cache.lengths
         for e in entries:
             if e.request in seen:
                 raise ValueError(f"request {e.request!r} appears twice in one step")
             seen.add(e.request)
-            if e.request not in self.cache:
+            if e.request not in lengths:
                 raise KeyError(f"unknown request {e.request!r}")
             n = len(e.tokens)
             if n == 0:
                 raise ValueError(f"request {e.request!r} brings no tokens")
-            if self.cache.length(e.request) + n > self.max_context:
-                raise ValueError(f"request {e.request!r} exceeds the context limit of {self.max_context}")
-            if any((not 0 <= int(t) < self.model.vocab_size) for t in e.tokens):
+            if lengths[e.request] + n > limit:
+                raise ValueError(f"request {e.request!r} exceeds the context limit of {limit}")
+            if n == 1:
+                if not 0 <= int(e.tokens[0]) < vocab:
+                    raise ValueError(f"request {e.request!r} has a token outside the vocabulary")
+            elif min(e.tokens) < 0 or max(e.tokens) >= vocab:
                 raise ValueError(f"request {e.request!r} has a token outside the vocabulary")
-            if any((not 0 <= int(w) < n) for w in e.want):
-                raise ValueError(f"request {e.request!r} wants a place outside its tokens")
+            for w in e.want:
+                if not 0 <= int(w) < n:
+                    raise ValueError(f"request {e.request!r} wants a place outside its tokens")
 
     def step(self, entries: List[StepEntry]):
         """Float logits [sum(len(want)), vocab] on the GPU (valid until the next step)."""

@@ -191,3 +191,43 @@ def test_random_orders_keep_every_page_accounted_for(seed):
         m.release(r)
     m.check()
     assert all(free == 12 for free in m.free_pages()) and len(m.slots.free) == 5
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_single_token_steps_take_the_same_pages_on_the_short_path(seed):
+    """Steps of one token a request run a short path; it must hand out exactly the pages, slots, copies and
+    errors of the general path, also after forks (shared last pages) and when the pool runs dry."""
+    def run(fast):
+        rng = random.Random(seed)
+        copies = []
+        m = CacheManager({0: KVNeed(2, 8, None), 1: KVNeed(2, 8, None), 2: KVNeed(1, 16, None)}, 10, 4, 6,
+                         copy_pages=lambda group, pairs: copies.append(list(pairs)))
+        m.fast_decode = fast
+        live, counter, log = [], 0, []
+        for _ in range(300):
+            action = rng.random()
+            if action < 0.2 and len(live) < 6:
+                name = f"r{counter}"; counter += 1
+                if live and rng.random() < 0.4:
+                    m.fork(rng.choice(live), name)
+                else:
+                    m.create(name)
+                    try:
+                        m.append_many([(name, rng.choice([1, 3, 4, 6]))])     # a prompt portion: the general path
+                    except OutOfPages:
+                        pass
+                live.append(name)
+            elif action < 0.9 and live:
+                picks = rng.sample(live, rng.randint(1, len(live)))
+                try:
+                    done = m.append_many([(r, 1) for r in picks])
+                    log.append([(d.request, d.start, d.state_slot, dict(d.slots)) for d in done])
+                except OutOfPages:
+                    log.append("out of pages")
+                    victim = rng.choice(live); m.release(victim); live.remove(victim)
+            elif live:
+                victim = rng.choice(live); m.release(victim); live.remove(victim)
+            m.check()
+        return log, copies, [dict(g.tables) for g in m.groups], [list(g.pool.free) for g in m.groups]
+
+    assert run(True) == run(False)

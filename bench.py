@@ -31,6 +31,9 @@ def main():
     ap.add_argument("--page-size", type=int, default=16)
     ap.add_argument("--points", default="1,64", help="other batch sizes to time (comma separated, empty for none)")
     ap.add_argument("--execution", default="graph", choices=["graph", "eager"])
+    ap.add_argument("--overlap", type=int, default=1, choices=[0, 1],
+                    help="1: picked tokens stay on the device and a step is launched before the tokens of the one "
+                         "before are read, as the scheduler's overlapped ticks do; 0: every step waits for its tokens")
     ap.add_argument("--workload", default="decode", choices=["decode", "serving"],
                     help="decode: fixed batch after whole prompts (the default, timed per step); serving: --requests "
                          "requests with prompts of 128..--prompt tokens and --new-tokens each through the scheduler")
@@ -100,10 +103,22 @@ def main():
             prefill_times.append(dt)
         params = [(0.0, 0, 0)] * batch
 
+        unread = None
+
         def one():
-            nonlocal last
-            logits = runner.step([StepEntry(k, [t], [0]) for k, t in zip(keys, last)])
-            last = sampler.pick(logits, params)
+            nonlocal last, unread
+            if args.overlap:
+                # the step takes its tokens from the device, where the last pick left them; the host reads
+                # the tokens of the step before while this one runs
+                logits = runner.step([StepEntry(k, [0], [0], pending=True) for k in keys] if unread is not None else
+                                     [StepEntry(k, [t], [0]) for k, t in zip(keys, last)])
+                picked = runner.pick(sampler, logits, params)
+                if unread is not None:
+                    last = unread.tokens()
+                unread = picked
+            else:
+                logits = runner.step([StepEntry(k, [t], [0]) for k, t in zip(keys, last)])
+                last = sampler.pick(logits, params)
 
         for _ in range(warmup):
             one()
@@ -112,6 +127,8 @@ def main():
         t0 = time.perf_counter()
         for _ in range(steps):
             one()
+        if unread is not None:
+            last = unread.tokens()
         torch.cuda.synchronize()
         elapsed = time.perf_counter() - t0
         ctx_mid = ctx0 + steps / 2
@@ -142,7 +159,7 @@ def main():
                    "parallelism": "single-gpu", "layers": L, "layers_of_configuration": full_layers, "hidden": H,
                    "heads": nh, "kv_heads": nkv, "head_dim": D, "intermediate": I, "vocab": V,
                    "rope_theta": c.rope_theta, "rms_norm_eps": c.rms_norm_eps, "tied_head": c.tie_word_embeddings,
-                   "page_size": args.page_size, "execution": args.execution},
+                   "page_size": args.page_size, "execution": args.execution + (", steps overlapped" if args.overlap else "")},
         "prefill": {"value": round(args.prompt / pf, 1), "tokens": args.prompt, "ms": round(pf * 1e3, 3),
                     "frac": round(prefill_flops(args.prompt) / pf / peak, 5)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBPS, "unit": "GB/s",
@@ -167,6 +184,7 @@ def serving(args, model, full_layers):
     pages = sum(-(-(n + args.new_tokens) // args.page_size) for n in lengths) + 8
     runner = ModelRunner(model, n_pages=pages, page_size=args.page_size, max_requests=args.requests, execution=args.execution)
     engine = Engine(runner, max_active=args.requests, token_budget=args.token_budget, prefill_chunk=args.prefill_chunk,
+                    overlap=bool(args.overlap),
                     policy="decode_first")
     # warm-up: a short run of the same shape of work compiles nothing new but fills the workspace
     for i in range(2):
@@ -196,7 +214,7 @@ def serving(args, model, full_layers):
                    "hidden": c.hidden_size, "heads": c.num_attention_heads, "kv_heads": c.num_key_value_heads,
                    "head_dim": c.head_dim, "intermediate": c.intermediate_size, "vocab": c.vocab_size,
                    "token_budget": args.token_budget, "prefill_chunk": args.prefill_chunk, "page_size": args.page_size,
-                   "execution": args.execution},
+                   "execution": args.execution + (", steps overlapped" if args.overlap else "")},
         "serving": {"seconds": round(elapsed, 3), "prompt_tokens": int(sum(lengths)), "generated_tokens": generated,
                     "all_tokens_per_s": round((sum(lengths) + generated) / elapsed, 1),
                     "ttft_median_ms": round(ttft[len(ttft) // 2] * 1e3, 1), "ttft_last_ms": round(ttft[-1] * 1e3, 1)},

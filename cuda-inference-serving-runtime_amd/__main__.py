@@ -33,6 +33,8 @@ def main(argv=None):
     parser.add_argument("--token-budget", type=int, default=32)
     parser.add_argument("--prefill-chunk", type=int, default=8)
     parser.add_argument("--max-active", type=int, default=8)
+    parser.add_argument("--overlap", action="store_true",
+                        help="launch each step before the tokens of the step before are read (same tokens, less idle GPU)")
     args = parser.parse_args(argv)
 
     from .config import read_config_json
@@ -42,7 +44,7 @@ def main(argv=None):
     execution = "graph" if args.execution == "graph" else "eager"
     common = dict(dtype=args.dtype, pages=args.pages, page_size=args.page_size, execution=execution,
                   policy=args.policy, token_budget=args.token_budget, prefill_chunk=args.prefill_chunk,
-                  max_active=args.max_active)
+                  max_active=args.max_active, overlap=args.overlap)
     if args.checkpoint:
         raw = read_config_json(args.checkpoint)
         engine = Engine.from_folder(args.checkpoint, **common)

@@ -62,44 +62,50 @@ argmax_partial_kernel(const float* __restrict__ logits, float* __restrict__ pval
 }
 
 __global__ void __launch_bounds__(64)
-argmax_final_kernel(const float* __restrict__ pval, const int* __restrict__ pidx, int* __restrict__ out, int chunks) {
+argmax_final_kernel(const float* __restrict__ pval, const int* __restrict__ pidx, int* __restrict__ out,
+                    const int* __restrict__ index, int out_n, int chunks) {
     const int row = blockIdx.x;
     if (threadIdx.x != 0) return;
+    const int dst = index ? index[row] : row;
+    if (dst < 0 || dst >= out_n) return;
     float bv = -INFINITY; int bi = 0x7fffffff;
     for (int c = 0; c < chunks; ++c) {
         const float v = pval[row * chunks + c]; const int i = pidx[row * chunks + c];
         if (i != 0x7fffffff && (bi == 0x7fffffff || v > bv)) { bv = v; bi = i; }
     }
-    out[row] = bi == 0x7fffffff ? 0 : bi;
+    out[dst] = bi == 0x7fffffff ? 0 : bi;
 }
 
 #define ARGMAX_CHUNKS 32
 
-// scratch: float [rows * 32] and int [rows * 32]
-extern "C" int cisr_argmax(const float* logits, int* out, float* scratch_val, int* scratch_idx, int rows, int vocab,
-                           hipStream_t stream) {
+// scratch: float [rows * 32] and int [rows * 32].  With `index`, row r's token goes to out[index[r]]
+// (nowhere if that is outside 0..out_n-1) instead of out[r]; without, out_n is rows.
+extern "C" int cisr_argmax(const float* logits, int* out, const int* index, int out_n, float* scratch_val, int* scratch_idx,
+                           int rows, int vocab, hipStream_t stream) {
     if (rows <= 0) return 0;
     argmax_partial_kernel<<<dim3(rows, ARGMAX_CHUNKS), 256, 0, stream>>>(logits, scratch_val, scratch_idx, vocab, ARGMAX_CHUNKS);
     int err = CISR_LAUNCH_CHECK();
     if (err) return err;
-    argmax_final_kernel<<<rows, 64, 0, stream>>>(scratch_val, scratch_idx, out, ARGMAX_CHUNKS);
+    argmax_final_kernel<<<rows, 64, 0, stream>>>(scratch_val, scratch_idx, out, index, index ? out_n : rows, ARGMAX_CHUNKS);
     return CISR_LAUNCH_CHECK();
 }
 
 __global__ void __launch_bounds__(256)
 sample_kernel(const float* __restrict__ logits, const float* __restrict__ temperature,
               const unsigned long long* __restrict__ seeds, const unsigned long long* __restrict__ counters,
-              int* __restrict__ out, int vocab) {
+              int* __restrict__ out, const int* __restrict__ index, int out_n, int vocab) {
     __shared__ float smax[256];
     __shared__ int sidx[256];
     __shared__ float ssum[256];
     const int row = blockIdx.x;
+    const int dst = index ? index[row] : row;
+    if (dst < 0 || dst >= out_n) return;       // the whole block: no barrier is passed by a part of it
     const float* x = logits + (size_t)row * vocab;
     float best; int best_idx;
     argmax_block(x, vocab, smax, sidx, best, best_idx);
     const float temp = temperature[row];
     if (!(temp > 0.f)) {  // greedy
-        if (threadIdx.x == 0) out[row] = best_idx == 0x7fffffff ? 0 : best_idx;
+        if (threadIdx.x == 0) out[dst] = best_idx == 0x7fffffff ? 0 : best_idx;
         return;
     }
     const float inv_t = 1.0f / temp;
@@ -127,13 +133,31 @@ sample_kernel(const float* __restrict__ logits, const float* __restrict__ temper
             if (choice < 0) choice = b - 1;
         }
         if (choice < 0) choice = best_idx;
-        out[row] = choice;
+        out[dst] = choice;
     }
 }
 
 extern "C" int cisr_sample(const float* logits, const float* temperature, const unsigned long long* seeds,
-                           const unsigned long long* counters, int* out, int rows, int vocab, hipStream_t stream) {
+                           const unsigned long long* counters, int* out, const int* index, int out_n, int rows, int vocab,
+                           hipStream_t stream) {
     if (rows <= 0) return 0;
-    sample_kernel<<<rows, 256, 0, stream>>>(logits, temperature, seeds, counters, out, vocab);
+    sample_kernel<<<rows, 256, 0, stream>>>(logits, temperature, seeds, counters, out, index, index ? out_n : rows, vocab);
+    return CISR_LAUNCH_CHECK();
+}
+
+// tokens[r] = sampled[source[r]] where source[r] >= 0: a row whose token is the one last picked for its
+// request and still only on the device takes it from there.
+__global__ void __launch_bounds__(256)
+take_tokens_kernel(int* __restrict__ tokens, const int* __restrict__ source, const int* __restrict__ sampled, int rows, int slots) {
+    const int r = blockIdx.x * 256 + threadIdx.x;
+    if (r >= rows) return;
+    const int s = source[r];
+    if (s >= 0 && s < slots) tokens[r] = sampled[s];
+}
+
+extern "C" int cisr_take_tokens(int* tokens, const int* source, const int* sampled, int rows, int slots, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    if (slots <= 0) return 1;
+    take_tokens_kernel<<<(rows + 255) / 256, 256, 0, stream>>>(tokens, source, sampled, rows, slots);
     return CISR_LAUNCH_CHECK();
 }

@@ -54,6 +54,7 @@ class StepContext:
         self.n_rows = self.n_segments = 0
         self.tokens = self.positions = self.seg_of_row = self.logit_rows = None
         self.seg_start = self.seg_first_pos = self.state_slots = None
+        self.token_source = None  # int32 [T]: state slot whose device-side picked token a row takes, or -1
         self.kv = []
         self.segments = []        # host: [(request, start, count)]
         self.max_context = 0      # host: largest position + 1 among the rows

@@ -29,6 +29,19 @@ class StepEntry:
     request: object
     tokens: Sequence[int]
     want: Sequence[int] = field(default_factory=list)  # indices into `tokens` whose logits are returned
+    pending: bool = False   # its one token is the one last picked for it, still only on the device (ModelRunner.pick)
+
+
+class PickedTokens:
+    """Tokens picked on the device for some requests, on their way to the host."""
+
+    def __init__(self, host, event, requests, slots):
+        self.host, self.event, self.requests, self.slots = host, event, requests, slots
+
+    def tokens(self):
+        """The token of each request, in the order of the logits they were picked from (waits for the copy)."""
+        self.event.synchronize()
+        return self.host[self.slots].tolist()
 
 
 _TORCH_OF = {"float32": torch.float32, "bfloat16": torch.bfloat16, "int32": torch.int32}
@@ -82,6 +95,12 @@ class ModelRunner:
                               for _ in self.cache.groups]
         self.task_tilings = []   # rows-per-tile values that mixers have asked task lists for
         self.steps = 0
+        # the token last picked on the device for each request, by state slot, and its copies on the way to the host
+        self.picked = torch.zeros(max_requests, dtype=torch.int32, device=self.device)
+        self._picked_host = [[torch.zeros(max_requests, dtype=torch.int32, pin_memory=True), None] for _ in range(4)]
+        self._picked_next = 0
+        self._has_picked = set()
+        self._last_wanted = None  # (requests, state slots on the host, state slots on the device) of the last step's logits
 
     # -- requests -------------------------------------------------------------
     def create(self, request):
@@ -93,6 +112,7 @@ class ModelRunner:
     def release(self, request):
         # later work that reuses the pages runs on the same stream, after every reader
         self.cache.release(request)
+        self._has_picked.discard(request)
 
     def length(self, request):
         return self.cache.length(request)
@@ -119,7 +139,10 @@ class ModelRunner:
                 raise ValueError(f"request {e.request!r} brings no tokens")
             if lengths[e.request] + n > limit:
                 raise ValueError(f"request {e.request!r} exceeds the context limit of {limit}")
-            if n == 1:
+            if e.pending:
+                if n != 1 or e.request not in self._has_picked:
+                    raise ValueError(f"request {e.request!r} has no one token picked on the device")
+            elif n == 1:
                 if not 0 <= int(e.tokens[0]) < vocab:
                     raise ValueError(f"request {e.request!r} has a token outside the vocabulary")
             elif min(e.tokens) < 0 or max(e.tokens) >= vocab:
@@ -136,17 +159,41 @@ class ModelRunner:
         if self.execution == "graph":
             return self._run_program(self._program_key(entries, done), entries, done)
         ctx = self._context(entries, done)
-        logits = self.model.forward(ctx)
+        logits = self._forward(ctx, any(e.pending for e in entries))
         if logits is None:
             return torch.empty((0, self.model.vocab_size), dtype=torch.float32, device=self.device)
         return logits
 
+    def _forward(self, ctx, take):
+        if take:   # rows whose token is still only on the device get it from there
+            ops.take_tokens(ctx.tokens, ctx.token_source, self.picked)
+        return self.model.forward(ctx)
+
+    def pick(self, sampler, logits, params):
+        """Pick a token for each row of the last step's logits and leave it on the device, where a later
+        step takes it from (StepEntry.pending); the host does not wait.  Returns PickedTokens, to be read
+        before three more calls of this function."""
+        requests, slots, where = self._last_wanted
+        if logits.shape[0] != len(requests):
+            raise ValueError("the logits are not those of the last step")
+        sampler.pick(logits, params, out=self.picked, index=where)
+        self._has_picked.update(requests)
+        entry = self._picked_host[self._picked_next % 4]
+        self._picked_next += 1
+        entry[0].copy_(self.picked, non_blocking=True)
+        if entry[1] is None:
+            entry[1] = torch.cuda.Event()
+        entry[1].record()
+        return PickedTokens(entry[0].numpy(), entry[1], requests, slots)
+
+    _FIXED = 9   # arrays of the metadata before the cache groups'
+
     def _layout(self, T, S, R):
         """Offsets of the packed int32 metadata: tokens, positions, seg_of_row, seg_start, seg_first_pos,
-        state_slots, logit_rows, then per group slots and tables, then one attention task list per
-        known tiling (its length is the most tiles that T rows in S segments can make)."""
+        state_slots, logit_rows, token_source, logit_slots, then per group slots and tables, then one
+        attention task list per known tiling (its length is the most tiles that T rows in S segments can make)."""
         W, G = self.table_width, len(self.cache.groups)
-        sizes = [T, T, T, S + 1, S, S, R] + [T, S * W] * G + [4 * (-(-T // r) + S) for r in self.task_tilings]
+        sizes = [T, T, T, S + 1, S, S, R, T, R] + [T, S * W] * G + [4 * (-(-T // r) + S) for r in self.task_tilings]
         return np.concatenate(([0], np.cumsum(sizes))).astype(np.int64)
 
     def _table_rows(self, g, done):
@@ -173,7 +220,7 @@ class ModelRunner:
         n_rows, n_seg = sum(counts), len(entries)
         n_want = sum(len(e.want) for e in entries)
         T, S, R = pad if pad is not None else (n_rows, n_seg, n_want)
-        W, G = self.table_width, len(self.cache.groups)
+        W, G, F = self.table_width, len(self.cache.groups), self._FIXED
         layout = (T, S, R, tuple(self.task_tilings))
         offsets = self._layouts.get(layout)
         if offsets is None:
@@ -181,15 +228,17 @@ class ModelRunner:
         total = offsets[-1]
         host = self._stage(total)
         arr = host.numpy()
-        tokens, positions, seg_of_row, seg_start, seg_first, state_slots, logit_rows = (
-            arr[offsets[i]:offsets[i + 1]] for i in range(7))
+        tokens, positions, seg_of_row, seg_start, seg_first, state_slots, logit_rows, token_source, logit_slots = (
+            arr[offsets[i]:offsets[i + 1]] for i in range(9))
         decode_only = n_rows == n_seg
+        slot_of = [d.state_slot for d in done]
+        wanted_seg = [s for s, e in enumerate(entries) for _ in e.want]
         if decode_only:
             first_row = np.arange(n_seg, dtype=np.int32)
             tokens[:n_rows] = [e.tokens[0] for e in entries]
             positions[:n_rows] = starts
             seg_of_row[:n_rows] = first_row
-            wanted = [s for s, e in enumerate(entries) for _ in e.want]
+            wanted = wanted_seg
         else:
             first_row = np.concatenate(([0], np.cumsum(counts[:-1]))).astype(np.int32)
             tokens[:n_rows] = np.concatenate([np.asarray(e.tokens, dtype=np.int32) for e in entries])
@@ -199,8 +248,18 @@ class ModelRunner:
         seg_start[:n_seg] = first_row
         seg_start[n_seg:] = n_rows
         seg_first[:n_seg] = starts
-        state_slots[:n_seg] = [d.state_slot for d in done]
+        state_slots[:n_seg] = slot_of
         logit_rows[:n_want] = wanted
+        wanted_slots = [slot_of[s] for s in wanted_seg]
+        logit_slots[:n_want] = wanted_slots
+        token_source[:] = -1
+        pending = [e.pending for e in entries]
+        if decode_only and all(pending):
+            token_source[:n_rows] = slot_of
+        elif any(pending):
+            for s, e in enumerate(entries):
+                if e.pending:
+                    token_source[first_row[s]] = slot_of[s]
         if pad is not None:      # the inert rest: token 0 at position 0, no segment, no slot, no table
             tokens[n_rows:] = 0
             positions[n_rows:] = 0
@@ -208,9 +267,10 @@ class ModelRunner:
             seg_first[n_seg:] = 0
             state_slots[n_seg:] = 0
             logit_rows[n_want:] = 0
+            logit_slots[n_want:] = -1
         for g in range(G):
-            slots = arr[offsets[7 + 2 * g]:offsets[8 + 2 * g]]
-            tables = arr[offsets[8 + 2 * g]:offsets[9 + 2 * g]].reshape(S, W)
+            slots = arr[offsets[F + 2 * g]:offsets[F + 1 + 2 * g]]
+            tables = arr[offsets[F + 1 + 2 * g]:offsets[F + 2 + 2 * g]].reshape(S, W)
             if decode_only:
                 slots[:n_rows] = [d.slots[g][0] for d in done]
             else:
@@ -221,7 +281,7 @@ class ModelRunner:
                 tables[n_seg:] = -1
         tilings = list(self.task_tilings)
         for i, rows_per_tile in enumerate(tilings):
-            tasks = arr[offsets[7 + 2 * G + i]:offsets[8 + 2 * G + i]].reshape(-1, 4)
+            tasks = arr[offsets[F + 2 * G + i]:offsets[F + 1 + 2 * G + i]].reshape(-1, 4)
             if decode_only:      # one tile of one row a segment
                 n = n_seg
                 tasks[:n, 0] = tasks[:n, 1] = first_row
@@ -240,8 +300,10 @@ class ModelRunner:
         ctx.n_rows, ctx.n_segments = T, S
         ctx.tokens, ctx.positions, ctx.seg_of_row = view(0), view(1), view(2)
         ctx.seg_start, ctx.seg_first_pos, ctx.state_slots, ctx.logit_rows = view(3), view(4), view(5), view(6)
-        ctx.kv = [GroupView(view(7 + 2 * g), view(8 + 2 * g, (S, W)), self.page_size, W) for g in range(G)]
-        ctx.tasks = {r: view(7 + 2 * G + i, (-1, 4)) for i, r in enumerate(tilings)}
+        ctx.token_source = view(7)
+        ctx.kv = [GroupView(view(F + 2 * g), view(F + 1 + 2 * g, (S, W)), self.page_size, W) for g in range(G)]
+        ctx.tasks = {r: view(F + 2 * G + i, (-1, 4)) for i, r in enumerate(tilings)}
+        self._last_wanted = ([entries[s].request for s in wanted_seg], wanted_slots, view(8)[:n_want])
         ctx.segments = [(d.request, d.start, d.count) for d in done]
         ctx.max_context = ctx.span_hint = max(s + c for s, c in zip(starts, counts))
         ctx.decode_only = decode_only
@@ -282,10 +344,11 @@ class ModelRunner:
         wanted = sum(len(e.want) for e in entries)
         decode_only = all(d.count == 1 for d in done)
         context = 1 << (max(d.start + d.count for d in done) - 1).bit_length()
-        return (_bucket(rows), _bucket(len(entries)), _bucket(wanted), decode_only, max(context, 256))
+        return (_bucket(rows), _bucket(len(entries)), _bucket(wanted), decode_only, max(context, 256),
+                any(e.pending for e in entries))
 
     def _run_program(self, key, entries, done):
-        T, S, R, decode_only, context = key
+        T, S, R, decode_only, context, take = key
         program = self.programs.get(key)
         if program is None:
             program = {"meta": None, "graph": None, "runs": 0, "tilings": None}
@@ -316,7 +379,7 @@ class ModelRunner:
             ctx.capturing = True
             try:
                 with torch.cuda.graph(graph, capture_error_mode="thread_local"):
-                    program["logits"] = self.model.forward(ctx)
+                    program["logits"] = self._forward(ctx, take)
             finally:
                 if collecting:
                     gc.enable()
@@ -325,7 +388,7 @@ class ModelRunner:
             program["graph"].replay()
             logits = program["logits"]
         else:
-            logits = self.model.forward(ctx)
+            logits = self._forward(ctx, take)
         program["runs"] += 1
         wanted = sum(len(e.want) for e in entries)
         if logits is None:

@@ -14,6 +14,12 @@ reserves the pages of its whole prompt and output (runtime/engine.py:65-76).
 A request that does not fit beside the running ones waits (later, smaller ones
 may pass it); one that could never fit is refused at submit
 (runtime/engine.py:46-47).  Nothing is preempted.
+
+With `overlap`, a tick launches its step before the tokens of the step before
+are read: picked tokens stay on the device, the next step takes them from
+there, and the host prepares step N+1 while the GPU runs step N.  The tokens
+are the same; a request that ends on an end-of-sequence token is found out one
+step late, and the token it decoded meanwhile is dropped.
 """
 import math
 import time
@@ -37,7 +43,8 @@ class Request:
     seed: int = 0
     generated: list = field(default_factory=list)
     cursor: int = 0
-    status: str = "waiting"  # waiting, prefill, decode, finished, cancelled
+    launched: int = 0        # tokens picked for it so far, read by the host or not (overlapped ticks)
+    status: str = "waiting"  # waiting, prefill, decode, draining (its last token is picked, not read), finished, cancelled
     submitted_at: float = 0.0
     first_token_at: Optional[float] = None
     token_times: list = field(default_factory=list)
@@ -45,7 +52,8 @@ class Request:
 
 
 class Engine:
-    def __init__(self, runner, max_active=8, token_budget=32, prefill_chunk=8, policy="chunked", sampler=None):
+    def __init__(self, runner, max_active=8, token_budget=32, prefill_chunk=8, policy="chunked", sampler=None,
+                 overlap=False):
         if min(max_active, token_budget, prefill_chunk) <= 0:
             raise ValueError("invalid scheduler limits")
         if policy not in POLICIES:
@@ -59,6 +67,7 @@ class Engine:
         self.sampler = sampler
         self.waiting, self.active, self.requests, self.reserved = deque(), [], {}, {}
         self.trace, self.start, self.rotation = [], time.perf_counter(), 0
+        self.overlap, self.inflight = overlap, None
 
     # -- page accounting ----------------------------------------------------------
     def _pool_pages(self):
@@ -133,12 +142,16 @@ class Engine:
         for r in order:
             if remaining == 0:
                 break
+            if r.status == "draining":
+                continue
             n = 1 if r.status == "decode" else min(self.prefill_chunk, len(r.prompt) - r.cursor, remaining)
             plan.append((r, n))
             remaining -= n
         return plan
 
     def tick(self):
+        if self.overlap:
+            return self._tick_overlapped()
         self._admit()
         if not self.active:
             return bool(self.waiting)
@@ -176,6 +189,60 @@ class Engine:
                            "processed_tokens": sum(n for _, n in plan), "active": len(self.active),
                            "resident_pages": sum(g.pool.used for g in cache.groups)})
         return bool(self.active or self.waiting)
+
+    def _tick_overlapped(self):
+        self._admit()
+        if not self.active and self.inflight is None:
+            return bool(self.waiting)
+        now = time.perf_counter()
+        plan = self.plan()
+        entries, sampled = [], []
+        for r, n in plan:
+            if r.status == "decode":
+                if r.launched > len(r.generated):     # its last token is still only on the device
+                    entries.append(StepEntry(r.key, [0], [0], pending=True))
+                else:
+                    entries.append(StepEntry(r.key, [r.generated[-1]], [0]))
+                sampled.append(r)
+            else:
+                last = r.cursor + n == len(r.prompt)
+                entries.append(StepEntry(r.key, r.prompt[r.cursor:r.cursor + n], [n - 1] if last else []))
+                if last:
+                    sampled.append(r)
+        launched = None
+        if entries:
+            logits = self.runner.step(entries)
+            if sampled:
+                picked = self.runner.pick(self.sampler, logits, [(r.temperature, r.seed, r.launched) for r in sampled])
+                launched = (picked, sampled)
+            for r, n in plan:
+                if r.status == "prefill":
+                    r.cursor += n
+                    if r.cursor < len(r.prompt):
+                        continue
+                    r.status = "decode"
+                r.launched += 1
+                if r.launched >= r.max_new_tokens:
+                    r.status = "draining"     # nothing more to decode; it ends when this token is read
+        previous, self.inflight = self.inflight, launched
+        if previous is not None:
+            picked, requests = previous
+            tokens = picked.tokens()
+            completed = time.perf_counter()
+            for r, token in zip(requests, tokens):
+                if r.status in ("finished", "cancelled"):
+                    continue                  # ended by an earlier token, or cancelled: this one is dropped
+                r.generated.append(int(token))
+                r.token_times.append(completed)
+                if r.first_token_at is None:
+                    r.first_token_at = completed
+                if len(r.generated) >= r.max_new_tokens or self._is_eos(r, token):
+                    self._finish(r)
+        cache = self.runner.cache
+        self.trace.append({"elapsed_s": time.perf_counter() - self.start, "step_s": time.perf_counter() - now,
+                           "processed_tokens": sum(n for _, n in plan), "active": len(self.active),
+                           "resident_pages": sum(g.pool.used for g in cache.groups)})
+        return bool(self.active or self.waiting or self.inflight)
 
     @staticmethod
     def _is_eos(r, token):

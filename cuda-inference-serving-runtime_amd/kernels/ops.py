@@ -52,8 +52,9 @@ def _declare(h):
         "cisr_gemm_skinny_bf16": [p, i, p, i, p, i, p, i, i, i, i, i, i, p, f, p, p],
         "cisr_qkv_rope_skinny": [p, i, p, i, p, i, i, i, p, f, p, p, p, p, p, p, i, i, i, i, i, p],
         "cisr_attn_merge": [p, p, p, i, i, i, i, p],
-        "cisr_argmax": [p, p, p, p, i, i, p],
-        "cisr_sample": [p, p, p, p, p, i, i, p],
+        "cisr_argmax": [p, p, p, i, p, p, i, i, p],
+        "cisr_sample": [p, p, p, p, p, p, i, i, i, p],
+        "cisr_take_tokens": [p, p, p, i, i, p],
     }
     for name, args in sig.items():
         fn = getattr(h, name)
@@ -462,23 +463,44 @@ def mfma_attention_supported(dtype, dim, page_size):
 _argmax_scratch = {}
 
 
-def argmax(logits, out):
-    """out[r] = index of the largest logit of row r (the lowest index wins a tie)."""
+def _scatter(out, index, rows):
+    """(pointer of index or None, length of out) for a token choice that writes out[index[r]]."""
+    if index is None:
+        _dev(out, "out", torch.int32, (rows,))
+        return None, rows
+    _dev(out, "out", torch.int32)
+    return _dev(index, "index", torch.int32, (rows,)), out.numel()
+
+
+def argmax(logits, out, index=None):
+    """out[r] = index of the largest logit of row r (the lowest index wins a tie).  With `index`
+    (int32 [R]) the result of row r goes to out[index[r]] instead, or nowhere if that is no place of out."""
     rows, vocab = logits.shape
     key = (logits.device, rows)
     if key not in _argmax_scratch:
         _argmax_scratch[key] = (torch.empty(rows * 32, dtype=torch.float32, device=logits.device),
                                 torch.empty(rows * 32, dtype=torch.int32, device=logits.device))
     val, idx = _argmax_scratch[key]
-    _check(lib().cisr_argmax(_dev(logits, "logits", torch.float32), _dev(out, "out", torch.int32, (rows,)),
+    where, out_n = _scatter(out, index, rows)
+    _check(lib().cisr_argmax(_dev(logits, "logits", torch.float32), out.data_ptr(), where, out_n,
                              val.data_ptr(), idx.data_ptr(), rows, vocab, _stream()), "argmax")
     return out
 
 
-def sample(logits, temperature, seeds, counters, out):
-    """Temperature sampling per row; temperature <= 0 is greedy.  seeds/counters int64 [R]."""
+def sample(logits, temperature, seeds, counters, out, index=None):
+    """Temperature sampling per row; temperature <= 0 is greedy.  seeds/counters int64 [R].
+    `index` as for argmax."""
     rows, vocab = logits.shape
+    where, out_n = _scatter(out, index, rows)
     _check(lib().cisr_sample(_dev(logits, "logits", torch.float32), _dev(temperature, "temperature", torch.float32, (rows,)),
                              _dev(seeds, "seeds", torch.int64, (rows,)), _dev(counters, "counters", torch.int64, (rows,)),
-                             _dev(out, "out", torch.int32, (rows,)), rows, vocab, _stream()), "sample")
+                             out.data_ptr(), where, out_n, rows, vocab, _stream()), "sample")
     return out
+
+
+def take_tokens(tokens, source, sampled):
+    """tokens[r] = sampled[source[r]] for the rows whose source is a place of `sampled` (all int32)."""
+    rows = tokens.numel()
+    _check(lib().cisr_take_tokens(_dev(tokens, "tokens", torch.int32), _dev(source, "source", torch.int32, (rows,)),
+                                  _dev(sampled, "sampled", torch.int32), rows, sampled.numel(), _stream()), "take_tokens")
+    return tokens

@@ -55,10 +55,12 @@ def test_policies_and_execution_modes_agree(folders, dtype):
     V = TINY["c"]["vocab_size"]
     prompts = [random_tokens(40 + i, n, V) for i, n in enumerate([1, 7, 3, 40])]
     outputs = []
-    for policy, execution, budget, chunk in [("serial", "eager", 3, 2), ("chunked", "eager", 3, 2), ("decode_first", "eager", 3, 2),
-                                             ("decode_first", "graph", 64, 64), ("chunked", "graph", 5, 3)]:
+    for policy, execution, budget, chunk, overlap in [
+            ("serial", "eager", 3, 2, False), ("chunked", "eager", 3, 2, False), ("decode_first", "eager", 3, 2, False),
+            ("decode_first", "graph", 64, 64, False), ("chunked", "graph", 5, 3, False),
+            ("chunked", "eager", 3, 2, True), ("decode_first", "graph", 64, 64, True), ("chunked", "graph", 5, 3, True)]:
         e = Engine.from_folder(folders["c"], dtype=dtype, pages=20, page_size=4, execution=execution, policy=policy,
-                               token_budget=budget, prefill_chunk=chunk)
+                               token_budget=budget, prefill_chunk=chunk, overlap=overlap)
         for i, p in enumerate(prompts):
             e.submit(Request(str(i), p, 12))
         result = e.run()
@@ -188,6 +190,34 @@ def test_temperature_sampling_is_seeded_and_independent_of_the_batch(folders):
     assert e.generate(prompts[:2], max_new_tokens=12) != [together["0"], together["1"]]   # sampling is not greedy here
 
 
+@pytest.mark.parametrize("execution", ["eager", "graph"])
+def test_overlapped_ticks_sample_and_stop_like_plain_ticks(folders, execution):
+    """Steps launched before the tokens of the step before are read: the same sampled tokens, the same
+    stop at an end-of-sequence token (found one step late, the extra token dropped), every page back."""
+    from runtime.engine.scheduler import Engine, Request
+    V = TINY["b"]["vocab_size"]
+    prompts = [random_tokens(60 + i, n, V) for i, n in enumerate([1, 9, 33, 20, 5])]
+    news = [12, 1, 7, 12, 2]
+
+    def run(overlap, eos=None):
+        e = Engine.from_folder(folders["b"], dtype="float32", pages=24, page_size=8, execution=execution,
+                               token_budget=12, prefill_chunk=7, max_active=3, overlap=overlap)
+        for i, (p, n) in enumerate(zip(prompts, news)):
+            e.submit(Request(str(i), p, n, eos_token_id=eos, temperature=0.7 if i % 2 else 0.0, seed=5 + i))
+        out = {r.key: r.generated for r in e.run()}
+        e.runner.cache.check()
+        assert e.runner.cache.free_pages() == [24] and not e.reserved and e.inflight is None
+        return out
+
+    plain = run(False)
+    assert run(True) == plain
+    assert [len(plain[str(i)]) for i in range(5)] == news
+    eos = plain["0"][4]
+    stopped = run(False, eos)
+    assert len(stopped["0"]) <= 5 and stopped["0"][-1] == eos
+    assert run(True, eos) == stopped
+
+
 def test_fork_shares_a_prefix_and_copies_on_write(folders):
     # reference tests/test_execution.py:55-64
     from runtime.engine import load_model, ModelRunner, StepEntry
@@ -226,7 +256,7 @@ def test_command_line(folders, tmp_path):
     assert by_key["x"]["generated"] == P.greedy(cfg, w, [1, 2, 3, 4, 5], 4) and by_key["x"]["status"] == "finished"
     assert by_key["y"]["generated"] == P.greedy(cfg, w, [9], 3) and by_key["y"]["ttft_ms"] > 0
     proc = subprocess.run([sys.executable, "-m", "runtime", "--model", "tiny-b", "--tokens", "5,6,7", "--max-new-tokens", "3",
-                           "--execution", "graph"], capture_output=True, text=True, timeout=300, env=env, cwd=str(tmp_path))
+                           "--execution", "graph", "--overlap"], capture_output=True, text=True, timeout=300, env=env, cwd=str(tmp_path))
     assert proc.returncode == 0, proc.stderr[-2000:]
     out = json.loads(proc.stdout)
     assert out["weights"] == "random-tiny-b" and len(out["requests"][0]["generated"]) == 3

@@ -547,6 +547,42 @@ def test_argmax_lowest_index_wins(ops):
     assert out[1] == 17 and out[2] == 0 and out[3] == 1002
 
 
+def test_token_choices_scattered_by_index_and_taken_back(ops):
+    """A token choice that leaves row r's token at out[index[r]] (nowhere for an index outside out), and the
+    rows of a step that take their token from there."""
+    z = rnd(7, 517, seed=12)
+    greedy = f64(z).argmax(-1)
+    index = torch.tensor([4, 0, -1, 9, 2, 40, 7], dtype=torch.int32, device=DEV)
+    for how in ("argmax", "sample"):
+        out = torch.full((10,), -5, dtype=torch.int32, device=DEV)
+        if how == "argmax":
+            ops.argmax(z, out, index)
+        else:
+            ops.sample(z, torch.zeros(7, device=DEV), torch.zeros(7, dtype=torch.int64, device=DEV),
+                       torch.zeros(7, dtype=torch.int64, device=DEV), out, index)
+        want = np.full(10, -5)
+        for r, i in enumerate(index.tolist()):
+            if 0 <= i < 10:
+                want[i] = greedy[r]
+        np.testing.assert_array_equal(out.cpu().numpy(), want)
+    # sampled rows land at their index too, with the same draw as without an index
+    temp, seeds = torch.full((7,), 0.9, device=DEV), torch.arange(7, dtype=torch.int64, device=DEV)
+    counters = torch.full((7,), 3, dtype=torch.int64, device=DEV)
+    direct = ops.sample(z, temp, seeds, counters, torch.empty(7, dtype=torch.int32, device=DEV)).cpu().numpy()
+    out = torch.full((10,), -5, dtype=torch.int32, device=DEV)
+    ops.sample(z, temp, seeds, counters, out, index)
+    for r, i in enumerate(index.tolist()):
+        if 0 <= i < 10:
+            assert out[i].item() == direct[r]
+    tokens = torch.arange(100, 106, dtype=torch.int32, device=DEV)
+    source = torch.tensor([-1, 9, 4, -1, 0, 77], dtype=torch.int32, device=DEV)
+    ops.take_tokens(tokens, source, out)
+    picked = out.cpu().numpy()
+    np.testing.assert_array_equal(tokens.cpu().numpy(), [100, picked[9], picked[4], 103, picked[0], 105])
+    with pytest.raises(Exception):
+        ops.argmax(z, out, index[:3].contiguous())
+
+
 def test_sampling_kernel(ops):
     from runtime.sampling import uniform01
     V = 11

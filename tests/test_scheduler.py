@@ -48,6 +48,43 @@ class ArgmaxSampler:
         return logits.argmax(-1).tolist()
 
 
+class Later:
+    def __init__(self, tokens):
+        self._tokens = tokens
+
+    def tokens(self):
+        return self._tokens
+
+
+class OverlapRunner(FakeRunner):
+    """The stand-in with picked tokens kept 'on the device': a pending entry takes its token from there."""
+
+    def __init__(self, *a, **kw):
+        super().__init__(*a, **kw)
+        self.device_tokens, self.wanted = {}, []
+
+    def step(self, entries):
+        from runtime.engine.runner import StepEntry
+        real = []
+        for e in entries:
+            if e.pending:
+                assert list(e.tokens) == [0] and e.request in self.device_tokens
+                real.append(StepEntry(e.request, [self.device_tokens[e.request]], e.want))
+            else:
+                real.append(e)
+        self.wanted = [e.request for e in entries for _ in e.want]
+        return super().step(real)
+
+    def pick(self, sampler, logits, params):
+        tokens = sampler.pick(logits, params)
+        self.device_tokens.update(zip(self.wanted, tokens))
+        return Later(tokens)
+
+    def release(self, key):
+        super().release(key)
+        self.device_tokens.pop(key, None)
+
+
 def make_engine(runner=None, **kw):
     return Engine(runner or FakeRunner(), sampler=ArgmaxSampler(), **kw)
 
@@ -191,3 +228,61 @@ def test_serial_runs_one_request_at_a_time():
     e.run()
     assert all(len({k for k, _, _ in call}) == 1 for call in e.runner.calls)
     assert e.max_active == 1
+
+
+@pytest.mark.parametrize("policy", ["serial", "chunked", "decode_first"])
+def test_overlapped_ticks_give_the_same_tokens(policy):
+    lengths, news = [1, 7, 3, 9, 2], [5, 1, 8, 3, 6]
+    plain = make_engine(policy=policy, token_budget=4, prefill_chunk=3)
+    for i, (length, new) in enumerate(zip(lengths, news)):
+        plain.submit(Request(str(i), list(range(length)), new))
+    want = [r.generated for r in plain.run()]
+    e = make_engine(OverlapRunner(), policy=policy, token_budget=4, prefill_chunk=3, overlap=True)
+    for i, (length, new) in enumerate(zip(lengths, news)):
+        e.submit(Request(str(i), list(range(length)), new))
+    result = e.run()
+    assert [r.generated for r in result] == want
+    assert all(r.status == "finished" for r in result) and not e.reserved and e.inflight is None
+    e.runner.cache.check()
+    assert e.runner.cache.free_pages() == [20]
+    assert all(t["processed_tokens"] <= 4 for t in e.trace)
+    # a request is never stepped past its last token: the count is known before the token is read
+    fed = {}
+    for call in e.runner.calls:
+        for key, n, _ in call:
+            fed[key] = fed.get(key, 0) + n
+    assert fed == {str(i): length + new - 1 for i, (length, new) in enumerate(zip(lengths, news))}
+
+
+def test_overlapped_ticks_end_on_eos_one_step_late_and_drop_the_extra_token():
+    probe = make_engine()
+    probe.submit(Request("probe", [5, 6], 8))
+    probe.submit(Request("other", [7], 8))
+    probe.run()
+    tokens = probe.requests["probe"].generated
+    e = make_engine(OverlapRunner(), overlap=True)
+    e.submit(Request("probe", [5, 6], 8, eos_token_id=tokens[2]))
+    e.submit(Request("other", [7], 8))
+    e.run()
+    stop = tokens.index(tokens[2])
+    assert e.requests["probe"].generated == tokens[:stop + 1]
+    assert e.requests["other"].generated == probe.requests["other"].generated
+    assert not e.reserved and e.inflight is None
+    e.runner.cache.check()
+    assert e.runner.cache.free_pages() == [20]
+    # the token after the end was decoded (the step was already launched) and thrown away
+    fed = sum(n for call in e.runner.calls for key, n, _ in call if key == "probe")
+    assert fed == 2 + stop + 1
+
+
+def test_overlapped_ticks_cancel_while_a_step_is_in_flight():
+    e = make_engine(OverlapRunner(), overlap=True)
+    e.submit(Request("a", [1, 2, 3], 6))
+    e.submit(Request("b", [4], 6))
+    e.tick(); e.tick()
+    e.cancel("a")
+    e.run()
+    assert e.requests["a"].status == "cancelled" and e.requests["b"].status == "finished"
+    assert len(e.requests["b"].generated) == 6 and not e.reserved
+    e.runner.cache.check()
+    assert e.runner.cache.free_pages() == [20]

@@ -7,6 +7,7 @@ stream, so they are ordered with torch's own work and can be captured into a
 graph.  Nothing here computes on the CPU.
 """
 import ctypes as C
+import os
 
 import torch
 
@@ -55,11 +56,14 @@ def _declare(h):
         "cisr_argmax": [p, p, p, i, p, p, i, i, p],
         "cisr_sample": [p, p, p, p, p, p, i, i, i, p],
         "cisr_take_tokens": [p, p, p, i, i, p],
+        "cisr_gemm_wide_bf16": [p, i, p, i, p, i, p, i, i, i, i, i, i, p, C.c_longlong, p],
     }
     for name, args in sig.items():
         fn = getattr(h, name)
         fn.argtypes = args
         fn.restype = C.c_int
+    h.cisr_gemm_wide_workspace.argtypes = [i, i, i, i]
+    h.cisr_gemm_wide_workspace.restype = C.c_longlong
 
 
 _attention_entries = {}
@@ -274,6 +278,8 @@ def gemm(a, w, out, residual=None):
             raise KernelError("gemm: float operands need a float output")
         code = lib().cisr_gemm_f32(a.data_ptr(), a.stride(0), w.data_ptr(), w.stride(0), out.data_ptr(), out.stride(0),
                                    rp, ldr, m, n, k, _stream())
+    elif a.dtype == torch.bfloat16 and m <= SKINNY_ROWS and _skinny_ok(a, w) and wide_ok(m, w):
+        return _gemm_wide(a, w, out, residual, False, "gemm")
     elif a.dtype == torch.bfloat16 and m <= SKINNY_ROWS and _skinny_ok(a, w):
         code = lib().cisr_gemm_skinny_bf16(a.data_ptr(), a.stride(0), w.data_ptr(), w.stride(0), out.data_ptr(),
                                            out.stride(0), rp, ldr, m, n, k, _storage(out, "out"), 0, None, 0.0, None,
@@ -284,6 +290,60 @@ def gemm(a, w, out, residual=None):
     else:
         raise KernelError(f"gemm: unsupported dtype {a.dtype}")
     _check(code, "gemm")
+    return out
+
+
+# Weights of at least this many bytes are streamed by the kernel that keeps the activations in registers
+# (norm, rotary embedding and cache write are then kernels of their own); smaller ones by the kernels that
+# fuse them, which cost fewer launches.  With at most 16 rows the activations are a small part of the
+# traffic and the fused kernels hold out longer.
+WIDE_MIN_BYTES = int(float(os.environ.get("CISR_WIDE_MIN_MB", "12")) * (1 << 20))
+WIDE_MIN_BYTES_FEW_ROWS = int(float(os.environ.get("CISR_WIDE_MIN_MB_FEW_ROWS", "64")) * (1 << 20))
+_wide_workspaces = {}    # device -> buffers, never freed: captured programs keep their addresses
+_wide_plans = {}
+
+
+def wide_ok(m, w, swiglu=False):
+    """Whether a product of m rows with the bf16 weights w runs the wide weight-streaming kernel."""
+    n, k = w.shape
+    least = WIDE_MIN_BYTES_FEW_ROWS if m <= 16 else WIDE_MIN_BYTES
+    if (w.dtype != torch.bfloat16 or not 0 < m <= SKINNY_ROWS or w.numel() * 2 < least or k % 8 or w.stride(0) % 8
+            or w.data_ptr() % 16 or w.stride(1) != 1):
+        return False
+    return _wide_plan(m, n // 2 if swiglu else n, k, swiglu) >= 0
+
+
+def _wide_plan(m, n, k, swiglu):
+    key = ((m + 15) // 16, m, n, k, swiglu)
+    need = _wide_plans.get(key)
+    if need is None:
+        need = _wide_plans[key] = int(lib().cisr_gemm_wide_workspace(m, n, k, n if swiglu else 0))
+    return need
+
+
+def _wide_workspace(device, floats):
+    if floats <= 0:
+        return None
+    pool = _wide_workspaces.setdefault(device, [])
+    for buf in pool:
+        if buf.numel() >= floats:
+            return buf
+    pool.append(torch.empty(1 << (floats - 1).bit_length(), dtype=torch.float32, device=device))
+    return pool[-1]
+
+
+def _gemm_wide(a, w, out, residual, swiglu, what):
+    m, k = a.shape
+    n = w.shape[0] // 2 if swiglu else w.shape[0]
+    need = _wide_plan(m, n, k, swiglu)
+    if need < 0 or a.stride(0) % 8 or a.data_ptr() % 16:
+        raise KernelError(f"{what}: shape not supported by the wide kernel")
+    work = _wide_workspace(a.device, need)
+    rp, ldr = (residual.data_ptr(), residual.stride(0)) if residual is not None else (None, 0)
+    _check(lib().cisr_gemm_wide_bf16(a.data_ptr(), a.stride(0), w.data_ptr(), w.stride(0), out.data_ptr(), out.stride(0),
+                                     rp, ldr, m, n, k, _storage(out, "out"), n if swiglu else 0,
+                                     None if work is None else work.data_ptr(), 0 if work is None else work.numel(),
+                                     _stream()), what)
     return out
 
 
@@ -305,8 +365,9 @@ def _norm_args(x, norm, k):
 
 
 def fused_norm_ok(x, w, rows_out):
-    """Whether the weight-streaming kernel can take RMSNorm(x) . w^T with the norm fused."""
-    return (w.dtype == torch.bfloat16 and rows_out <= SKINNY_ROWS and x.dtype == torch.float32 and x.shape[1] % 8 == 0
+    """Whether the weight-streaming kernel can take RMSNorm(x) . w^T with the norm fused (and large weights
+    do not make the norm as a kernel of its own and the wide kernel the better choice)."""
+    return (not wide_ok(rows_out, w) and w.dtype == torch.bfloat16 and rows_out <= SKINNY_ROWS and x.dtype == torch.float32 and x.shape[1] % 8 == 0
             and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w.stride(0) % 8 == 0 and w.data_ptr() % 16 == 0)
 
 
@@ -349,6 +410,8 @@ def gemm_swiglu(a, w_gate_up, out, scratch=None, norm=None):
     if out.dtype != a.dtype or a.dtype != w_gate_up.dtype:
         raise KernelError("gemm_swiglu: dtypes differ")
     if swiglu_fused_ok(a, w_gate_up):
+        if m <= SKINNY_ROWS and wide_ok(m, w_gate_up, True):
+            return _gemm_wide(a, w_gate_up, out, None, True, "gemm_swiglu")
         if m <= SKINNY_ROWS:
             _check(lib().cisr_gemm_skinny_bf16(a.data_ptr(), a.stride(0), w_gate_up.data_ptr(), w_gate_up.stride(0),
                                                out.data_ptr(), out.stride(0), None, 0, m, inter, k, BF16, inter, None, 0.0,
@@ -366,7 +429,7 @@ def gemm_swiglu(a, w_gate_up, out, scratch=None, norm=None):
 def qkv_rope_fused_ok(a, w, head_dim, cos, normed):
     """Whether the fused projection + rotary + scatter kernel takes this shape."""
     m, k = a.shape
-    return (w.dtype == torch.bfloat16 and m <= SKINNY_ROWS and k % 8 == 0 and head_dim % 16 == 0
+    return (not wide_ok(m, w) and w.dtype == torch.bfloat16 and m <= SKINNY_ROWS and k % 8 == 0 and head_dim % 16 == 0
             and 2 * cos.shape[1] == head_dim and a.stride(0) % 8 == 0 and a.data_ptr() % 16 == 0
             and w.stride(0) % 8 == 0 and w.data_ptr() % 16 == 0
             and a.dtype == (torch.float32 if normed else torch.bfloat16))

@@ -495,6 +495,42 @@ def test_fused_projection_rotary_scatter(ops, heads, kv_heads, dim, theta, norme
 GEMM_SHAPES = [(1, 1, 1), (5, 7, 9), (64, 64, 32), (130, 200, 172), (33, 513, 144), (17, 130, 1000), (300, 129, 72), (8, 1536, 576)]
 
 
+def test_gemm_wide_for_large_weights(ops, monkeypatch):
+    """Few rows against weights of many megabytes run the kernel that keeps the activations in registers and cuts
+    K into slices: forced here for small shapes: every number of row tiles, widths off the 16-column unit,
+    inner sizes of one step, of a partial pair, of several slices with an uneven cut, residual, bf16 output, SwiGLU."""
+    monkeypatch.setattr(ops, "WIDE_MIN_BYTES", 0)
+    monkeypatch.setattr(ops, "WIDE_MIN_BYTES_FEW_ROWS", 0)
+    shapes = [(1, 16, 8), (3, 100, 72), (8, 1728, 576), (16, 576, 1536), (17, 49, 264), (33, 130, 200), (48, 40, 2056),
+              (64, 96, 4096), (50, 1003, 200), (8, 64, 14336), (64, 48, 9000), (20, 33, 4104)]
+    for M, N, K in shapes:
+        a, w, r = rnd(M, K, dtype=torch.bfloat16, seed=1), rnd(N, K, dtype=torch.bfloat16, seed=2), rnd(M, N, seed=3)
+        assert ops.wide_ok(M, w)
+        want = f64(a) @ f64(w).T
+        np.testing.assert_allclose(f64(ops.gemm(a, w, torch.empty(M, N, device=DEV))), want, rtol=1e-4, atol=1e-4 * math.sqrt(K))
+        np.testing.assert_allclose(f64(ops.gemm(a, w, torch.empty(M, N, dtype=torch.bfloat16, device=DEV))), want, rtol=1e-2, atol=1e-2 * math.sqrt(K))
+        out = r.clone(); ops.gemm(a, w, out, residual=out)
+        np.testing.assert_allclose(f64(out), want + f64(r), rtol=1e-4, atol=1e-4 * math.sqrt(K))
+    for M, I, K in [(1, 16, 32), (8, 1536, 576), (24, 100, 4096), (40, 172, 64), (64, 264, 2200)]:
+        a = rnd(M, K, dtype=torch.bfloat16, seed=4, scale=0.5)
+        w = rnd(2 * I, K, dtype=torch.bfloat16, seed=5, scale=0.2 if K < 1000 else 0.05)
+        assert ops.wide_ok(M, w, True)
+        gu = f64(a) @ f64(w).T
+        gq = torch.from_numpy(gu).to(torch.bfloat16).double().numpy()
+        got = ops.gemm_swiglu(a, w, torch.empty(M, I, dtype=torch.bfloat16, device=DEV))
+        np.testing.assert_allclose(f64(got), P.swiglu(gq[:, :I], gq[:, I:]), rtol=2e-2, atol=2e-2)
+    # a row's result does not depend on the rows beside it (same number of row tiles: the same launch)
+    a, w = rnd(16, 4104, dtype=torch.bfloat16, seed=6), rnd(80, 4104, dtype=torch.bfloat16, seed=7)
+    whole = ops.gemm(a, w, torch.empty(16, 80, device=DEV)).clone()
+    for rows in (1, 5, 9):
+        part = ops.gemm(a[:rows].contiguous(), w, torch.empty(rows, 80, device=DEV))
+        assert torch.equal(part, whole[:rows])
+    # with large weights the fused forms step aside for it
+    assert not ops.fused_norm_ok(rnd(8, 576), rnd(1728, 576, dtype=torch.bfloat16), 8)
+    monkeypatch.setattr(ops, "WIDE_MIN_BYTES_FEW_ROWS", 1 << 40)
+    assert ops.fused_norm_ok(rnd(8, 576), rnd(1728, 576, dtype=torch.bfloat16), 8) and not ops.wide_ok(8, w)
+
+
 @pytest.mark.parametrize("M, N, K", GEMM_SHAPES)
 def test_gemm_f32(ops, M, N, K):
     a, w, r = rnd(M, K, seed=1), rnd(N, K, seed=2), rnd(M, N, seed=3)

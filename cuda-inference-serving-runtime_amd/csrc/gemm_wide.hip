@@ -212,18 +212,21 @@ static int wide_launch(WideArgs a, size_t workspace_floats, bool plan_only, long
     return CISR_LAUNCH_CHECK();
 }
 
-// Rounds a slice (SPW / 2): the one with the least work for the busiest block, counted in rounds (the rounds of
-// a last slice past K are loaded from clamped addresses and add nothing, but cost like the others), plus about
-// two rounds for the second kernel that several slices need; ties go to the longer slice.
+// Rounds a slice (SPW / 2): the one with the least work for the busiest block, counted in rounds (a round of a
+// block streams NW * 2 KB of each block of W; the rounds of a last slice past K are loaded from clamped addresses
+// and add nothing, but cost like the others).  Several slices add the traffic of their partial sums, written
+// and read once, shared among the compute units, and about two rounds for the second kernel.  Ties go to the
+// longer slice.
 template <int MT, int NW, int MAXSPW, int NB>
 static int wide_steps(const WideArgs& a, size_t workspace_floats, bool plan_only, long long* need, hipStream_t stream) {
     const int pairs = (a.K + 63) / 64, rounds = (pairs + NW - 1) / NW, cus = wide_cus();
     int best = 1;
-    long long best_cost = -1;
+    double best_cost = -1.0;
     for (int r = MAXSPW / 2; r >= 1; r /= 2) {
         const int slices = (rounds + r - 1) / r;
         const long long items = (long long)a.units * slices;
-        const long long cost = (items + cus - 1) / cus * r + (slices > 1 ? 2 : 0);
+        double cost = (double)((items + cus - 1) / cus) * r;
+        if (slices > 1) cost += 2.0 + (double)slices * a.M * a.N * 8.0 / ((double)NW * 2048.0 * cus);
         if (best_cost < 0 || cost < best_cost) { best = r; best_cost = cost; }
     }
     if constexpr (MAXSPW >= 8) if (best == 4) return wide_launch<MT, NW, 8, NB>(a, workspace_floats, plan_only, need, stream);

@@ -295,10 +295,13 @@ def gemm(a, w, out, residual=None):
 
 # Weights of at least this many bytes are streamed by the kernel that keeps the activations in registers
 # (norm, rotary embedding and cache write are then kernels of their own); smaller ones by the kernels that
-# fuse them, which cost fewer launches.  With at most 16 rows the activations are a small part of the
-# traffic and the fused kernels hold out longer.
-WIDE_MIN_BYTES = int(float(os.environ.get("CISR_WIDE_MIN_MB", "12")) * (1 << 20))
+# fuse them, which cost fewer launches.  Measured on an MI355X against the other kernel in captured graphs:
+# with at most 16 rows the activations are a small part of the traffic and the fused kernels hold out up to
+# about 64 MB; with 17 to 32 rows the wide kernel wins from about 12 MB on, with more from about 30 MB on
+# (a block then holds so much of the activations that it needs many rows of W to spread their cost over).
 WIDE_MIN_BYTES_FEW_ROWS = int(float(os.environ.get("CISR_WIDE_MIN_MB_FEW_ROWS", "64")) * (1 << 20))
+WIDE_MIN_BYTES = int(float(os.environ.get("CISR_WIDE_MIN_MB", "12")) * (1 << 20))
+WIDE_MIN_BYTES_MANY_ROWS = int(float(os.environ.get("CISR_WIDE_MIN_MB_MANY_ROWS", "30")) * (1 << 20))
 _wide_workspaces = {}    # device -> buffers, never freed: captured programs keep their addresses
 _wide_plans = {}
 
@@ -306,7 +309,7 @@ _wide_plans = {}
 def wide_ok(m, w, swiglu=False):
     """Whether a product of m rows with the bf16 weights w runs the wide weight-streaming kernel."""
     n, k = w.shape
-    least = WIDE_MIN_BYTES_FEW_ROWS if m <= 16 else WIDE_MIN_BYTES
+    least = WIDE_MIN_BYTES_FEW_ROWS if m <= 16 else WIDE_MIN_BYTES if m <= 32 else WIDE_MIN_BYTES_MANY_ROWS
     if (w.dtype != torch.bfloat16 or not 0 < m <= SKINNY_ROWS or w.numel() * 2 < least or k % 8 or w.stride(0) % 8
             or w.data_ptr() % 16 or w.stride(1) != 1):
         return False

@@ -145,6 +145,50 @@ def test_captured_prompt_and_mixed_steps_match_the_plain_model(folders, name, dt
     runner.cache.check()
 
 
+@pytest.mark.parametrize("name", ["a", "b"])
+@pytest.mark.parametrize("execution", ["eager", "graph"])
+def test_steps_through_the_wide_product_match_the_plain_model(folders, name, execution, monkeypatch):
+    """With large weights the products of steps of up to 64 rows run the kernel that keeps the activations in
+    registers, with norm, rotary embedding and cache write as kernels of their own; forced here on the tiny
+    models: decode steps, short portions, mixed steps, again and again (its workspace is shared by the steps)."""
+    from runtime.engine import load_model, ModelRunner, StepEntry
+    from runtime.kernels import ops
+    from conftest import plain_logits, assert_close
+    for limit in ("WIDE_MIN_BYTES", "WIDE_MIN_BYTES_FEW_ROWS", "WIDE_MIN_BYTES_MANY_ROWS"):
+        monkeypatch.setattr(ops, limit, 0)
+    V = TINY[name]["vocab_size"]
+    model = load_model(folders[name], dtype="bfloat16")
+    runner = ModelRunner(model, n_pages=24, page_size=8, max_requests=4, execution=execution)
+    calls = []
+    wide = ops._gemm_wide
+    monkeypatch.setattr(ops, "_gemm_wide", lambda *a: (calls.append(a[-1]), wide(*a))[1])
+    seqs = {k: random_tokens(500 + i, 60, V) for i, k in enumerate("xyz")}
+    refs = {k: plain_logits(folders[name], seqs[k]) for k in seqs}
+    for k in seqs:
+        runner.create(k)
+    fed = {k: 0 for k in seqs}
+
+    def feed(*parts):
+        entries, places = [], []
+        for k, n in parts:
+            entries.append(StepEntry(k, seqs[k][fed[k]:fed[k] + n], [0, n - 1] if n > 1 else [0]))
+            places += [(k, fed[k]), (k, fed[k] + n - 1)] if n > 1 else [(k, fed[k])]
+            fed[k] += n
+        logits = runner.step(entries).float().cpu().numpy()
+        for row, (k, pos) in zip(logits, places):
+            assert_close(row[None], refs[k][pos][None], "bfloat16", f"request {k} position {pos}")
+
+    feed(("x", 33))                              # three row tiles
+    feed(("y", 17), ("z", 2))                    # two
+    for _ in range(3):
+        feed(("x", 1), ("y", 1), ("z", 1))       # decode steps
+    feed(("x", 1), ("y", 9), ("z", 30))
+    for _ in range(3):
+        feed(("x", 1), ("y", 1), ("z", 1))
+    assert {"gemm", "gemm_swiglu"} <= set(calls)
+    runner.cache.check()
+
+
 @pytest.mark.parametrize("name", ["a", "c"])
 @pytest.mark.parametrize("item_tiles", [1, 2])
 def test_long_portions_through_block_tiles_match_the_plain_model(folders, name, item_tiles):

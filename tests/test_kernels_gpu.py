@@ -501,6 +501,7 @@ def test_gemm_wide_for_large_weights(ops, monkeypatch):
     inner sizes of one step, of a partial pair, of several slices with an uneven cut, residual, bf16 output, SwiGLU."""
     monkeypatch.setattr(ops, "WIDE_MIN_BYTES", 0)
     monkeypatch.setattr(ops, "WIDE_MIN_BYTES_FEW_ROWS", 0)
+    monkeypatch.setattr(ops, "WIDE_MIN_BYTES_MANY_ROWS", 0)
     shapes = [(1, 16, 8), (3, 100, 72), (8, 1728, 576), (16, 576, 1536), (17, 49, 264), (33, 130, 200), (48, 40, 2056),
               (64, 96, 4096), (50, 1003, 200), (8, 64, 14336), (64, 48, 9000), (20, 33, 4104)]
     for M, N, K in shapes:

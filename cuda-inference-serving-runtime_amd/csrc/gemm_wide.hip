@@ -212,21 +212,30 @@ static int wide_launch(WideArgs a, size_t workspace_floats, bool plan_only, long
     return CISR_LAUNCH_CHECK();
 }
 
-// Rounds a slice (SPW / 2): the one with the least work for the busiest block, counted in rounds (a round of a
-// block streams NW * 2 KB of each block of W; the rounds of a last slice past K are loaded from clamped addresses
-// and add nothing, but cost like the others).  Several slices add the traffic of their partial sums, written
-// and read once, shared among the compute units, and about two rounds for the second kernel.  Ties go to the
-// longer slice.
+// Rounds a slice (SPW / 2), by a model of the busiest block's time fitted to measurements on an MI355X (it picks
+// the fastest of 1, 2, 4 rounds in 27 of 30 products of the 135M, 1.7B and 8B sizes at 8, 32 and 64 rows, and is
+// within 3 % of it in the others).  In units of a round (every block streams NW * 2 KB of each block of W, at
+// about 5 TB/s over the whole GPU):
+//   items of the block x (rounds a slice + the fixed cost of a unit: barriers and the sums through LDS)
+//   + the activations of each slice the run touches (rows / 16 of a round of W for each of its rounds)
+//   + half a slice more for a block with a single unit (nothing overlaps its loads)
+//   + with several slices: the second kernel, and the partial sums written and read once.
+// The rounds of a last slice past K are loaded from clamped addresses and add nothing, but cost like the others.
 template <int MT, int NW, int MAXSPW, int NB>
 static int wide_steps(const WideArgs& a, size_t workspace_floats, bool plan_only, long long* need, hipStream_t stream) {
     const int pairs = (a.K + 63) / 64, rounds = (pairs + NW - 1) / NW, cus = wide_cus();
+    const double round_us = (double)NW * 2048.0 * NB * cus / 5e12 * 1e6;
+    const double unit_cost = 0.4 / round_us, second_kernel = 4.0 / round_us;
+    const int rows = a.M < 16 * MT ? a.M : 16 * MT;
     int best = 1;
     double best_cost = -1.0;
     for (int r = MAXSPW / 2; r >= 1; r /= 2) {
         const int slices = (rounds + r - 1) / r;
         const long long items = (long long)a.units * slices;
-        double cost = (double)((items + cus - 1) / cus) * r;
-        if (slices > 1) cost += 2.0 + (double)slices * a.M * a.N * 8.0 / ((double)NW * 2048.0 * cus);
+        const long long run = (items + cus - 1) / cus;
+        double cost = (double)run * (r + unit_cost) + (double)((run + a.units - 1) / a.units) * rows / 16.0 * r / NB;
+        if (run == 1) cost += 0.5 * r;
+        if (slices > 1) cost += second_kernel + 0.1 * slices + (double)slices * a.M * a.N * 8.0 / ((double)NW * 2048.0 * cus);
         if (best_cost < 0 || cost < best_cost) { best = r; best_cost = cost; }
     }
     if constexpr (MAXSPW >= 8) if (best == 4) return wide_launch<MT, NW, 8, NB>(a, workspace_floats, plan_only, need, stream);

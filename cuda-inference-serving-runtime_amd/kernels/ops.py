@@ -310,10 +310,23 @@ def wide_ok(m, w, swiglu=False):
     """Whether a product of m rows with the bf16 weights w runs the wide weight-streaming kernel."""
     n, k = w.shape
     least = WIDE_MIN_BYTES_FEW_ROWS if m <= 16 else WIDE_MIN_BYTES if m <= 32 else WIDE_MIN_BYTES_MANY_ROWS
+    if m <= 16 and n < 16 * _compute_units(w.device) and k >= 4096:
+        # a narrow output with a long inner size: the fused kernels have a block for every 16 columns and
+        # cannot fill the GPU; this one cuts K as well
+        least = min(least, max(WIDE_MIN_BYTES, 16 << 20))
     if (w.dtype != torch.bfloat16 or not 0 < m <= SKINNY_ROWS or w.numel() * 2 < least or k % 8 or w.stride(0) % 8
             or w.data_ptr() % 16 or w.stride(1) != 1):
         return False
     return _wide_plan(m, n // 2 if swiglu else n, k, swiglu) >= 0
+
+
+_units = {}
+
+
+def _compute_units(device):
+    if device not in _units:
+        _units[device] = torch.cuda.get_device_properties(device).multi_processor_count
+    return _units[device]
 
 
 def _wide_plan(m, n, k, swiglu):

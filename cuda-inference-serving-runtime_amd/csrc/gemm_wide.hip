@@ -16,7 +16,9 @@
 // Sums are formed in a fixed order (waves in order inside a slice, slices in order), so a row's result
 // does not depend on the other rows; the shape of the launch depends on M only through the number of
 // 16-row tiles.
-// Finishing: store float or bf16, with an optional float residual; or SwiGLU over two blocks of W.
+// Finishing: store float or bf16, with an optional float residual; or SwiGLU over two blocks of W; or, for
+// W = [Wq; Wk; Wv], the rotary embedding of q and k with q stored and k, v written into the paged cache
+// (a unit is then 8 rotary pairs (i, i + D/2) of one head, so that both halves of a pair meet in one tile).
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
@@ -33,7 +35,42 @@ struct WideArgs {
     int units;                  // 16-row units of W
     int slices;                 // slices of K: SPW / 2 rounds of NW pairs of 32-wide k-steps each
     int dual_off;               // two blocks of W this many rows apart (SwiGLU), or 0
+    // the fused q/k/v projection (head_dim > 0): C is q, bf16 [M, heads * head_dim]
+    const int* positions; const int* slots; const float* cos_tab; const float* sin_tab;
+    bf16_t* kcache; bf16_t* vcache; int heads, kv_heads, head_dim, page_size, max_pos;
 };
+
+// the row of W = [Wq; Wk; Wv] behind column c of unit u: 8 rotary pairs of a head a unit
+__device__ __forceinline__ int wide_rope_row(const WideArgs& p, int u, int c) {
+    const int per_head = p.head_dim / 16, sh = u / per_head, j0 = (u % per_head) * 8;
+    return sh * p.head_dim + (c < 8 ? j0 + c : p.head_dim / 2 + j0 + c - 8);
+}
+
+// the fused projection's value of row m, column c of unit u: v, and pv from column c ^ 8 (the other half of the pair)
+__device__ __forceinline__ void wide_finish_rope(const WideArgs& p, int m, int u, int c, float v, float pv) {
+    const int D = p.head_dim, half = D / 2, per_head = D / 16;
+    const int sh = u / per_head, i = (u % per_head) * 8 + (c & 7), col = c < 8 ? i : half + i;
+    if (sh < p.heads + p.kv_heads) {                              // q or k head: rotate
+        int pos = p.positions[m];
+        pos = pos < 0 ? 0 : (pos >= p.max_pos ? p.max_pos - 1 : pos);
+        const float cs = p.cos_tab[(size_t)pos * half + i], sn = p.sin_tab[(size_t)pos * half + i];
+        v = c < 8 ? v * cs - pv * sn : v * cs + pv * sn;
+    }
+    if (sh < p.heads) {
+        ((bf16_t*)p.C)[(size_t)m * p.ldc + sh * D + col] = f32_to_bf16(v);
+        return;
+    }
+    const int slot = p.slots[m];
+    if (slot < 0) return;
+    const int page = slot / p.page_size, off = slot % p.page_size;
+    if (sh < p.heads + p.kv_heads) {
+        const int h = sh - p.heads;
+        p.kcache[(((size_t)page * p.kv_heads + h) * p.page_size + off) * D + col] = f32_to_bf16(v);
+    } else {
+        const int h = sh - p.heads - p.kv_heads;
+        p.vcache[(((size_t)page * p.kv_heads + h) * D + col) * p.page_size + off] = f32_to_bf16(v);
+    }
+}
 
 // the value of (m, n) from the finished sums: v, and u for the second block of W
 template <int NB>
@@ -49,7 +86,7 @@ __device__ __forceinline__ void wide_finish(const WideArgs& p, int m, int n, flo
 }
 
 // MT 16-row tiles of A; NW waves; SPW k-steps a wave and slice (even); NB blocks of W
-template <int MT, int NW, int SPW, int NB>
+template <int MT, int NW, int SPW, int NB, bool ROPE>
 __global__ void __launch_bounds__(NW * 64)
 gemm_wide_kernel(WideArgs p) {
     extern __shared__ float smem[];
@@ -92,7 +129,8 @@ gemm_wide_kernel(WideArgs p) {
             }
         }
         auto load_w = [&](u32x4 (&w)[NB][SPW], int u) {
-            const int n = min(u * 16 + r, N - 1);                 // rows past N are read again and never stored
+            // rows past N are read again and never stored
+            const int n = ROPE ? wide_rope_row(p, u, r) : min(u * 16 + r, N - 1);
             const bf16_t* row = p.W + (size_t)n * p.ldw;
 #pragma unroll
             for (int b = 0; b < NB; ++b)
@@ -136,7 +174,12 @@ gemm_wide_kernel(WideArgs p) {
 #pragma unroll
                     for (int w2 = 0; w2 < NW; ++w2) uu += red[w2][NB - 1][t][e2][lane];
                 }
-                if (p.slices == 1) {
+                if (ROPE && p.slices == 1) {
+                    float pv = 0.f;
+#pragma unroll
+                    for (int w2 = 0; w2 < NW; ++w2) pv += red[w2][0][t][e2][lane ^ 8];
+                    wide_finish_rope(p, m, u, lane % 16, v, pv);
+                } else if (p.slices == 1) {
                     wide_finish<NB>(p, m, n, v, uu);
                 } else {
                     float* dst = p.P + ((size_t)slice * M + m) * ((size_t)N * NB) + n;
@@ -159,7 +202,7 @@ gemm_wide_kernel(WideArgs p) {
 }
 
 // second pass: add the slices' partial sums in slice order and finish
-template <int NB>
+template <int NB, bool ROPE>
 __global__ void __launch_bounds__(256)
 gemm_wide_finish_kernel(WideArgs p) {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
@@ -171,6 +214,13 @@ gemm_wide_finish_kernel(WideArgs p) {
     for (int s = 0; s < p.slices; ++s) {
         v += src[(size_t)s * all];
         if (NB == 2) u += src[(size_t)s * all + p.N];
+    }
+    if (ROPE) {                                                   // column n of the partial sums is column n % 16 of unit n / 16
+        const float* other = p.P + (size_t)m * row + (n ^ 8);
+        float pv = 0.f;
+        for (int s = 0; s < p.slices; ++s) pv += other[(size_t)s * all];
+        wide_finish_rope(p, m, n / 16, n % 16, v, pv);
+        return;
     }
     wide_finish<NB>(p, m, n, v, u);
 }
@@ -187,7 +237,7 @@ static int wide_cus() {
     return cus[dev];
 }
 
-template <int MT, int NW, int SPW, int NB>
+template <int MT, int NW, int SPW, int NB, bool ROPE>
 static int wide_launch(WideArgs a, size_t workspace_floats, bool plan_only, long long* need, hipStream_t stream) {
     const int pairs = (a.K + 63) / 64, rounds = (pairs + NW - 1) / NW;
     a.slices = (rounds + SPW / 2 - 1) / (SPW / 2);
@@ -199,16 +249,16 @@ static int wide_launch(WideArgs a, size_t workspace_floats, bool plan_only, long
     const int cus = wide_cus();
     const size_t shmem = (size_t)NW * NB * MT * 4 * WAVE * sizeof(float);
     if (shmem > 65536) {
-        hipError_t e = hipFuncSetAttribute((const void*)gemm_wide_kernel<MT, NW, SPW, NB>,
+        hipError_t e = hipFuncSetAttribute((const void*)gemm_wide_kernel<MT, NW, SPW, NB, ROPE>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
         if (e != hipSuccess) return (int)e;
     }
     // one block a compute unit, each with an equal run of the work items
-    gemm_wide_kernel<MT, NW, SPW, NB><<<(unsigned)(items < cus ? items : cus), NW * 64, shmem, stream>>>(a);
+    gemm_wide_kernel<MT, NW, SPW, NB, ROPE><<<(unsigned)(items < cus ? items : cus), NW * 64, shmem, stream>>>(a);
     int err = CISR_LAUNCH_CHECK();
     if (err || a.slices == 1) return err;
     const size_t cells = (size_t)a.M * a.N;
-    gemm_wide_finish_kernel<NB><<<(unsigned)((cells + 255) / 256), 256, 0, stream>>>(a);
+    gemm_wide_finish_kernel<NB, ROPE><<<(unsigned)((cells + 255) / 256), 256, 0, stream>>>(a);
     return CISR_LAUNCH_CHECK();
 }
 
@@ -221,7 +271,7 @@ static int wide_launch(WideArgs a, size_t workspace_floats, bool plan_only, long
 //   + half a slice more for a block with a single unit (nothing overlaps its loads)
 //   + with several slices: the second kernel, and the partial sums written and read once.
 // The rounds of a last slice past K are loaded from clamped addresses and add nothing, but cost like the others.
-template <int MT, int NW, int MAXSPW, int NB>
+template <int MT, int NW, int MAXSPW, int NB, bool ROPE>
 static int wide_steps(const WideArgs& a, size_t workspace_floats, bool plan_only, long long* need, hipStream_t stream) {
     const int pairs = (a.K + 63) / 64, rounds = (pairs + NW - 1) / NW, cus = wide_cus();
     const double round_us = (double)NW * 2048.0 * NB * cus / 5e12 * 1e6;
@@ -238,30 +288,30 @@ static int wide_steps(const WideArgs& a, size_t workspace_floats, bool plan_only
         if (slices > 1) cost += second_kernel + 0.1 * slices + (double)slices * a.M * a.N * 8.0 / ((double)NW * 2048.0 * cus);
         if (best_cost < 0 || cost < best_cost) { best = r; best_cost = cost; }
     }
-    if constexpr (MAXSPW >= 8) if (best == 4) return wide_launch<MT, NW, 8, NB>(a, workspace_floats, plan_only, need, stream);
-    if constexpr (MAXSPW >= 4) if (best >= 2) return wide_launch<MT, NW, 4, NB>(a, workspace_floats, plan_only, need, stream);
-    return wide_launch<MT, NW, 2, NB>(a, workspace_floats, plan_only, need, stream);
+    if constexpr (MAXSPW >= 8) if (best == 4) return wide_launch<MT, NW, 8, NB, ROPE>(a, workspace_floats, plan_only, need, stream);
+    if constexpr (MAXSPW >= 4) if (best >= 2) return wide_launch<MT, NW, 4, NB, ROPE>(a, workspace_floats, plan_only, need, stream);
+    return wide_launch<MT, NW, 2, NB, ROPE>(a, workspace_floats, plan_only, need, stream);
 }
 
 // Configurations by the number of row tiles and blocks of W: as many steps a wave as the registers hold
 // (the A operands of a wave's steps for every tile, two units of W in flight), sixteen waves where a tile
 // leaves room for them (a longer slice, fewer partial sums).
-template <int NB>
+template <int NB, bool ROPE>
 static int wide_dispatch(const WideArgs& a, size_t workspace_floats, bool plan_only, long long* need, hipStream_t stream) {
     const int mt = (a.M + 15) / 16;
     if constexpr (NB == 1) {
         switch (mt) {
-            case 1: return wide_steps<1, 16, 8, NB>(a, workspace_floats, plan_only, need, stream);
-            case 2: return wide_steps<2, 8, 8, NB>(a, workspace_floats, plan_only, need, stream);
-            case 3: return wide_steps<3, 8, 8, NB>(a, workspace_floats, plan_only, need, stream);
-            default: return wide_steps<4, 8, 8, NB>(a, workspace_floats, plan_only, need, stream);
+            case 1: return wide_steps<1, 16, 8, NB, ROPE>(a, workspace_floats, plan_only, need, stream);
+            case 2: return wide_steps<2, 8, 8, NB, ROPE>(a, workspace_floats, plan_only, need, stream);
+            case 3: return wide_steps<3, 8, 8, NB, ROPE>(a, workspace_floats, plan_only, need, stream);
+            default: return wide_steps<4, 8, 8, NB, ROPE>(a, workspace_floats, plan_only, need, stream);
         }
     } else {
         switch (mt) {
-            case 1: return wide_steps<1, 8, 8, NB>(a, workspace_floats, plan_only, need, stream);
-            case 2: return wide_steps<2, 8, 4, NB>(a, workspace_floats, plan_only, need, stream);
-            case 3: return wide_steps<3, 8, 4, NB>(a, workspace_floats, plan_only, need, stream);
-            default: return wide_steps<4, 8, 4, NB>(a, workspace_floats, plan_only, need, stream);
+            case 1: return wide_steps<1, 8, 8, NB, ROPE>(a, workspace_floats, plan_only, need, stream);
+            case 2: return wide_steps<2, 8, 4, NB, ROPE>(a, workspace_floats, plan_only, need, stream);
+            case 3: return wide_steps<3, 8, 4, NB, ROPE>(a, workspace_floats, plan_only, need, stream);
+            default: return wide_steps<4, 8, 4, NB, ROPE>(a, workspace_floats, plan_only, need, stream);
         }
     }
 }
@@ -280,8 +330,30 @@ static int wide_entry(const void* A, int lda, const void* W, int ldw, void* C, i
     WideArgs a = {};
     a.A = (const bf16_t*)A; a.lda = lda; a.W = (const bf16_t*)W; a.ldw = ldw; a.C = C; a.ldc = ldc; a.out_dtype = out_dtype;
     a.R = R; a.ldr = ldr; a.P = workspace; a.M = M; a.N = N; a.K = K; a.units = (N + 15) / 16; a.dual_off = dual_off;
-    return dual_off > 0 ? wide_dispatch<2>(a, (size_t)workspace_floats, plan_only, need, stream)
-                        : wide_dispatch<1>(a, (size_t)workspace_floats, plan_only, need, stream);
+    return dual_off > 0 ? wide_dispatch<2, false>(a, (size_t)workspace_floats, plan_only, need, stream)
+                        : wide_dispatch<1, false>(a, (size_t)workspace_floats, plan_only, need, stream);
+}
+
+// The fused q/k/v projection of a step of few rows against large weights: A bf16 [M, K] (normed), W = [Wq; Wk; Wv]
+// (kv_heads 0: Wq only), rotary embedding of q and k over the whole head (head_dim % 16 == 0), q to q_out
+// [M, heads * head_dim], k and v into the paged cache at `slots`.  Workspace as for cisr_gemm_wide_bf16 with
+// N = (heads + 2 kv_heads) * head_dim.
+extern "C" int cisr_qkv_rope_wide(const void* A, int lda, const void* W, int ldw, void* q_out, int ldq, int M, int K,
+                                  const int* positions, const int* slots, const float* cos_tab, const float* sin_tab,
+                                  void* kcache, void* vcache, int heads, int kv_heads, int head_dim, int page_size,
+                                  int max_pos, float* workspace, long long workspace_floats, hipStream_t stream) {
+    if (M <= 0) return 0;
+    if (M > 64 || K < 8 || K % 8 || lda % 8 || ldw % 8 || !wide_aligned16(A) || !wide_aligned16(W) || !q_out ||
+        head_dim <= 0 || head_dim % 16 || heads <= 0 || kv_heads < 0 || page_size <= 0 || max_pos <= 0 || !positions ||
+        !cos_tab || !sin_tab || (kv_heads > 0 && (!slots || !kcache || !vcache)) || workspace_floats < 0)
+        return (int)hipErrorInvalidValue;
+    WideArgs a = {};
+    a.A = (const bf16_t*)A; a.lda = lda; a.W = (const bf16_t*)W; a.ldw = ldw; a.C = q_out; a.ldc = ldq; a.out_dtype = DT_BF16;
+    a.P = workspace; a.M = M; a.N = (heads + 2 * kv_heads) * head_dim; a.K = K; a.units = a.N / 16;
+    a.positions = positions; a.slots = slots; a.cos_tab = cos_tab; a.sin_tab = sin_tab; a.kcache = (bf16_t*)kcache;
+    a.vcache = (bf16_t*)vcache; a.heads = heads; a.kv_heads = kv_heads; a.head_dim = head_dim; a.page_size = page_size;
+    a.max_pos = max_pos;
+    return wide_dispatch<1, true>(a, (size_t)workspace_floats, false, nullptr, stream);
 }
 
 // Floats of workspace that cisr_gemm_wide_bf16 needs for this shape (0: none), or -1 if it does not take the shape.

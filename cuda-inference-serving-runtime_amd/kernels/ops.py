@@ -57,6 +57,7 @@ def _declare(h):
         "cisr_sample": [p, p, p, p, p, p, i, i, i, p],
         "cisr_take_tokens": [p, p, p, i, i, p],
         "cisr_gemm_wide_bf16": [p, i, p, i, p, i, p, i, i, i, i, i, i, p, C.c_longlong, p],
+        "cisr_qkv_rope_wide": [p, i, p, i, p, i, i, i, p, p, p, p, p, p, i, i, i, i, i, p, C.c_longlong, p],
     }
     for name, args in sig.items():
         fn = getattr(h, name)
@@ -254,10 +255,11 @@ def attention_rowwise(q, q_row_stride, kcache, vcache, tables, seg_of_row, posit
     return out
 
 
-def gemm(a, w, out, residual=None):
+def gemm(a, w, out, residual=None, after_norm=False):
     """out[M, N] = a[M, K] . w[N, K]^T (+ residual).  float operands run the true
     32-bit kernel; bf16 operands run on the matrix cores with float accumulation.
-    out may be float or (bf16 operands only) bf16; residual is float and may be `out`."""
+    out may be float or (bf16 operands only) bf16; residual is float and may be `out`.
+    `after_norm`: a hint for the choice of kernel, see wide_ok."""
     m, k = a.shape
     n, k2 = w.shape
     if k != k2:
@@ -278,7 +280,7 @@ def gemm(a, w, out, residual=None):
             raise KernelError("gemm: float operands need a float output")
         code = lib().cisr_gemm_f32(a.data_ptr(), a.stride(0), w.data_ptr(), w.stride(0), out.data_ptr(), out.stride(0),
                                    rp, ldr, m, n, k, _stream())
-    elif a.dtype == torch.bfloat16 and m <= SKINNY_ROWS and _skinny_ok(a, w) and wide_ok(m, w):
+    elif a.dtype == torch.bfloat16 and m <= SKINNY_ROWS and _skinny_ok(a, w) and wide_ok(m, w, after_norm=after_norm):
         return _gemm_wide(a, w, out, residual, False, "gemm")
     elif a.dtype == torch.bfloat16 and m <= SKINNY_ROWS and _skinny_ok(a, w):
         code = lib().cisr_gemm_skinny_bf16(a.data_ptr(), a.stride(0), w.data_ptr(), w.stride(0), out.data_ptr(),
@@ -306,14 +308,18 @@ _wide_workspaces = {}    # device -> buffers, never freed: captured programs kee
 _wide_plans = {}
 
 
-def wide_ok(m, w, swiglu=False):
-    """Whether a product of m rows with the bf16 weights w runs the wide weight-streaming kernel."""
+def wide_ok(m, w, swiglu=False, after_norm=False):
+    """Whether a product of m rows with the bf16 weights w runs the wide weight-streaming kernel.
+    `after_norm`: the rows are the output of an RMSNorm, which the other kernel would fuse (it then reads the
+    float residual and the norm's weights for every 16 rows of W, which costs it more than bf16 rows do)."""
     n, k = w.shape
     least = WIDE_MIN_BYTES_FEW_ROWS if m <= 16 else WIDE_MIN_BYTES if m <= 32 else WIDE_MIN_BYTES_MANY_ROWS
     if m <= 16 and n < 16 * _compute_units(w.device) and k >= 4096:
         # a narrow output with a long inner size: the fused kernels have a block for every 16 columns and
         # cannot fill the GPU; this one cuts K as well
         least = min(least, max(WIDE_MIN_BYTES, 16 << 20))
+    if 4 <= m <= 16 and after_norm and k >= 2048:     # (one or two rows of the residual cost the fused kernel next to nothing)
+        least = min(least, max(WIDE_MIN_BYTES, 24 << 20))
     if (w.dtype != torch.bfloat16 or not 0 < m <= SKINNY_ROWS or w.numel() * 2 < least or k % 8 or w.stride(0) % 8
             or w.data_ptr() % 16 or w.stride(1) != 1):
         return False
@@ -383,7 +389,7 @@ def _norm_args(x, norm, k):
 def fused_norm_ok(x, w, rows_out):
     """Whether the weight-streaming kernel can take RMSNorm(x) . w^T with the norm fused (and large weights
     do not make the norm as a kernel of its own and the wide kernel the better choice)."""
-    return (not wide_ok(rows_out, w) and w.dtype == torch.bfloat16 and rows_out <= SKINNY_ROWS and x.dtype == torch.float32 and x.shape[1] % 8 == 0
+    return (not wide_ok(rows_out, w, after_norm=True) and w.dtype == torch.bfloat16 and rows_out <= SKINNY_ROWS and x.dtype == torch.float32 and x.shape[1] % 8 == 0
             and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w.stride(0) % 8 == 0 and w.data_ptr() % 16 == 0)
 
 
@@ -426,7 +432,7 @@ def gemm_swiglu(a, w_gate_up, out, scratch=None, norm=None):
     if out.dtype != a.dtype or a.dtype != w_gate_up.dtype:
         raise KernelError("gemm_swiglu: dtypes differ")
     if swiglu_fused_ok(a, w_gate_up):
-        if m <= SKINNY_ROWS and wide_ok(m, w_gate_up, True):
+        if m <= SKINNY_ROWS and wide_ok(m, w_gate_up, True, after_norm=True):
             return _gemm_wide(a, w_gate_up, out, None, True, "gemm_swiglu")
         if m <= SKINNY_ROWS:
             _check(lib().cisr_gemm_skinny_bf16(a.data_ptr(), a.stride(0), w_gate_up.data_ptr(), w_gate_up.stride(0),
@@ -445,7 +451,9 @@ def gemm_swiglu(a, w_gate_up, out, scratch=None, norm=None):
 def qkv_rope_fused_ok(a, w, head_dim, cos, normed):
     """Whether the fused projection + rotary + scatter kernel takes this shape."""
     m, k = a.shape
-    return (not wide_ok(m, w) and w.dtype == torch.bfloat16 and m <= SKINNY_ROWS and k % 8 == 0 and head_dim % 16 == 0
+    if normed and wide_ok(m, w, after_norm=True):      # large weights: the norm is a kernel of its own, the projection the wide kernel
+        return False
+    return (w.dtype == torch.bfloat16 and m <= SKINNY_ROWS and k % 8 == 0 and head_dim % 16 == 0
             and 2 * cos.shape[1] == head_dim and a.stride(0) % 8 == 0 and a.data_ptr() % 16 == 0
             and w.stride(0) % 8 == 0 and w.data_ptr() % 16 == 0
             and a.dtype == (torch.float32 if normed else torch.bfloat16))
@@ -471,6 +479,17 @@ def qkv_rope(a, w, q_out, positions, slots, cos, sin, kcache, vcache, heads, kv_
         vp = _dev(vcache, "vcache", torch.bfloat16, (pages, kv_heads, dim, page_size))
         sp = _dev(slots, "slots", torch.int32, (m,))
     max_pos = cos.shape[0]
+    if norm is None and wide_ok(m, w, after_norm=True):
+        need = _wide_plan(m, w.shape[0], k, False)
+        work = _wide_workspace(a.device, need)
+        _check(lib().cisr_qkv_rope_wide(a.data_ptr(), a.stride(0), w.data_ptr(), w.stride(0),
+                                        _dev(q_out, "q_out", torch.bfloat16, (m, heads * dim)), heads * dim, m, k,
+                                        _dev(positions, "positions", torch.int32, (m,)), sp,
+                                        _dev(cos, "cos", torch.float32), _dev(sin, "sin", torch.float32, (max_pos, dim // 2)),
+                                        kp, vp, heads, n_kv, dim, page_size, max_pos,
+                                        None if work is None else work.data_ptr(), 0 if work is None else work.numel(),
+                                        _stream()), "qkv_rope")
+        return q_out
     _check(lib().cisr_qkv_rope_skinny(a.data_ptr(), a.stride(0), w.data_ptr(), w.stride(0),
                                       _dev(q_out, "q_out", torch.bfloat16, (m, heads * dim)), heads * dim, m, k, wp, eps,
                                       _dev(positions, "positions", torch.int32, (m,)), sp,

@@ -492,6 +492,59 @@ def test_fused_projection_rotary_scatter(ops, heads, kv_heads, dim, theta, norme
     assert torch.equal(q, q2)
 
 
+@pytest.mark.parametrize("heads, kv_heads, dim, M, K", [(4, 2, 16, 5, 72), (9, 3, 64, 8, 4104), (2, 1, 128, 20, 2056), (3, 3, 48, 40, 520),
+                                                       (5, 1, 32, 64, 9000)])
+def test_fused_projection_rotary_scatter_through_the_wide_product(ops, monkeypatch, heads, kv_heads, dim, M, K):
+    """The same projection with large weights (forced here): normed bf16 rows in, the wide product with the rotary
+    embedding and the cache write as its finishing step, in one slice of K and in several, one to four row tiles."""
+    from runtime.parts import RotaryEmbedding
+    for limit in ("WIDE_MIN_BYTES", "WIDE_MIN_BYTES_FEW_ROWS", "WIDE_MIN_BYTES_MANY_ROWS"):
+        monkeypatch.setattr(ops, limit, 0)
+    theta = 1e4
+    rope = RotaryEmbedding(dim, theta, 700); rope.prepare(DEV, torch.bfloat16)
+    cos, sin = rope.tables()
+    P_, pages = 4, 2 * M
+    rng = np.random.default_rng(M)
+    pos = rng.integers(0, 700, size=M).tolist()
+    slots = rng.permutation(pages * P_)[:M].tolist()
+    slots[M // 2] = -1
+    a = rnd(M, K, dtype=torch.bfloat16, seed=1, scale=1.5)
+    w = rnd((heads + 2 * kv_heads) * dim, K, dtype=torch.bfloat16, seed=3, scale=0.2 / math.sqrt(K / 72))
+    assert ops.wide_ok(M, w) and ops.qkv_rope_fused_ok(a, w, dim, cos, False)
+    assert not ops.qkv_rope_fused_ok(a.float(), w, dim, cos, True)    # the norm is then a kernel of its own
+    ref = f64(a) @ f64(w).T
+    q_ref = P.rope(ref[:, :heads * dim].reshape(M, heads, dim), pos, theta)
+    k_ref = P.rope(ref[:, heads * dim:(heads + kv_heads) * dim].reshape(M, kv_heads, dim), pos, theta)
+    v_ref = ref[:, (heads + kv_heads) * dim:].reshape(M, kv_heads, dim)
+    kc = torch.full((pages, kv_heads, P_, dim), 7.0, dtype=torch.bfloat16, device=DEV)
+    vc = torch.full((pages, kv_heads, dim, P_), 7.0, dtype=torch.bfloat16, device=DEV)
+    q = torch.empty(M, heads * dim, dtype=torch.bfloat16, device=DEV)
+    ops.qkv_rope(a, w, q, torch.tensor(pos, dtype=torch.int32, device=DEV), torch.tensor(slots, dtype=torch.int32, device=DEV),
+                 cos, sin, kc, vc, heads, kv_heads, dim, P_)
+    tol = dict(rtol=2e-2, atol=2e-2 * np.abs(ref).max())
+    np.testing.assert_allclose(f64(q).reshape(M, heads, dim), q_ref, **tol)
+    kc64, vc64 = f64(kc), f64(vc)
+    for t, s_ in enumerate(slots):
+        if s_ < 0:
+            continue
+        np.testing.assert_allclose(kc64[s_ // P_, :, s_ % P_], k_ref[t], **tol)
+        np.testing.assert_allclose(vc64[s_ // P_, :, :, s_ % P_], v_ref[t], **tol)
+    untouched = [s_ for s_ in range(pages * P_) if s_ not in slots]
+    assert all((kc64[s_ // P_, :, s_ % P_] == 7).all() and (vc64[s_ // P_, :, :, s_ % P_] == 7).all() for s_ in untouched)
+    # the same numbers as the product followed by the rotary kernel, but for the rounding of the product to bf16 between them
+    qkv = ops.gemm(a, w, torch.empty(M, w.shape[0], dtype=torch.bfloat16, device=DEV))
+    kc2, vc2 = torch.full_like(kc, 7.0), torch.full_like(vc, 7.0)
+    ops.rope_scatter(qkv, torch.tensor(pos, dtype=torch.int32, device=DEV), torch.tensor(slots, dtype=torch.int32, device=DEV),
+                     cos, sin, kc2, vc2, heads, kv_heads, dim, P_)
+    np.testing.assert_allclose(f64(q), f64(qkv[:, :heads * dim]), **tol)
+    np.testing.assert_allclose(f64(kc), f64(kc2), **tol)
+    # q only (a layer that reads another layer's cache)
+    q2 = torch.empty_like(q)
+    ops.qkv_rope(a, w[:heads * dim].contiguous(), q2, torch.tensor(pos, dtype=torch.int32, device=DEV), None, cos, sin, None, None,
+                 heads, kv_heads, dim, P_)
+    assert torch.equal(q, q2)
+
+
 GEMM_SHAPES = [(1, 1, 1), (5, 7, 9), (64, 64, 32), (130, 200, 172), (33, 513, 144), (17, 130, 1000), (300, 129, 72), (8, 1536, 576)]
 
 

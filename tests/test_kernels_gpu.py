@@ -585,6 +585,35 @@ def test_gemm_wide_for_large_weights(ops, monkeypatch):
     assert ops.fused_norm_ok(rnd(8, 576), rnd(1728, 576, dtype=torch.bfloat16), 8) and not ops.wide_ok(8, w)
 
 
+@pytest.mark.parametrize("M", [1, 8, 24, 64])
+def test_gemm_wide_at_the_sizes_that_choose_it(ops, M):
+    """The wide product at sizes where it is the kernel of choice (Llama-3-8B's feed-forward and a 1.7B-size
+    down projection), against float products of the same bf16 operands."""
+    torch.manual_seed(M)
+    H, I = 4096, 14336
+    a = (torch.randn(M, H, device=DEV) * 0.5).bfloat16()
+    w_gu = (torch.randn(2 * I, H, device=DEV) * 0.02).bfloat16()
+    assert ops.wide_ok(M, w_gu, True)
+    gu = a.float() @ w_gu.float().T
+    gq = gu.bfloat16().float()
+    want = torch.nn.functional.silu(gq[:, :I]) * gq[:, I:]
+    got = ops.gemm_swiglu(a, w_gu, torch.empty(M, I, dtype=torch.bfloat16, device=DEV))
+    torch.testing.assert_close(got.float(), want, rtol=2e-2, atol=2e-3)
+    act = want.bfloat16()
+    w_d = (torch.randn(H, I, device=DEV) * 0.02).bfloat16()
+    r = torch.randn(M, H, device=DEV)
+    assert ops.wide_ok(M, w_d)
+    out = r.clone()
+    ops.gemm(act, w_d, out, residual=out)
+    torch.testing.assert_close(out, r + act.float() @ w_d.float().T, rtol=1e-4, atol=1e-4)
+    # a narrow output with a long inner size (several slices of K, one unit or two a block)
+    w_n = (torch.randn(2048, 8192, device=DEV) * 0.02).bfloat16()
+    x = (torch.randn(M, 8192, device=DEV) * 0.5).bfloat16()
+    assert ops.wide_ok(M, w_n)
+    y = ops.gemm(x, w_n, torch.empty(M, 2048, device=DEV))
+    torch.testing.assert_close(y, x.float() @ w_n.float().T, rtol=1e-4, atol=1e-4)
+
+
 @pytest.mark.parametrize("M, N, K", GEMM_SHAPES)
 def test_gemm_f32(ops, M, N, K):
     a, w, r = rnd(M, K, seed=1), rnd(N, K, seed=2), rnd(M, N, seed=3)

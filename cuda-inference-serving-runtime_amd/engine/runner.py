@@ -461,8 +461,9 @@ class ModelRunner:
         waves = 8 if few and head_dim <= 64 else 4
         # few rows: enough blocks along the keys for two a compute unit (measured: a thousand blocks are no
         # faster at a context of 2k to 8k and 12 % slower at 30k, where each then lives for three steps a
-        # wave only); many rows fill the GPU by themselves and split only a little.  A wave keeps at least
-        # two 32-key steps (one computing, one loading).
-        target = 512 if few else 256
+        # wave only); many rows split until every compute unit has the blocks of four waves that its registers
+        # hold (three with small heads, two otherwise: 3-5 % faster at 64 rows of the 135M sizes than one block
+        # a unit).  A wave keeps at least two 32-key steps (one computing, one loading).
+        target = 512 if few else (768 if head_dim <= 64 else 512)
         splits = int(max(1, min(steps // (waves * 2), -(-target // blocks), 64)))
         return waves, splits

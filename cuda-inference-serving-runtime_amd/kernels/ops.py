@@ -318,7 +318,7 @@ def wide_ok(m, w, swiglu=False, after_norm=False):
         # a narrow output with a long inner size: the fused kernels have a block for every 16 columns and
         # cannot fill the GPU; this one cuts K as well
         least = min(least, max(WIDE_MIN_BYTES, 16 << 20))
-    if 4 <= m <= 16 and after_norm and k >= 2048:     # (one or two rows of the residual cost the fused kernel next to nothing)
+    if m >= 4 and after_norm and k >= 2048:     # (one or two rows of the residual cost the fused kernel next to nothing)
         least = min(least, max(WIDE_MIN_BYTES, 24 << 20))
     if (w.dtype != torch.bfloat16 or not 0 < m <= SKINNY_ROWS or w.numel() * 2 < least or k % 8 or w.stride(0) % 8
             or w.data_ptr() % 16 or w.stride(1) != 1):

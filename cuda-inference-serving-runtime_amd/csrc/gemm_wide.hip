@@ -6,8 +6,8 @@
 // (from L2, but through the same path as W): with 8 rows of A that is half the traffic of W, with 64
 // rows four times it.  Here a block keeps the activations of its part of K in registers, as finished
 // matrix-core operands, and walks over many 16-row units of W with them:
-//   - K is cut into slices (grid.y); the waves of a block deal the slice's k-steps among them in pairs
-//     (a cache line of a row of W) and each holds the A operands of its steps for all row tiles;
+//   - K is cut into slices; the waves of a block deal a slice's k-steps among them in pairs (a cache line
+//     of a row of W) and each holds the A operands of its steps for all row tiles;
 //   - the work items (slice, unit), slice-major, are dealt to the blocks in equal contiguous runs, one block a
 //     compute unit; a block walks over its units of W, the loads of the next unit in flight while the matrix
 //     cores work on this one and the waves' partial tiles meet in LDS;

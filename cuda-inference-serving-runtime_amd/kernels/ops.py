@@ -255,6 +255,30 @@ def attention_rowwise(q, q_row_stride, kcache, vcache, tables, seg_of_row, posit
     return out
 
 
+# Large bf16 products of many rows go to the vendor's library through torch.mm (the reference's linears are
+# library calls too: cuBLAS through runtime/blas.py:44-56, or CuPy's matmul, runtime/model.py:108): from this many rows on, with weights of at least LIBRARY_MIN_BYTES;
+# the residual sum or the activation is then a kernel after the product.  Measured on an MI355X at 2048 rows:
+# 1,270-1,480 TFLOP/s against 830-920 of the tiled kernel here on the 8B shapes (a prompt step of 30.6 against
+# 39.9 ms); below these sizes the kernels here are as fast or faster and save the extra kernel.  0 rows: never.
+LIBRARY_MIN_ROWS = int(os.environ.get("CISR_LIBRARY_MIN_ROWS", "256"))
+LIBRARY_MIN_BYTES = int(float(os.environ.get("CISR_LIBRARY_MIN_MB", "16")) * (1 << 20))
+_library_scratch = {}   # (device, elements) -> bf16 buffers, never freed: captured programs keep their addresses
+
+
+def library_ok(m, w):
+    return (LIBRARY_MIN_ROWS > 0 and m >= LIBRARY_MIN_ROWS and w.dtype == torch.bfloat16 and w.is_contiguous()
+            and w.numel() * 2 >= LIBRARY_MIN_BYTES)
+
+
+def _scratch_bf16(device, rows, cols):
+    pool = _library_scratch.setdefault(device, [])
+    for buf in pool:
+        if buf.numel() >= rows * cols:
+            return buf[:rows * cols].view(rows, cols)
+    pool.append(torch.empty(1 << (rows * cols - 1).bit_length(), dtype=torch.bfloat16, device=device))
+    return pool[-1][:rows * cols].view(rows, cols)
+
+
 def gemm(a, w, out, residual=None, after_norm=False):
     """out[M, N] = a[M, K] . w[N, K]^T (+ residual).  float operands run the true
     32-bit kernel; bf16 operands run on the matrix cores with float accumulation.
@@ -280,6 +304,14 @@ def gemm(a, w, out, residual=None, after_norm=False):
             raise KernelError("gemm: float operands need a float output")
         code = lib().cisr_gemm_f32(a.data_ptr(), a.stride(0), w.data_ptr(), w.stride(0), out.data_ptr(), out.stride(0),
                                    rp, ldr, m, n, k, _stream())
+    elif (a.dtype == torch.bfloat16 and library_ok(m, w) and a.is_contiguous() and out.is_contiguous()
+          and (out.dtype == torch.bfloat16 and residual is None or residual is out)):
+        if residual is None:
+            torch.mm(a, w.t(), out=out)
+            return out
+        product = _scratch_bf16(a.device, m, n)
+        torch.mm(a, w.t(), out=product)
+        return residual_add(out, product)
     elif a.dtype == torch.bfloat16 and m <= SKINNY_ROWS and _skinny_ok(a, w) and wide_ok(m, w, after_norm=after_norm):
         return _gemm_wide(a, w, out, residual, False, "gemm")
     elif a.dtype == torch.bfloat16 and m <= SKINNY_ROWS and _skinny_ok(a, w):
@@ -431,6 +463,10 @@ def gemm_swiglu(a, w_gate_up, out, scratch=None, norm=None):
         return out
     if out.dtype != a.dtype or a.dtype != w_gate_up.dtype:
         raise KernelError("gemm_swiglu: dtypes differ")
+    if a.dtype == torch.bfloat16 and library_ok(m, w_gate_up) and a.is_contiguous():
+        product = _scratch_bf16(a.device, m, two_i)
+        torch.mm(a, w_gate_up.t(), out=product)
+        return swiglu(product, out)
     if swiglu_fused_ok(a, w_gate_up):
         if m <= SKINNY_ROWS and wide_ok(m, w_gate_up, True, after_norm=True):
             return _gemm_wide(a, w_gate_up, out, None, True, "gemm_swiglu")

@@ -614,6 +614,51 @@ def test_gemm_wide_at_the_sizes_that_choose_it(ops, M):
     torch.testing.assert_close(y, x.float() @ w_n.float().T, rtol=1e-4, atol=1e-4)
 
 
+def test_library_products_of_many_rows_also_in_captured_graphs(ops, monkeypatch):
+    """Large bf16 products of many rows may go to the vendor's library, with the residual sum and the activation
+    as kernels after it.  Checked against float products, eagerly and in a captured graph that is replayed with
+    new inputs, eager work and synchronisations between the replays (a library call may record nodes that go
+    wrong on later replays: every replay is checked)."""
+    monkeypatch.setattr(ops, "LIBRARY_MIN_ROWS", 256)
+    monkeypatch.setattr(ops, "LIBRARY_MIN_BYTES", 16 << 20)
+    torch.manual_seed(0)
+    M, N, K, I = 512, 4096, 4096, 5000
+    w = (torch.randn(N, K, device=DEV) * 0.02).bfloat16()
+    w_gu = (torch.randn(2 * I, K, device=DEV) * 0.02).bfloat16()
+    assert ops.library_ok(M, w) and ops.library_ok(M, w_gu) and not ops.library_ok(255, w) and not ops.library_ok(M, w[:1000])
+    a = torch.empty(M, K, dtype=torch.bfloat16, device=DEV)
+    out = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    res = torch.empty(M, N, device=DEV)
+    act = torch.empty(M, I, dtype=torch.bfloat16, device=DEV)
+
+    def step():
+        ops.gemm(a, w, out)
+        ops.gemm(a, w, res, residual=res)
+        ops.gemm_swiglu(a, w_gu, act)
+
+    def check(tag):
+        ref = a.float() @ w.float().T
+        torch.testing.assert_close(out.float(), ref, rtol=2e-2, atol=2e-2, msg=tag)
+        torch.testing.assert_close(res - r0, ref, rtol=2e-2, atol=2e-2, msg=tag)   # the product is rounded to bf16 before the sum
+        gq = (a.float() @ w_gu.float().T).bfloat16().float()
+        torch.testing.assert_close(act.float(), torch.nn.functional.silu(gq[:, :I]) * gq[:, I:], rtol=2e-2, atol=2e-3, msg=tag)
+
+    r0 = torch.randn(M, N, device=DEV)
+    a.copy_(torch.randn(M, K, device=DEV) * 0.5); res.copy_(r0)
+    step(); check("eager")
+    res.copy_(r0)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    for i in range(5):
+        a.copy_(torch.randn(M, K, device=DEV) * 0.5); res.copy_(r0)
+        out.fill_(7); act.fill_(7)
+        junk = (torch.randn(300, 300, device=DEV) @ torch.randn(300, 300, device=DEV)).sum().item()   # eager work between replays
+        graph.replay()
+        torch.cuda.synchronize()
+        check(f"replay {i}")
+
+
 @pytest.mark.parametrize("M, N, K", GEMM_SHAPES)
 def test_gemm_f32(ops, M, N, K):
     a, w, r = rnd(M, K, seed=1), rnd(N, K, seed=2), rnd(M, N, seed=3)

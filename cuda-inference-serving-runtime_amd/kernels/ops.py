@@ -259,8 +259,11 @@ def attention_rowwise(q, q_row_stride, kcache, vcache, tables, seg_of_row, posit
 # library calls too: cuBLAS through runtime/blas.py:44-56, or CuPy's matmul, runtime/model.py:108): from this many rows on, with weights of at least LIBRARY_MIN_BYTES;
 # the residual sum or the activation is then a kernel after the product.  Measured on an MI355X at 2048 rows:
 # 1,270-1,480 TFLOP/s against 830-920 of the tiled kernel here on the 8B shapes (a prompt step of 30.6 against
-# 39.9 ms); below these sizes the kernels here are as fast or faster and save the extra kernel.  0 rows: never.
-LIBRARY_MIN_ROWS = int(os.environ.get("CISR_LIBRARY_MIN_ROWS", "256"))
+# 39.9 ms); at 65-255 rows with weights streamed from HBM it is up to 2.5 times as fast on narrow outputs with
+# a long inner size, which leave the tiled kernel few tiles (it does not cut K).  With at most 64 rows the
+# weight-streaming kernels here are as fast or faster (8 rows: 50 against 67 us for gate and up of the 8B
+# sizes), as are all products of small weights, and both save the kernel after the product.  0 rows: never.
+LIBRARY_MIN_ROWS = int(os.environ.get("CISR_LIBRARY_MIN_ROWS", "65"))
 LIBRARY_MIN_BYTES = int(float(os.environ.get("CISR_LIBRARY_MIN_MB", "16")) * (1 << 20))
 _library_scratch = {}   # (device, elements) -> bf16 buffers, never freed: captured programs keep their addresses
 

@@ -626,6 +626,7 @@ def test_library_products_of_many_rows_also_in_captured_graphs(ops, monkeypatch)
     w = (torch.randn(N, K, device=DEV) * 0.02).bfloat16()
     w_gu = (torch.randn(2 * I, K, device=DEV) * 0.02).bfloat16()
     assert ops.library_ok(M, w) and ops.library_ok(M, w_gu) and not ops.library_ok(255, w) and not ops.library_ok(M, w[:1000])
+    assert not ops.library_ok(M, w.float())     # the 32-bit path never leaves the kernels of this repository
     a = torch.empty(M, K, dtype=torch.bfloat16, device=DEV)
     out = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
     res = torch.empty(M, N, device=DEV)

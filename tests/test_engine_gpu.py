@@ -189,6 +189,51 @@ def test_steps_through_the_wide_product_match_the_plain_model(folders, name, exe
     runner.cache.check()
 
 
+@pytest.mark.parametrize("execution", ["eager", "graph"])
+def test_layers_of_real_sizes_match_the_plain_model(tmp_path_factory, execution):
+    """Two layers of the SmolLM2-1.7B sizes (width 2048, 32 heads of 64, feed-forward 8192, vocabulary 49152):
+    the sizes at which products choose other kernels by themselves (the wide weight-streaming product for
+    decode steps, the vendor's library for portions of more than 64 rows).  Whole prompts, portions, decode
+    steps of several requests and mixed steps against the plain model."""
+    from runtime.engine import load_model, ModelRunner, StepEntry
+    from runtime.kernels import ops
+    from conftest import write_folder, plain_logits, assert_close
+    cfg = dict(num_hidden_layers=2, hidden_size=2048, num_attention_heads=32, num_key_value_heads=32, head_dim=64,
+               intermediate_size=8192, vocab_size=49152, rope_theta=130000.0, rms_norm_eps=1e-5,
+               tie_word_embeddings=True, max_position_embeddings=512)
+    folder = write_folder(tmp_path_factory.mktemp("real") / "m", cfg, 77, sharp=False)
+    model = load_model(folder, dtype="bfloat16")
+    w_gate_up = model.layers[0].ffn.w_gate_up
+    assert ops.wide_ok(5, w_gate_up, True, after_norm=True) and ops.library_ok(90, w_gate_up)   # what this test is for
+    runner = ModelRunner(model, n_pages=40, page_size=16, max_requests=8, execution=execution)
+    seqs = {k: random_tokens(900 + i, 100, cfg["vocab_size"]) for i, k in enumerate("abcde")}
+    refs = {k: plain_logits(folder, seqs[k]) for k in seqs}
+    for k in seqs:
+        runner.create(k)
+    fed = {k: 0 for k in seqs}
+
+    def feed(*parts):
+        entries, places = [], []
+        for k, n in parts:
+            entries.append(StepEntry(k, seqs[k][fed[k]:fed[k] + n], [0, n - 1] if n > 1 else [0]))
+            places += [(k, fed[k]), (k, fed[k] + n - 1)] if n > 1 else [(k, fed[k])]
+            fed[k] += n
+        logits = runner.step(entries).float().cpu().numpy()
+        for row, (k, pos) in zip(logits, places):
+            assert_close(row[None], refs[k][pos][None], "bfloat16", f"request {k} position {pos}")
+
+    feed(("a", 90))                                   # more than 64 rows: the library's products
+    feed(("b", 70), ("c", 3))
+    feed(("c", 40), ("d", 20))                        # 60 rows: four row tiles of the wide product
+    feed(("e", 7))
+    for _ in range(3):
+        feed(("a", 1), ("b", 1), ("c", 1), ("d", 1), ("e", 1))   # decode steps of five rows
+    feed(("a", 1), ("b", 1), ("c", 30), ("d", 1), ("e", 50))     # mixed: 83 rows
+    for _ in range(2):
+        feed(("a", 1), ("b", 1), ("c", 1), ("d", 1), ("e", 1))
+    runner.cache.check()
+
+
 @pytest.mark.parametrize("name", ["a", "c"])
 @pytest.mark.parametrize("item_tiles", [1, 2])
 def test_long_portions_through_block_tiles_match_the_plain_model(folders, name, item_tiles):

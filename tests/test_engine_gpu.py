@@ -189,18 +189,29 @@ def test_steps_through_the_wide_product_match_the_plain_model(folders, name, exe
     runner.cache.check()
 
 
+REAL_SIZES = {
+    # two layers of the SmolLM2-1.7B sizes
+    "1.7b": dict(num_hidden_layers=2, hidden_size=2048, num_attention_heads=32, num_key_value_heads=32, head_dim=64,
+                 intermediate_size=8192, vocab_size=49152, rope_theta=130000.0, rms_norm_eps=1e-5,
+                 tie_word_embeddings=True, max_position_embeddings=512),
+    # one layer with Llama-3-8B's attention (grouped heads of 128) and width, a narrower feed-forward and vocabulary
+    "8b": dict(num_hidden_layers=1, hidden_size=4096, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
+               intermediate_size=6144, vocab_size=16000, rope_theta=500000.0, rms_norm_eps=1e-5,
+               tie_word_embeddings=False, max_position_embeddings=512),
+}
+
+
 @pytest.mark.parametrize("execution", ["eager", "graph"])
-def test_layers_of_real_sizes_match_the_plain_model(tmp_path_factory, execution):
-    """Two layers of the SmolLM2-1.7B sizes (width 2048, 32 heads of 64, feed-forward 8192, vocabulary 49152):
-    the sizes at which products choose other kernels by themselves (the wide weight-streaming product for
-    decode steps, the vendor's library for portions of more than 64 rows).  Whole prompts, portions, decode
-    steps of several requests and mixed steps against the plain model."""
+@pytest.mark.parametrize("sizes", ["1.7b", "8b"])
+def test_layers_of_real_sizes_match_the_plain_model(tmp_path_factory, sizes, execution):
+    """Layers of real sizes: the sizes at which products choose other kernels by themselves (the wide
+    weight-streaming product for decode steps, with the fused projection finishing in it; the vendor's library
+    for portions of more than 64 rows).  Whole prompts, portions, decode steps of several requests and mixed
+    steps against the plain model."""
     from runtime.engine import load_model, ModelRunner, StepEntry
     from runtime.kernels import ops
     from conftest import write_folder, plain_logits, assert_close
-    cfg = dict(num_hidden_layers=2, hidden_size=2048, num_attention_heads=32, num_key_value_heads=32, head_dim=64,
-               intermediate_size=8192, vocab_size=49152, rope_theta=130000.0, rms_norm_eps=1e-5,
-               tie_word_embeddings=True, max_position_embeddings=512)
+    cfg = REAL_SIZES[sizes]
     folder = write_folder(tmp_path_factory.mktemp("real") / "m", cfg, 77, sharp=False)
     model = load_model(folder, dtype="bfloat16")
     w_gate_up = model.layers[0].ffn.w_gate_up

@@ -217,31 +217,37 @@ def test_layers_of_real_sizes_match_the_plain_model(tmp_path_factory, sizes, exe
     w_gate_up = model.layers[0].ffn.w_gate_up
     assert ops.wide_ok(5, w_gate_up, True, after_norm=True) and ops.library_ok(90, w_gate_up)   # what this test is for
     runner = ModelRunner(model, n_pages=40, page_size=16, max_requests=8, execution=execution)
-    seqs = {k: random_tokens(900 + i, 100, cfg["vocab_size"]) for i, k in enumerate("abcde")}
-    refs = {k: plain_logits(folder, seqs[k]) for k in seqs}
-    for k in seqs:
-        runner.create(k)
-    fed = {k: 0 for k in seqs}
+    for round_ in range(3):    # the same step shapes again with other requests: in graph mode eager, captured, replayed
+        seqs = {k: random_tokens(900 + 10 * round_ + i, 100, cfg["vocab_size"]) for i, k in enumerate("abcde")}
+        refs = {k: plain_logits(folder, seqs[k]) for k in seqs}
+        for k in seqs:
+            runner.create(k)
+        fed = {k: 0 for k in seqs}
 
-    def feed(*parts):
-        entries, places = [], []
-        for k, n in parts:
-            entries.append(StepEntry(k, seqs[k][fed[k]:fed[k] + n], [0, n - 1] if n > 1 else [0]))
-            places += [(k, fed[k]), (k, fed[k] + n - 1)] if n > 1 else [(k, fed[k])]
-            fed[k] += n
-        logits = runner.step(entries).float().cpu().numpy()
-        for row, (k, pos) in zip(logits, places):
-            assert_close(row[None], refs[k][pos][None], "bfloat16", f"request {k} position {pos}")
+        def feed(*parts):
+            entries, places = [], []
+            for k, n in parts:
+                entries.append(StepEntry(k, seqs[k][fed[k]:fed[k] + n], [0, n - 1] if n > 1 else [0]))
+                places += [(k, fed[k]), (k, fed[k] + n - 1)] if n > 1 else [(k, fed[k])]
+                fed[k] += n
+            logits = runner.step(entries).float().cpu().numpy()
+            for row, (k, pos) in zip(logits, places):
+                assert_close(row[None], refs[k][pos][None], "bfloat16", f"round {round_} request {k} position {pos}")
 
-    feed(("a", 90))                                   # more than 64 rows: the library's products
-    feed(("b", 70), ("c", 3))
-    feed(("c", 40), ("d", 20))                        # 60 rows: four row tiles of the wide product
-    feed(("e", 7))
-    for _ in range(3):
-        feed(("a", 1), ("b", 1), ("c", 1), ("d", 1), ("e", 1))   # decode steps of five rows
-    feed(("a", 1), ("b", 1), ("c", 30), ("d", 1), ("e", 50))     # mixed: 83 rows
-    for _ in range(2):
-        feed(("a", 1), ("b", 1), ("c", 1), ("d", 1), ("e", 1))
+        feed(("a", 90))                                   # more than 64 rows: the library's products
+        feed(("b", 70), ("c", 3))
+        feed(("c", 40), ("d", 20))                        # 60 rows: four row tiles of the wide product
+        feed(("e", 7))
+        for _ in range(3):
+            feed(("a", 1), ("b", 1), ("c", 1), ("d", 1), ("e", 1))   # decode steps of five rows
+        feed(("a", 1), ("b", 1), ("c", 30), ("d", 1), ("e", 50))     # mixed: 83 rows
+        for _ in range(2):
+            feed(("a", 1), ("b", 1), ("c", 1), ("d", 1), ("e", 1))
+        for k in seqs:
+            runner.release(k)
+    if execution == "graph":
+        replayed = [key for key, p in runner.programs.items() if p["graph"] is not None and p["runs"] >= 3]
+        assert any(key[0] > 64 for key in replayed) and any(key[3] for key in replayed)
     runner.cache.check()
 
 

@@ -150,3 +150,173 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path):
         runner.cache.check()
     finally:
         cleanup()
+
+
+def build_routed_toy():
+    """A feed-forward with routing (two experts, the best one scaled by its softmax weight) and a position
+    encoding of its own (rotary angles that grow linearly with the pair index), both defined here."""
+    from runtime import register_part, make_part, register_architecture, TensorSpec
+    from runtime.config import unregister_architecture
+    from runtime.parts import FeedForward, Part, TokenEmbedding, LMHead, unregister_part
+    from runtime.models import Model
+
+    class LinearRotary(Part):
+        """Pair (i, i + D/2) of a head turns by pos * step * (i + 1)."""
+
+        def __init__(self, head_dim, step, max_positions):
+            self.head_dim, self.step, self.max_positions, self._tables = head_dim, step, max_positions, None
+
+        def prepare(self, device, dtype):
+            a = np.arange(self.max_positions, dtype=np.float64)[:, None] * self.step * np.arange(1, self.head_dim // 2 + 1)[None, :]
+            self._tables = (torch.from_numpy(np.cos(a).astype(np.float32)).to(device), torch.from_numpy(np.sin(a).astype(np.float32)).to(device))
+
+        def tables(self):
+            return self._tables
+
+    class RoutedMLP(FeedForward):
+        """out = p_e * expert_e(h) for the expert e with the largest router logit; p = softmax of the logits (float)."""
+
+        def __init__(self, name, hidden, intermediate, experts):
+            self.name, self.hidden, self.intermediate, self.experts = name, hidden, intermediate, experts
+
+        def tensor_specs(self):
+            specs = [TensorSpec(f"{self.name}.router.weight", (self.experts, self.hidden))]
+            for e in range(self.experts):
+                specs += [TensorSpec(f"{self.name}.experts.{e}.gate_proj.weight", (self.intermediate, self.hidden)),
+                          TensorSpec(f"{self.name}.experts.{e}.up_proj.weight", (self.intermediate, self.hidden)),
+                          TensorSpec(f"{self.name}.experts.{e}.down_proj.weight", (self.hidden, self.intermediate))]
+            return specs
+
+        def bind(self, tensors, dtype):
+            self.w = {k[len(self.name) + 1:]: v.float() for k, v in tensors.items() if k.startswith(self.name + ".")}
+
+        def forward(self, h, residual, ctx, norm=None):
+            x = h.float()
+            p = torch.softmax(x @ self.w["router.weight"].T, dim=-1)
+            best = p.argmax(-1)
+            for e in range(self.experts):
+                act = torch.nn.functional.silu(x @ self.w[f"experts.{e}.gate_proj.weight"].T) * (x @ self.w[f"experts.{e}.up_proj.weight"].T)
+                out = (act @ self.w[f"experts.{e}.down_proj.weight"].T) * p[:, e:e + 1]
+                residual += torch.where((best == e)[:, None], out, torch.zeros_like(out))
+            return residual
+
+    @dataclass(frozen=True)
+    class RoutedConfig:
+        vocab_size: int
+        hidden_size: int
+        experts: int
+        angle_step: float
+        max_position_embeddings: int
+        rms_norm_eps: float
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(*(raw[k] for k in ("vocab_size", "hidden_size", "experts", "angle_step", "max_position_embeddings", "rms_norm_eps")))
+
+    def build(c):
+        def norm(n): return make_part("norm", "rmsnorm", name=n, dim=c.hidden_size, eps=c.rms_norm_eps)
+        turning = make_part("position", "toy-linear-rotary", head_dim=16, step=c.angle_step, max_positions=c.max_position_embeddings)
+        still = make_part("position", "none", head_dim=16, max_positions=c.max_position_embeddings)
+        def attention(n, position):
+            return make_part("mixer", "attention", name=n, hidden=c.hidden_size, heads=3, kv_heads=1, head_dim=16, position=position)
+        layers = [
+            make_part("block", "prenorm", mixer_norm=norm("l0.n1"), mixer=attention("l0.attn", turning), ffn_norm=norm("l0.n2"),
+                      ffn=make_part("ffn", "toy-routed", name="l0.moe", hidden=c.hidden_size, intermediate=20, experts=c.experts)),
+            make_part("block", "prenorm", mixer_norm=norm("l1.n1"), mixer=attention("l1.attn", still), ffn_norm=norm("l1.n2"),
+                      ffn=make_part("ffn", "gated_mlp", name="l1.mlp", hidden=c.hidden_size, intermediate=24)),
+        ]
+        return Model(c, TokenEmbedding("embed", c.vocab_size, c.hidden_size), layers, norm("final"),
+                     LMHead("head", c.vocab_size, c.hidden_size))
+
+    register_part("position", "toy-linear-rotary", LinearRotary)
+    register_part("ffn", "toy-routed", RoutedMLP)
+    register_architecture("toy-routed-lm", RoutedConfig, build)
+
+    def cleanup():
+        unregister_part("position", "toy-linear-rotary")
+        unregister_part("ffn", "toy-routed")
+        unregister_architecture("toy-routed-lm")
+    return cleanup
+
+
+def plain_routed_toy(raw, w, tokens, chosen=None):
+    import plain_llama as P
+    eps, step, E = raw["rms_norm_eps"], raw["angle_step"], raw["experts"]
+    T = len(tokens)
+    x = w["embed.weight"][tokens]
+
+    def turn(v):   # [T, heads, 16]: pair (i, i + 8) by pos * step * (i + 1)
+        a = np.arange(T)[:, None, None] * step * np.arange(1, 9)[None, None, :]
+        lo, hi = v[..., :8], v[..., 8:]
+        return np.concatenate([lo * np.cos(a) - hi * np.sin(a), hi * np.cos(a) + lo * np.sin(a)], axis=-1)
+
+    def attention(x, p, rotate):
+        h = P.rmsnorm(x, w[p + ".n1.weight"], eps)
+        q = P.linear(h, w[p + ".attn.q_proj.weight"]).reshape(T, 3, 16)
+        k = P.linear(h, w[p + ".attn.k_proj.weight"]).reshape(T, 1, 16)
+        v = P.linear(h, w[p + ".attn.v_proj.weight"]).reshape(T, 1, 16)
+        if rotate:
+            q, k = turn(q), turn(k)
+        return x + P.linear(P.causal_attention(q, k, v).reshape(T, 48), w[p + ".attn.o_proj.weight"])
+
+    x = attention(x, "l0", True)
+    h = P.rmsnorm(x, w["l0.n2.weight"], eps)
+    logits = P.linear(h, w["l0.moe.router.weight"])
+    prob = np.exp(logits - logits.max(-1, keepdims=True)); prob /= prob.sum(-1, keepdims=True)
+    best = logits.argmax(-1)
+    if chosen is not None:
+        chosen.extend(best.tolist())
+    out = np.zeros_like(x)
+    for e in range(E):
+        pre = f"l0.moe.experts.{e}."
+        y = P.linear(P.swiglu(P.linear(h, w[pre + "gate_proj.weight"]), P.linear(h, w[pre + "up_proj.weight"])), w[pre + "down_proj.weight"])
+        out += np.where((best == e)[:, None], y * prob[:, e:e + 1], 0.0)
+    x = x + out
+    x = attention(x, "l1", False)
+    h = P.rmsnorm(x, w["l1.n2.weight"], eps)
+    x = x + P.linear(P.swiglu(P.linear(h, w["l1.mlp.gate_proj.weight"]), P.linear(h, w["l1.mlp.up_proj.weight"])), w["l1.mlp.down_proj.weight"])
+    return P.linear(P.rmsnorm(x, w["final.weight"], eps), w["head.weight"])
+
+
+def test_toy_routed_feed_forward_and_position_encoding_are_registered_built_and_stepped(tmp_path):
+    """A feed-forward with routing and a position encoding of another law, defined in this file, in one model beside the
+    framework's attention, norm and dense feed-forward (one layer without any position encoding): registered,
+    given random weights, loaded and stepped in portions, without a change to the framework's files."""
+    import plain_llama as P
+    from runtime.engine import load_model, ModelRunner, StepEntry
+    from runtime.engine.loading import build_from_config_dict
+    from runtime.weights import write_model_folder
+    cleanup = build_routed_toy()
+    try:
+        raw = {"model_type": "toy-routed-lm", "vocab_size": 53, "hidden_size": 24, "experts": 2, "angle_step": 0.37,
+               "max_position_embeddings": 64, "rms_norm_eps": 1e-5}
+        tmp_path.mkdir(exist_ok=True)
+        _, _, blueprint = build_from_config_dict(raw)
+        write_model_folder(tmp_path, raw, blueprint.tensor_specs(), seed=5, dtype=torch.float32)
+        cfg, w = P.read_folder(tmp_path)
+        w["l0.moe.router.weight"] = w["l0.moe.router.weight"] * 40      # decided routing: both experts are used
+        from safetensors.torch import save_file
+        save_file({k: torch.from_numpy(np.asarray(v, np.float32)) for k, v in w.items()}, str(tmp_path / "model.safetensors"))
+        model = load_model(tmp_path, dtype="float32")
+        assert set(model.cache_needs()) == {0, 1} and not model.state_needs()
+        runner = ModelRunner(model, n_pages=12, page_size=8, max_requests=2)
+        tokens = {"x": np.random.default_rng(2).integers(0, 53, 29).tolist(), "y": np.random.default_rng(3).integers(0, 53, 16).tolist()}
+        chosen = []
+        want = {k: plain_routed_toy(raw, w, v, chosen) for k, v in tokens.items()}
+        assert min(chosen.count(0), chosen.count(1)) >= 5                # both experts do work
+        runner.create("x"); runner.create("y")
+        got, fed = {"x": [], "y": []}, {"x": 0, "y": 0}
+        for step in [[("x", 11), ("y", 2)], [("x", 1), ("y", 5)], [("x", 1), ("y", 1)], [("x", 16), ("y", 8)]]:
+            entries = [StepEntry(k, tokens[k][fed[k]:fed[k] + n], list(range(n))) for k, n in step]
+            out = runner.step(entries).cpu().numpy()
+            row = 0
+            for k, n in step:
+                got[k].append(out[row:row + n]); row += n; fed[k] += n
+        for k in tokens:
+            np.testing.assert_allclose(np.concatenate(got[k]), want[k], rtol=3e-4, atol=3e-5)
+        # the position encoding matters: the same tokens without the turn give other logits
+        raw_still = dict(raw, angle_step=0.0)
+        assert np.abs(plain_routed_toy(raw_still, w, tokens["x"]) - want["x"]).max() > 1e-3
+        runner.cache.check()
+    finally:
+        cleanup()

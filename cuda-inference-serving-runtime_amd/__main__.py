@@ -28,7 +28,7 @@ def main(argv=None):
     parser.add_argument("--temperature", type=float, default=0.0, help="0 = greedy")
     parser.add_argument("--requests", type=Path, help="JSON list: key,prompt (IDs),max_new_tokens,arrival_s")
     parser.add_argument("--policy", choices=["serial", "chunked", "decode_first"], default="decode_first")
-    parser.add_argument("--pages", type=int, default=128)
+    parser.add_argument("--pages", type=int, default=128, help="cache pages; 0: as many as fit into the free GPU memory")
     parser.add_argument("--page-size", type=int, default=16)
     parser.add_argument("--token-budget", type=int, default=32)
     parser.add_argument("--prefill-chunk", type=int, default=8)

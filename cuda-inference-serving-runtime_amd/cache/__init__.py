@@ -1,3 +1,3 @@
 from .pages import KVNeed, StateNeed, OutOfPages, PagePool, CacheGroup
 from .state import StateSlots
-from .manager import CacheManager, Appended
+from .manager import CacheManager, Appended, pages_that_fit

@@ -209,3 +209,19 @@ class CacheManager:
                         "shared_pages": sum(1 for r in g.pool.refs if r > 1), "requests": len(g.tables),
                         "elements_per_token": token_bytes})
         return out
+
+
+def pages_that_fit(site_needs, page_size, itemsize, free_bytes, fraction=0.8, most=None):
+    """How many pages a pool may have so that the caches of all sites take `fraction` of `free_bytes`:
+    a page index costs, in every site that keeps keys and values, 2 x kv_heads x page_size x head_dim
+    elements.  `most` caps the answer (more pages than the requests can ever address are of no use)."""
+    per_page = sum(2 * need.kv_heads * page_size * need.head_dim * itemsize for need in site_needs.values() if need is not None)
+    if per_page == 0:
+        return 1
+    pages = int(free_bytes * fraction) // per_page
+    if most is not None:
+        pages = min(pages, most)
+    if pages < 1:
+        raise MemoryError(f"no room for a single cache page ({per_page} bytes) in {free_bytes} free bytes")
+    return pages
+

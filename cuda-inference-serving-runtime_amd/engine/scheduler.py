@@ -260,11 +260,19 @@ class Engine:
     # -- conveniences ---------------------------------------------------------------
     @classmethod
     def from_folder(cls, folder, dtype="bfloat16", pages=128, page_size=16, execution="eager", device="cuda:0", **limits):
-        """An engine for the model in `folder` (config.json + safetensors)."""
+        """An engine for the model in `folder` (config.json + safetensors).  pages None (or 0): as many as fit
+        into four fifths of the GPU memory that is free once the weights are loaded, at most what the
+        requests can address."""
+        import torch
+        from ..cache import pages_that_fit
         from .loading import load_model
         from .runner import ModelRunner
         model = load_model(folder, dtype=dtype, device=device)
         max_requests = max(8, limits.get("max_active", 8))
+        if not pages:
+            free, _ = torch.cuda.mem_get_info(torch.device(device))
+            addressable = max_requests * -(-model.max_positions // page_size)
+            pages = pages_that_fit(model.cache_needs(), page_size, 2 if dtype == "bfloat16" else 4, free, most=addressable)
         runner = ModelRunner(model, n_pages=pages, page_size=page_size, max_requests=max_requests, device=device,
                              execution=execution)
         return cls(runner, **limits)

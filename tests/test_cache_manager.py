@@ -231,3 +231,16 @@ def test_single_token_steps_take_the_same_pages_on_the_short_path(seed):
         return log, copies, [dict(g.tables) for g in m.groups], [list(g.pool.free) for g in m.groups]
 
     assert run(True) == run(False)
+
+
+def test_pages_that_fit_the_free_memory():
+    from runtime.cache import KVNeed, pages_that_fit
+    needs = {0: KVNeed(3, 64), 1: None, 2: KVNeed(3, 64), 3: KVNeed(2, 32, window=100)}
+    per_page = 2 * 16 * 2 * (3 * 64 + 3 * 64 + 2 * 32)          # keys and values, 16 tokens, bf16
+    assert pages_that_fit(needs, 16, 2, 10 * per_page, fraction=1.0) == 10
+    assert pages_that_fit(needs, 16, 2, 10 * per_page) == 8                  # four fifths by default
+    assert pages_that_fit(needs, 16, 4, 10 * per_page, fraction=1.0) == 5    # float32 pages are twice as large
+    assert pages_that_fit(needs, 16, 2, 10 ** 12, most=777) == 777
+    assert pages_that_fit({0: None}, 16, 2, 5) == 1                          # no site keeps keys: nothing to size
+    with pytest.raises(MemoryError):
+        pages_that_fit(needs, 16, 2, per_page - 1, fraction=1.0)

@@ -136,16 +136,31 @@ __global__ void attn_merge_kernel(const float* __restrict__ part_o, const float*
         }
         return;
     }
-    float m = -INFINITY;
-    for (int s = 0; s < splits; ++s) m = fmaxf(m, part_ml[(base + s) * 2]);
+    // more splits: sixteen at a time, all their loads issued before the first is used, merged into running sums
+    // (maximum, denominator, numerator) in the order of the splits
     for (int d = threadIdx.x; d < dim; d += blockDim.x) {
-        float den = 0.f, num = 0.f;
-        for (int s = 0; s < splits; ++s) {
-            const float l = part_ml[(base + s) * 2 + 1];
-            const float dm = part_ml[(base + s) * 2] - m;
-            const float w = l > 0.f ? (LOG2 ? exp2f(dm) : expf(dm)) * l : 0.f;
-            den += w;
-            num += w * part_o[(base + s) * dim + d];
+        float m = -INFINITY, den = 0.f, num = 0.f;
+        for (int s0 = 0; s0 < splits; s0 += 16) {
+            float ms[16], ls[16], os[16];
+#pragma unroll
+            for (int s = 0; s < 16; ++s) {
+                const size_t at = base + min(s0 + s, splits - 1);
+                ms[s] = part_ml[at * 2]; ls[s] = part_ml[at * 2 + 1]; os[s] = part_o[at * dim + d];
+            }
+            float m_new = m;
+#pragma unroll
+            for (int s = 0; s < 16; ++s) if (s0 + s < splits) m_new = fmaxf(m_new, ms[s]);
+            if (m_new == -INFINITY) continue;             // nothing visible so far
+            const float keep = LOG2 ? exp2f(m - m_new) : expf(m - m_new);   // m = -inf gives 0
+            den *= keep; num *= keep; m = m_new;
+#pragma unroll
+            for (int s = 0; s < 16; ++s) {
+                if (s0 + s >= splits) continue;
+                const float dm = ms[s] - m;
+                const float w = ls[s] > 0.f ? (LOG2 ? exp2f(dm) : expf(dm)) * ls[s] : 0.f;
+                den += w;
+                num += w * os[s];
+            }
         }
         store_f32(out + ((size_t)row * heads + head) * dim + d, den > 0.f ? num / den : 0.f);
     }

@@ -218,7 +218,7 @@ def test_attention_rowwise(ops, dtype, heads, kv_heads, dim, page_size):
     # split counts 1/3/16 where 16 exceeds the shorter request's tokens
     qt, kt, vt, tables, rows = paged_case(heads, kv_heads, dim, page_size, [17, 7, 1, 130], dtype, seed=dim)
     want = reference_attention(qt, kt, vt, tables, rows, page_size)
-    for splits in (1, 3, 16):
+    for splits in (1, 3, 16, 33):
         got = run_rowwise(ops, qt, kt, vt, tables, rows, page_size, splits)
         np.testing.assert_allclose(got, want, **tol(dtype), err_msg=f"splits={splits}")
 
@@ -300,7 +300,7 @@ def test_attention_mfma_rows(ops, heads, kv_heads, dim, page_size):
     """Decode form: single rows at scattered positions, every split count, including more splits than 32-key steps."""
     qt, kt, vt, tables, rows = paged_case(heads, kv_heads, dim, page_size, [17, 7, 1, 130, 333], torch.bfloat16, seed=dim + heads)
     want = reference_attention(qt, kt, vt, tables, rows, page_size)
-    for splits in (1, 2, 3, 16):
+    for splits in (1, 2, 3, 16, 40):
         for waves in (4, 8):
             got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, "rows", splits, waves=waves)
             np.testing.assert_allclose(got, want, **MFMA_TOL, err_msg=f"splits={splits} waves={waves}")

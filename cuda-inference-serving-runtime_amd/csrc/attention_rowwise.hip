@@ -104,13 +104,14 @@ attn_rowwise_kernel(const T* __restrict__ q, int q_row_stride, const T* __restri
 
 // Merge split partials: m = max m_i; w_i = l_i > 0 ? exp(m_i - m) * l_i : 0;
 // out = sum w_i o_i / sum w_i (reference: kernels/ops.cu:72-86).  A row with no
-// keys at all (padding) gives zeros.  LOG2: the maxima are in units of log2.
-template <typename T, bool LOG2>
+// keys at all (padding) gives zeros.  LOG2: the maxima are in units of log2.  MANY: more than sixteen splits
+// (a kernel of its own, so that the common few-split form keeps its registers and code to itself).
+template <typename T, bool LOG2, bool MANY>
 __global__ void attn_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                   T* __restrict__ out, int heads, int dim, int splits) {
     const int row = blockIdx.x, head = blockIdx.y;
     const size_t base = ((size_t)row * heads + head) * splits;
-    if (splits <= 16) {
+    if (!MANY) {
         // every load is issued before the first is used (one trip to memory instead of two); splits
         // past the count read the last one again and are left out of the sums
         for (int d = threadIdx.x; d < dim; d += blockDim.x) {
@@ -171,7 +172,8 @@ extern "C" int cisr_attn_merge(const float* part_o, const float* part_ml, void* 
                                int splits, hipStream_t stream) {
     if (rows <= 0) return 0;
     if (heads > 65535 || splits < 1) return (int)hipErrorInvalidValue;
-    attn_merge_kernel<bf16_t, true><<<dim3(rows, heads), 64, 0, stream>>>(part_o, part_ml, (bf16_t*)out, heads, dim, splits);
+    if (splits <= 16) attn_merge_kernel<bf16_t, true, false><<<dim3(rows, heads), 64, 0, stream>>>(part_o, part_ml, (bf16_t*)out, heads, dim, splits);
+    else attn_merge_kernel<bf16_t, true, true><<<dim3(rows, heads), 64, 0, stream>>>(part_o, part_ml, (bf16_t*)out, heads, dim, splits);
     return CISR_LAUNCH_CHECK();
 }
 
@@ -194,9 +196,12 @@ extern "C" int cisr_attn_rowwise(const void* q, int q_row_stride, const void* kc
             dim, page_size, width, window, scale, splits);
     int err = CISR_LAUNCH_CHECK();
     if (err || splits == 1) return err;
-    if (dtype == DT_F32)
-        attn_merge_kernel<float, false><<<dim3(rows, heads), 64, 0, stream>>>(part_o, part_ml, (float*)out, heads, dim, splits);
-    else
-        attn_merge_kernel<bf16_t, false><<<dim3(rows, heads), 64, 0, stream>>>(part_o, part_ml, (bf16_t*)out, heads, dim, splits);
+    if (dtype == DT_F32) {
+        if (splits <= 16) attn_merge_kernel<float, false, false><<<dim3(rows, heads), 64, 0, stream>>>(part_o, part_ml, (float*)out, heads, dim, splits);
+        else attn_merge_kernel<float, false, true><<<dim3(rows, heads), 64, 0, stream>>>(part_o, part_ml, (float*)out, heads, dim, splits);
+    } else {
+        if (splits <= 16) attn_merge_kernel<bf16_t, false, false><<<dim3(rows, heads), 64, 0, stream>>>(part_o, part_ml, (bf16_t*)out, heads, dim, splits);
+        else attn_merge_kernel<bf16_t, false, true><<<dim3(rows, heads), 64, 0, stream>>>(part_o, part_ml, (bf16_t*)out, heads, dim, splits);
+    }
     return CISR_LAUNCH_CHECK();
 }

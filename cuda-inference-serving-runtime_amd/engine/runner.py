@@ -462,11 +462,18 @@ class ModelRunner:
         # blocks of four waves a compute unit keep more loads in flight than the one block of eight that fits
         # (4-6 % faster at 8 rows and 8k to 30k, 2 % slower at 2k to 4k; a single row keeps its eight)
         waves = 8 if few and head_dim <= 64 and (steps <= 128 or blocks < 8) else 4
-        # few rows: enough blocks along the keys for two a compute unit (measured: a thousand blocks are no
-        # faster at a context of 2k to 8k and 12 % slower at 30k, where each then lives for three steps a
-        # wave only); many rows split until every compute unit has the blocks of four waves that its registers
-        # hold (three with small heads, two otherwise: 3-5 % faster at 64 rows of the 135M sizes than one block
-        # a unit).  A wave keeps at least two 32-key steps (one computing, one loading).
-        target = 512 if few else (768 if head_dim <= 64 else 512)
-        splits = int(max(1, min(steps // (waves * 2), -(-target // blocks), 64)))
+        if few:
+            # Few rows: split the keys until the blocks fill the GPU once: an eight-wave block fills a compute
+            # unit (256 blocks; more start a second round: 16 splits of 8 rows at 2k to 4k are 10 % slower than
+            # 8), four-wave blocks fit three a unit, of which two are worth having (512 blocks: a thousand are
+            # 12 % slower at 30k, where each then lives for three steps a wave only).  A wave keeps at least one
+            # 32-key step (with two, 8 rows at 2k have 4 splits and are 5 % slower).
+            room = 256 if waves == 8 else 512
+            splits = int(max(1, min(steps // waves, room // blocks, 64)))
+        else:
+            # Many rows split until every compute unit has the blocks of four waves that its registers hold (three
+            # with small heads, two otherwise: 3-5 % faster at 64 rows of the 135M sizes than one block a unit); a
+            # wave keeps at least two 32-key steps.
+            target = 768 if head_dim <= 64 else 512
+            splits = int(max(1, min(steps // (waves * 2), -(-target // blocks), 64)))
         return waves, splits

@@ -4,7 +4,8 @@ Every function validates device, dtype, contiguity and shapes on the host
 before the launch, because a kernel that reads out of bounds can take the GPU
 down.  Tensors are torch tensors on the GPU; launches go to torch's current
 stream, so they are ordered with torch's own work and can be captured into a
-graph.  Nothing here computes on the CPU.
+graph.  Nothing here computes on the CPU.  One kind of call leaves the kernels of this repository: large bf16
+products of more than 64 rows, which go to the vendor's library through torch.mm (see library_ok).
 """
 import ctypes as C
 import os

@@ -148,8 +148,28 @@ __global__ void add_kernel(float* __restrict__ x, const TD* __restrict__ delta, 
     if (i < n) x[i] += load_f32(delta + i);
 }
 
+// the same for a bf16 delta, eight elements a thread with 16-byte accesses (n % 8 == 0, aligned pointers)
+__global__ void __launch_bounds__(256) add_bf16x8_kernel(float* __restrict__ x, const bf16_t* __restrict__ delta, size_t n8) {
+    typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+    typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n8) return;
+    const u32x4_t d = *(const u32x4_t*)(delta + i * 8);
+    f32x4_t a = *(const f32x4_t*)(x + i * 8), b = *(const f32x4_t*)(x + i * 8 + 4);
+    a.x += __uint_as_float(d.x << 16); a.y += __uint_as_float(d.x & 0xffff0000u);
+    a.z += __uint_as_float(d.y << 16); a.w += __uint_as_float(d.y & 0xffff0000u);
+    b.x += __uint_as_float(d.z << 16); b.y += __uint_as_float(d.z & 0xffff0000u);
+    b.z += __uint_as_float(d.w << 16); b.w += __uint_as_float(d.w & 0xffff0000u);
+    *(f32x4_t*)(x + i * 8) = a; *(f32x4_t*)(x + i * 8 + 4) = b;
+}
+
 extern "C" int cisr_residual_add(float* x, const void* delta, long long n, int dtype, hipStream_t stream) {
     if (n <= 0) return 0;
+    if (dtype == DT_BF16 && n % 8 == 0 && ((uintptr_t)x) % 16 == 0 && ((uintptr_t)delta) % 16 == 0) {
+        const size_t n8 = (size_t)n / 8;
+        add_bf16x8_kernel<<<(unsigned)((n8 + 255) / 256), 256, 0, stream>>>(x, (const bf16_t*)delta, n8);
+        return CISR_LAUNCH_CHECK();
+    }
     unsigned blocks = (unsigned)((n + 255) / 256);
     if (dtype == DT_F32) add_kernel<float><<<blocks, 256, 0, stream>>>(x, (const float*)delta, (size_t)n);
     else add_kernel<bf16_t><<<blocks, 256, 0, stream>>>(x, (const bf16_t*)delta, (size_t)n);
@@ -169,9 +189,33 @@ __global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ act, int
     store_f32(act + i, g / (1.0f + expf(-g)) * u);
 }
 
+// the same for bf16, eight elements a thread with 16-byte accesses (inter % 8 == 0, aligned pointers)
+__global__ void __launch_bounds__(256) swiglu_bf16x8_kernel(const bf16_t* __restrict__ gu, bf16_t* __restrict__ act, int inter8, size_t n8) {
+    typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n8) return;
+    const size_t row = i / inter8; const int col = (int)(i % inter8) * 8;
+    const bf16_t* base = gu + row * (size_t)(16 * inter8);
+    const u32x4_t g = *(const u32x4_t*)(base + col), u = *(const u32x4_t*)(base + 8 * inter8 + col);
+    const uint32_t gw[4] = {g.x, g.y, g.z, g.w}, uw[4] = {u.x, u.y, u.z, u.w};
+    uint32_t out[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const float g0 = __uint_as_float(gw[k] << 16), g1 = __uint_as_float(gw[k] & 0xffff0000u);
+        const float u0 = __uint_as_float(uw[k] << 16), u1 = __uint_as_float(uw[k] & 0xffff0000u);
+        out[k] = pack_bf16x2(g0 / (1.0f + expf(-g0)) * u0, g1 / (1.0f + expf(-g1)) * u1);
+    }
+    *(u32x4_t*)(act + i * 8) = (u32x4_t){out[0], out[1], out[2], out[3]};
+}
+
 extern "C" int cisr_swiglu(const void* gu, void* act, int rows, int inter, int dtype, hipStream_t stream) {
     size_t n = (size_t)rows * inter;
     if (n == 0) return 0;
+    if (dtype == DT_BF16 && inter % 8 == 0 && ((uintptr_t)gu) % 16 == 0 && ((uintptr_t)act) % 16 == 0) {
+        const size_t n8 = n / 8;
+        swiglu_bf16x8_kernel<<<(unsigned)((n8 + 255) / 256), 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)act, inter / 8, n8);
+        return CISR_LAUNCH_CHECK();
+    }
     unsigned blocks = (unsigned)((n + 255) / 256);
     if (dtype == DT_F32) swiglu_kernel<float><<<blocks, 256, 0, stream>>>((const float*)gu, (float*)act, inter, n);
     else swiglu_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)act, inter, n);

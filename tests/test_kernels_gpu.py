@@ -84,6 +84,11 @@ def test_add_rmsnorm_and_residual_add(ops, dtype):
     x2 = x.clone()
     ops.residual_add(x2, d)
     np.testing.assert_allclose(f64(x2), want_sum, rtol=1e-6, atol=1e-6)
+    # widths of whole 16-byte runs take the form with eight elements a thread (bf16 delta)
+    x, d = rnd(7, 136, seed=4), rnd(7, 136, dtype=dtype, seed=5)
+    x3 = x.clone()
+    ops.residual_add(x3, d)
+    np.testing.assert_allclose(f64(x3), f64(x) + f64(d), rtol=1e-6, atol=1e-6)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -93,6 +98,12 @@ def test_swiglu(ops, dtype):
     out = ops.swiglu(gu, torch.empty(6, 173, dtype=dtype, device=DEV))
     np.testing.assert_allclose(f64(out), P.swiglu(f64(gu)[:, :173], f64(gu)[:, 173:]), **tol(dtype))
     assert torch.isfinite(out.float()).all() and out[0, 0] == 0
+    # a width of whole 16-byte runs takes the form with eight elements a thread (bf16)
+    gu = rnd(5, 2 * 176, dtype=dtype, scale=4.0, seed=9)
+    gu[1, 7], gu[1, 8], gu[1, 175] = 0.0, 60.0, -60.0
+    out = ops.swiglu(gu, torch.empty(5, 176, dtype=dtype, device=DEV))
+    np.testing.assert_allclose(f64(out), P.swiglu(f64(gu)[:, :176], f64(gu)[:, 176:]), **tol(dtype))
+    assert torch.isfinite(out.float()).all()
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])

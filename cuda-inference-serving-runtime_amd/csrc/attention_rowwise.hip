@@ -106,11 +106,14 @@ attn_rowwise_kernel(const T* __restrict__ q, int q_row_stride, const T* __restri
 // out = sum w_i o_i / sum w_i (reference: kernels/ops.cu:72-86).  A row with no
 // keys at all (padding) gives zeros.  LOG2: the maxima are in units of log2.  MANY: more than sixteen splits
 // (a kernel of its own, so that the common few-split form keeps its registers and code to itself).
+// `row_ids`: the partials of block row i belong to output row row_ids[i] (negative: to none).
 template <typename T, bool LOG2, bool MANY>
 __global__ void attn_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                  T* __restrict__ out, int heads, int dim, int splits) {
-    const int row = blockIdx.x, head = blockIdx.y;
-    const size_t base = ((size_t)row * heads + head) * splits;
+                                  T* __restrict__ out, int heads, int dim, int splits, const int* __restrict__ row_ids = nullptr) {
+    const int head = blockIdx.y;
+    const size_t base = ((size_t)blockIdx.x * heads + head) * splits;
+    const int row = row_ids ? row_ids[blockIdx.x] : (int)blockIdx.x;
+    if (row < 0) return;
     if (!MANY) {
         // every load is issued before the first is used (one trip to memory instead of two); splits
         // past the count read the last one again and are left out of the sums
@@ -169,11 +172,11 @@ __global__ void attn_merge_kernel(const float* __restrict__ part_o, const float*
 
 // merge of the matrix-core kernel's partials (bf16 output, maxima in log2 units)
 extern "C" int cisr_attn_merge(const float* part_o, const float* part_ml, void* out, int rows, int heads, int dim,
-                               int splits, hipStream_t stream) {
+                               int splits, const int* row_ids, hipStream_t stream) {
     if (rows <= 0) return 0;
     if (heads > 65535 || splits < 1) return (int)hipErrorInvalidValue;
-    if (splits <= 16) attn_merge_kernel<bf16_t, true, false><<<dim3(rows, heads), 64, 0, stream>>>(part_o, part_ml, (bf16_t*)out, heads, dim, splits);
-    else attn_merge_kernel<bf16_t, true, true><<<dim3(rows, heads), 64, 0, stream>>>(part_o, part_ml, (bf16_t*)out, heads, dim, splits);
+    if (splits <= 16) attn_merge_kernel<bf16_t, true, false><<<dim3(rows, heads), 64, 0, stream>>>(part_o, part_ml, (bf16_t*)out, heads, dim, splits, row_ids);
+    else attn_merge_kernel<bf16_t, true, true><<<dim3(rows, heads), 64, 0, stream>>>(part_o, part_ml, (bf16_t*)out, heads, dim, splits, row_ids);
     return CISR_LAUNCH_CHECK();
 }
 

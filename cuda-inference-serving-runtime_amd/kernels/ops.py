@@ -53,7 +53,7 @@ def _declare(h):
         "cisr_gemm_bf16_swiglu": [p, i, p, i, p, i, i, i, i, i, p],
         "cisr_gemm_skinny_bf16": [p, i, p, i, p, i, p, i, i, i, i, i, i, p, f, p, p],
         "cisr_qkv_rope_skinny": [p, i, p, i, p, i, i, i, p, f, p, p, p, p, p, p, i, i, i, i, i, p],
-        "cisr_attn_merge": [p, p, p, i, i, i, i, p],
+        "cisr_attn_merge": [p, p, p, i, i, i, i, p, p],
         "cisr_argmax": [p, p, p, i, p, p, i, i, p],
         "cisr_sample": [p, p, p, p, p, p, i, i, i, p],
         "cisr_take_tokens": [p, p, p, i, i, p],
@@ -540,14 +540,15 @@ def qkv_rope(a, w, q_out, positions, slots, cos, sin, kcache, vcache, heads, kv_
 
 def attention_mfma(q, q_row_stride, kcache, vcache, tables, seg_of_row, positions, out, heads, kv_heads, dim,
                    page_size, window, scale, tasks=None, splits=1, workspace=None, waves=4, block_tiles=False,
-                   item_tiles=1):
+                   item_tiles=1, row_ids=None):
     """Matrix-core attention (bf16).  tasks int32 [n, 4] = (segment, first row, rows, 0) runs tiles of
     prompt rows: one tile of 16/GC rows a block whose waves share the keys (with item_tiles=2, head sizes up to
     64: 32/GC rows, two item tiles a wave), or with `block_tiles` (head sizes up to 128) one tile of
     64 item_tiles / GC rows a block whose four waves own different rows and share keys and values through LDS
     (GC = query heads per key head, at most 16); tasks None runs one block
     per row (decode) of `waves` wavefronts (4 or 8) with `splits` blocks along the keys; splits > 1 needs
-    workspace = (partials float, statistics float) and a merge."""
+    workspace = (partials float, statistics float) and a merge.  `row_ids` (int32 [n], with tasks None): only
+    the rows it lists are computed and written (negative entries are skipped): the decode rows of a mixed step."""
     rows = out.shape[0]
     if not mfma_attention_supported(out.dtype, dim, page_size):
         raise KernelError(f"attention_mfma: head size {dim} / page size {page_size} / dtype {out.dtype} not supported")
@@ -575,12 +576,15 @@ def attention_mfma(q, q_row_stride, kcache, vcache, tables, seg_of_row, position
         tp = _dev(tasks, "tasks", torch.int32, (n_tasks, 4))
     else:
         n_tasks, mode = rows, 1
+        if row_ids is not None:
+            n_tasks = row_ids.numel()
+            tp = _dev(row_ids, "row_ids", torch.int32, (n_tasks,))
         if splits > 1:
             if workspace is None:
                 raise KernelError("attention: split runs need a workspace")
             part_o, part_ml = workspace
             po, pm = _dev(part_o, "part_o", torch.float32), _dev(part_ml, "part_ml", torch.float32)
-            if part_o.numel() < rows * heads * splits * dim or part_ml.numel() < rows * heads * splits * 2:
+            if part_o.numel() < n_tasks * heads * splits * dim or part_ml.numel() < n_tasks * heads * splits * 2:
                 raise KernelError("attention: split workspace too small")
     _check(fn(q.data_ptr(), q_row_stride, _dev(kcache, "kcache", None, (pages, kv_heads, page_size, dim)),
               _dev(vcache, "vcache", None, (pages, kv_heads, dim, page_size)), _dev(tables, "tables", torch.int32),
@@ -589,7 +593,7 @@ def attention_mfma(q, q_row_stride, kcache, vcache, tables, seg_of_row, position
               heads, kv_heads, dim, page_size.bit_length() - 1, int(window or 0), float(scale), int(splits), mode, int(waves),
               _stream()), "attention_mfma")
     if mode == 1 and splits > 1:
-        _check(lib().cisr_attn_merge(po, pm, out.data_ptr(), rows, heads, dim, int(splits), _stream()), "attention_merge")
+        _check(lib().cisr_attn_merge(po, pm, out.data_ptr(), n_tasks, heads, dim, int(splits), tp, _stream()), "attention_merge")
     return out
 
 

@@ -276,7 +276,8 @@ def test_attention_equal_large_scores_give_the_mean(ops):
     np.testing.assert_allclose(f64(out).reshape(heads, dim)[3], f64(vc)[0, 1, :, :n].mean(-1), rtol=1e-6)
 
 
-def run_mfma(ops, qt, kt, vt, tables, rows, page_size, mode, splits=1, window=None, scale=None, rows_per_tile=None, waves=4):
+def run_mfma(ops, qt, kt, vt, tables, rows, page_size, mode, splits=1, window=None, scale=None, rows_per_tile=None, waves=4,
+             row_ids=None):
     """mode "tiles": rows are grouped into tiles of consecutive rows of one segment;
     mode "rows": one block per row with `splits` blocks along the keys."""
     T, heads, dim = qt.shape
@@ -298,7 +299,8 @@ def run_mfma(ops, qt, kt, vt, tables, rows, page_size, mode, splits=1, window=No
         tasks = torch.tensor(items, dtype=torch.int32, device=DEV)
     ops.attention_mfma(qt.reshape(T, heads * dim), heads * dim, kt, vt, tables, seg, pos, out, heads, kv_heads, dim,
                        page_size, window, scale if scale is not None else 1 / math.sqrt(dim), tasks, splits, ws, waves,
-                       block_tiles=mode.startswith("block"), item_tiles=(2 if mode in ("tiles2", "block2") else 1))
+                       block_tiles=mode.startswith("block"), item_tiles=(2 if mode in ("tiles2", "block2") else 1),
+                       row_ids=None if row_ids is None else torch.tensor(row_ids, dtype=torch.int32, device=DEV))
     return f64(out).reshape(T, heads, dim)
 
 
@@ -321,6 +323,11 @@ def test_attention_mfma_rows(ops, heads, kv_heads, dim, page_size):
     np.testing.assert_allclose(got[1:], want[1:], **MFMA_TOL)
     again = [run_mfma(ops, qt, kt, vt, tables, rows, page_size, "rows", 16) for _ in range(3)]
     assert all((a == again[0]).all() for a in again)  # the merge order is fixed: repeated runs agree bit for bit
+    # a list of rows (the decode rows of a mixed step): only those are computed and written, a negative entry is none
+    for splits in (1, 5, 20):
+        got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, "rows", splits, waves=8, row_ids=[3, -1, 0, -1])
+        np.testing.assert_allclose(got[[3, 0]], want[[3, 0]], **MFMA_TOL, err_msg=f"listed rows, splits={splits}")
+        assert (got[[1, 2, 4]] == 9.0).all()
 
 
 def portion_case(heads, kv_heads, dim, page_size, plan, seed):

@@ -22,15 +22,16 @@ class GroupView:
     width: int
 
 
-def fill_tasks(tasks, counts, rows_per_tile, starts=None):
+def fill_tasks(tasks, counts, rows_per_tile, starts=None, skip_single=False):
     """Write (segment, first row, rows, 0) for tiles of at most `rows_per_tile` consecutive
     rows of one segment into the int32 array tasks[n, 4]; returns how many were written.
     With `starts` (the position of each segment's first row) the tiles are ordered by the
     number of keys they attend to, most first: blocks are handed out in this order, and the
-    long ones must not be the last to start."""
+    long ones must not be the last to start.  `skip_single`: segments of one row get no tile
+    (they are attended to by a launch of their own)."""
     n = row = 0
     for seg, count in enumerate(counts):
-        tiles = -(-count // rows_per_tile)
+        tiles = 0 if skip_single and count == 1 else -(-count // rows_per_tile)
         firsts = np.arange(tiles, dtype=np.int64) * rows_per_tile
         tasks[n:n + tiles, 0] = seg
         tasks[n:n + tiles, 1] = row + firsts
@@ -61,6 +62,8 @@ class StepContext:
         self.decode_only = False  # host: every segment brings exactly one token
         self.span_hint = 0        # host: context length that sizes attention launches (a bucket under capture)
         self.tasks = {}           # rows per tile -> int32 [n, 4] task list on the device
+        self.single_rows = None   # int32 [S]: the rows of the one-token segments of a mixed step, then -1
+        self.n_single = 0         # host: how many entries of single_rows a launch of their own covers (0: none)
         self.capturing = False    # the step is being recorded into a graph: launches only
         self.owner = None         # key of the captured program this step belongs to, if any
 
@@ -80,7 +83,7 @@ class StepContext:
                 raise RuntimeError(f"a task list of {rows_per_tile} rows a tile was first asked for under graph capture")
             counts = [count for _, _, count in self.segments]
             host = np.full((sum(-(-c // rows_per_tile) for c in counts), 4), -1, dtype=np.int32)
-            fill_tasks(host, counts, rows_per_tile, [start for _, start, _ in self.segments])
+            fill_tasks(host, counts, rows_per_tile, [start for _, start, _ in self.segments], skip_single=self.n_single > 0)
             tasks = torch.from_numpy(host).to(self.device, non_blocking=False)
             self.tasks[rows_per_tile] = tasks
             if rows_per_tile not in self.runner.task_tilings:

@@ -68,6 +68,9 @@ class ModelRunner:
         self.block_tiles = None    # long portions through LDS-shared tiles of 64 x this items: None = by the number of blocks
         self.tile_waves = int(os.environ.get("CISR_TILE_WAVES", "4"))   # wavefronts that share one tile's keys
         self.item_tiles = int(os.environ.get("CISR_ITEM_TILES", "2"))   # 16-item tiles a wave of long portions (small heads)
+        # In a mixed step a decoded token is a tile whose keys one block walks; from this context on the
+        # one-token segments get a launch of their own instead, which splits their keys over blocks
+        self.split_single_from = 4096
         self.device = torch.device(device)
         self.page_size = page_size
         self.max_requests = max_requests
@@ -186,14 +189,14 @@ class ModelRunner:
         entry[1].record()
         return PickedTokens(entry[0].numpy(), entry[1], requests, slots)
 
-    _FIXED = 9   # arrays of the metadata before the cache groups'
+    _FIXED = 10   # arrays of the metadata before the cache groups'
 
     def _layout(self, T, S, R):
         """Offsets of the packed int32 metadata: tokens, positions, seg_of_row, seg_start, seg_first_pos,
-        state_slots, logit_rows, token_source, logit_slots, then per group slots and tables, then one
+        state_slots, logit_rows, token_source, logit_slots, single_rows, then per group slots and tables, then one
         attention task list per known tiling (its length is the most tiles that T rows in S segments can make)."""
         W, G = self.table_width, len(self.cache.groups)
-        sizes = [T, T, T, S + 1, S, S, R, T, R] + [T, S * W] * G + [4 * (-(-T // r) + S) for r in self.task_tilings]
+        sizes = [T, T, T, S + 1, S, S, R, T, R, S] + [T, S * W] * G + [4 * (-(-T // r) + S) for r in self.task_tilings]
         return np.concatenate(([0], np.cumsum(sizes))).astype(np.int64)
 
     def _table_rows(self, g, done):
@@ -211,7 +214,15 @@ class ModelRunner:
                 stamps[d.state_slot] = stamp
         return mirror[[d.state_slot for d in done]]
 
-    def _context(self, entries, done, pad=None, device_buffer=None):
+    def _single_segments(self, done):
+        """How many one-token segments of a mixed step get an attention launch of their own: all of them, if
+        one of them has a long context; none in a step of one-token segments only, or of short contexts."""
+        singles = [d.start + 1 for d in done if d.count == 1]
+        if not singles or len(singles) == len(done) or max(singles) < self.split_single_from:
+            return 0
+        return len(singles)
+
+    def _context(self, entries, done, pad=None, device_buffer=None, n_single=None):
         """Build the step's metadata on the host, upload it in one copy and wrap it.
         `pad` = (T, S, R) pads the batch with inert rows (for captured programs):
         token 0 at position 0, no segment, no cache slot."""
@@ -228,8 +239,10 @@ class ModelRunner:
         total = offsets[-1]
         host = self._stage(total)
         arr = host.numpy()
-        tokens, positions, seg_of_row, seg_start, seg_first, state_slots, logit_rows, token_source, logit_slots = (
-            arr[offsets[i]:offsets[i + 1]] for i in range(9))
+        tokens, positions, seg_of_row, seg_start, seg_first, state_slots, logit_rows, token_source, logit_slots, single_rows = (
+            arr[offsets[i]:offsets[i + 1]] for i in range(10))
+        if n_single is None:      # (a captured program brings its padded number)
+            n_single = self._single_segments(done)
         decode_only = n_rows == n_seg
         slot_of = [d.state_slot for d in done]
         wanted_seg = [s for s, e in enumerate(entries) for _ in e.want]
@@ -279,6 +292,10 @@ class ModelRunner:
             if pad is not None:
                 slots[n_rows:] = -1
                 tables[n_seg:] = -1
+        single_rows[:] = -1
+        if n_single:
+            own = [int(first_row[s]) for s, c in enumerate(counts) if c == 1]
+            single_rows[:len(own)] = own
         tilings = list(self.task_tilings)
         for i, rows_per_tile in enumerate(tilings):
             tasks = arr[offsets[F + 2 * G + i]:offsets[F + 1 + 2 * G + i]].reshape(-1, 4)
@@ -288,7 +305,7 @@ class ModelRunner:
                 tasks[:n, 2] = 1
                 tasks[:n, 3] = 0
             else:
-                n = fill_tasks(tasks, counts, rows_per_tile, starts)
+                n = fill_tasks(tasks, counts, rows_per_tile, starts, skip_single=n_single > 0)
             tasks[n:] = (-1, 0, 0, 0)   # tiles of no segment do nothing
         dev = self._upload(host, total, device_buffer)
 
@@ -301,6 +318,7 @@ class ModelRunner:
         ctx.tokens, ctx.positions, ctx.seg_of_row = view(0), view(1), view(2)
         ctx.seg_start, ctx.seg_first_pos, ctx.state_slots, ctx.logit_rows = view(3), view(4), view(5), view(6)
         ctx.token_source = view(7)
+        ctx.single_rows, ctx.n_single = view(9), n_single
         ctx.kv = [GroupView(view(F + 2 * g), view(F + 1 + 2 * g, (S, W)), self.page_size, W) for g in range(G)]
         ctx.tasks = {r: view(F + 2 * G + i, (-1, 4)) for i, r in enumerate(tilings)}
         self._last_wanted = ([entries[s].request for s in wanted_seg], wanted_slots, view(8)[:n_want])
@@ -345,10 +363,10 @@ class ModelRunner:
         decode_only = all(d.count == 1 for d in done)
         context = 1 << (max(d.start + d.count for d in done) - 1).bit_length()
         return (_bucket(rows), _bucket(len(entries)), _bucket(wanted), decode_only, max(context, 256),
-                any(e.pending for e in entries))
+                any(e.pending for e in entries), _bucket(self._single_segments(done)))
 
     def _run_program(self, key, entries, done):
-        T, S, R, decode_only, context, take = key
+        T, S, R, decode_only, context, take, n_single = key
         program = self.programs.get(key)
         if program is None:
             program = {"meta": None, "graph": None, "runs": 0, "tilings": None}
@@ -365,7 +383,7 @@ class ModelRunner:
             torch.cuda.synchronize()
             program.update(meta=torch.zeros(int(self._layout(T, S, R)[-1]), dtype=torch.int32, device=self.device),
                            graph=None, runs=0, tilings=list(self.task_tilings))
-        ctx = self._context(entries, done, pad=(T, S, R), device_buffer=program["meta"])
+        ctx = self._context(entries, done, pad=(T, S, R), device_buffer=program["meta"], n_single=n_single)
         ctx.owner = key
         ctx.span_hint = context   # launch shapes inside a captured program depend on the key only
         ctx.decode_only = decode_only
@@ -419,6 +437,17 @@ class ModelRunner:
                 # a block own different rows and share each step's keys and values through LDS.  Otherwise (few
                 # heads, short portions) the waves of a block share one tile of 16 items (32 with small heads)
                 # and split its keys, which is what hides the latency of a step when blocks are scarce.
+                if ctx.n_single:
+                    # the decoded tokens of this mixed step: a launch of their own that splits their keys
+                    n = ctx.n_single
+                    waves, splits = self._rows_launch(n * kv_heads * -(-group // heads_per_chunk), span, heads_per_chunk, head_dim)
+                    workspace = None
+                    if splits > 1:
+                        workspace = (ctx.buffer("attn.part_o", (n * heads * splits * head_dim,), torch.float32),
+                                     ctx.buffer("attn.part_ml", (n * heads * splits * 2,), torch.float32))
+                    ops.attention_mfma(q, q_row_stride, kcache, vcache, view.tables, ctx.seg_of_row, ctx.positions, out,
+                                       heads, kv_heads, head_dim, view.page_size, window, scale, None, splits, workspace, waves,
+                                       row_ids=ctx.single_rows[:n])
                 long_portions = rows >= 16 * ctx.n_segments
                 block_tiles = 0
                 if long_portions and head_dim <= 128:

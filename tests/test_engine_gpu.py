@@ -145,6 +145,62 @@ def test_captured_prompt_and_mixed_steps_match_the_plain_model(folders, name, dt
     runner.cache.check()
 
 
+@pytest.mark.parametrize("name,dtype", [("a", "bfloat16"), ("b", "bfloat16"), ("c", "bfloat16")])
+@pytest.mark.parametrize("execution", ["eager", "graph"])
+@pytest.mark.parametrize("launch", [None, (4, 3)])
+def test_decoded_tokens_of_mixed_steps_in_a_launch_of_their_own(folders, name, dtype, execution, launch):
+    """From a certain context on, the one-token segments of a mixed step leave the tile list and are attended
+    to by the decode kernel over a list of rows, their keys split over blocks; forced here from the first
+    token, with the natural launch shape and with three splits (some of them empty at these lengths).  Under
+    graphs the list is padded to the program's size with rows of no request."""
+    from runtime.engine import load_model, ModelRunner, StepEntry
+    from runtime.kernels import ops
+    from conftest import plain_logits, assert_close
+    V = TINY[name]["vocab_size"]
+    model = load_model(folders[name], dtype=dtype)
+    runner = ModelRunner(model, n_pages=32, page_size=8, max_requests=4, execution=execution)
+    runner.split_single_from = 1
+    if launch:
+        runner._rows_launch = lambda *a: launch
+    seen = []
+    attend = ops.attention_mfma
+    def spy(*a, **kw):
+        seen.append(kw.get("row_ids"))
+        return attend(*a, **kw)
+    ops_attention, ops.attention_mfma = ops.attention_mfma, spy
+    try:
+        for round_ in range(3):
+            seqs = {k: random_tokens(700 + 10 * round_ + i, 50, V) for i, k in enumerate("wxyz")}
+            refs = {k: plain_logits(folders[name], seqs[k]) for k in seqs}
+            for k in seqs:
+                runner.create(k)
+            fed = {k: 0 for k in seqs}
+
+            def feed(*parts):
+                entries, places = [], []
+                for k, n in parts:
+                    entries.append(StepEntry(k, seqs[k][fed[k]:fed[k] + n], [0, n - 1] if n > 1 else [0]))
+                    places += [(k, fed[k]), (k, fed[k] + n - 1)] if n > 1 else [(k, fed[k])]
+                    fed[k] += n
+                logits = runner.step(entries).float().cpu().numpy()
+                for row, (k, pos) in zip(logits, places):
+                    assert_close(row[None], refs[k][pos][None], dtype, f"round {round_} request {k} position {pos}")
+
+            feed(("w", 21), ("x", 9))
+            feed(("w", 1), ("y", 13))                          # one decoded token beside a portion
+            feed(("y", 1), ("z", 17), ("w", 1), ("x", 1))      # three, the portion between them
+            feed(("w", 1), ("x", 7), ("y", 1))
+            feed(("x", 1), ("y", 1), ("z", 2), ("w", 1))       # a portion of two tokens
+            feed(("w", 1), ("x", 1), ("y", 1), ("z", 1))       # decode only: the ordinary launch
+            feed(("z", 1), ("x", 5))
+            for k in seqs:
+                runner.release(k)
+    finally:
+        ops.attention_mfma = ops_attention
+    assert sum(r is not None for r in seen) >= (30 if execution == "eager" else 1), "the decoded tokens of mixed steps had no launch of their own"
+    runner.cache.check()
+
+
 @pytest.mark.parametrize("name", ["a", "b"])
 @pytest.mark.parametrize("execution", ["eager", "graph"])
 def test_steps_through_the_wide_product_match_the_plain_model(folders, name, execution, monkeypatch):

@@ -335,10 +335,13 @@ extern "C" int cisr_gemm_bf16_swiglu(const void* A, int lda, const void* W, int 
     auto blocks = [&](int bm, int bn) { return (long long)((M + bm - 1) / bm) * ((2 * N + bn - 1) / bn); };
     if (blocks(128, 128) >= 512) return launch_bf16_swiglu<4, 4, 64>(a, lda, w, ldw, (bf16_t*)C, ldc, M, N, K, dual_off, stream);
     if (blocks(128, 64) >= 512) return launch_bf16_swiglu<4, 2, 64>(a, lda, w, ldw, (bf16_t*)C, ldc, M, N, K, dual_off, stream);
+    if (blocks(64, 64) < 256) return launch_bf16_swiglu<1, 2, 64>(a, lda, w, ldw, (bf16_t*)C, ldc, M, N, K, dual_off, stream);
     return launch_bf16_swiglu<2, 2, 64>(a, lda, w, ldw, (bf16_t*)C, ldc, M, N, K, dual_off, stream);
 }
 
-// Tile choice: the largest tile that still gives the 256 compute units a few blocks each.
+// Tile choice: the largest tile that still gives the 256 compute units a few blocks each; when even 64 x 64 leaves
+// most of them idle (a portion of a few hundred rows against small weights), 32 x 64 and 32 x 32 (measured on an
+// MI355X at 128 and 512 rows: 10-30 % faster there, slower from about one block a compute unit on).
 extern "C" int cisr_gemm_bf16(const void* A, int lda, const void* W, int ldw, void* C, int ldc, const float* R,
                               int ldr, int M, int N, int K, int out_dtype, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
@@ -348,5 +351,7 @@ extern "C" int cisr_gemm_bf16(const void* A, int lda, const void* W, int ldw, vo
     if (M <= 32) return launch_bf16<1, 2, 64>(a, lda, w, ldw, C, ldc, R, ldr, M, N, K, out_dtype, stream);
     if (blocks(128, 128) >= 512) return launch_bf16<4, 4, 64>(a, lda, w, ldw, C, ldc, R, ldr, M, N, K, out_dtype, stream);
     if (blocks(128, 64) >= 512) return launch_bf16<4, 2, 64>(a, lda, w, ldw, C, ldc, R, ldr, M, N, K, out_dtype, stream);
+    if (blocks(32, 64) <= 64) return launch_bf16<1, 1, 64>(a, lda, w, ldw, C, ldc, R, ldr, M, N, K, out_dtype, stream);
+    if (blocks(64, 64) < 256) return launch_bf16<1, 2, 64>(a, lda, w, ldw, C, ldc, R, ldr, M, N, K, out_dtype, stream);
     return launch_bf16<2, 2, 64>(a, lda, w, ldw, C, ldc, R, ldr, M, N, K, out_dtype, stream);
 }

@@ -413,7 +413,7 @@ def test_gemm_skinny_and_fused_swiglu(ops):
         want = P.swiglu(gq[:, :I], gq[:, I:])
         got = ops.gemm_swiglu(a, w, torch.empty(M, I, dtype=torch.bfloat16, device=DEV))
         np.testing.assert_allclose(f64(got), want, rtol=2e-2, atol=2e-2)
-        for rows in (70, 300):   # more rows: the tiled product with the activation as its epilogue
+        for rows in (70, 300, 1200):   # more rows: the tiled product with the activation as its epilogue
             big = rnd(rows, K, dtype=torch.bfloat16, seed=4, scale=0.5)
             gq = torch.from_numpy(f64(big) @ f64(w).T).to(torch.bfloat16).double().numpy()
             tiled = ops.gemm_swiglu(big, w, torch.empty(rows, I, dtype=torch.bfloat16, device=DEV))
@@ -563,7 +563,7 @@ def test_fused_projection_rotary_scatter_through_the_wide_product(ops, monkeypat
     assert torch.equal(q, q2)
 
 
-GEMM_SHAPES = [(1, 1, 1), (5, 7, 9), (64, 64, 32), (130, 200, 172), (33, 513, 144), (17, 130, 1000), (300, 129, 72), (8, 1536, 576)]
+GEMM_SHAPES = [(1, 1, 1), (5, 7, 9), (64, 64, 32), (130, 200, 172), (33, 513, 144), (17, 130, 1000), (300, 129, 72), (8, 1536, 576), (512, 576, 200), (1024, 1100, 64)]
 
 
 def test_gemm_wide_for_large_weights(ops, monkeypatch):

@@ -484,7 +484,8 @@ class ModelRunner:
         """Matrix-core decode kernel: (wavefronts a block, blocks along the keys).  Few rows:
         eight waves share a row's keys inside one block; when that still leaves the GPU idle
         and the context is long, the keys are also split over blocks (a merge kernel follows).
-        Many rows: four waves a block, one block a row and head group."""
+        Many rows: four waves a block, one block a row and head group, or with small heads eight waves
+        when that gives every compute unit at most one block."""
         steps = -(-span // 32)
         few = blocks < 128
         # eight waves a block with few rows and small heads, except at long contexts (more than 4k), where three
@@ -499,10 +500,16 @@ class ModelRunner:
             # 32-key step (with two, 8 rows at 2k have 4 splits and are 5 % slower).
             room = 256 if waves == 8 else 512
             splits = int(max(1, min(steps // waves, room // blocks, 64)))
+        elif head_dim <= 64 and 140 <= blocks <= 256:
+            # enough rows to give most compute units one block of eight waves, and no more than one each: the
+            # keys are not split and no merge follows (9-11 % faster than four waves and three or four splits at
+            # 144 to 256 blocks and 2k keys, 4-5 % at 8k)
+            waves, splits = 8, 1
         else:
             # Many rows split until every compute unit has the blocks of four waves that its registers hold (three
-            # with small heads, two otherwise: 3-5 % faster at 64 rows of the 135M sizes than one block a unit); a
-            # wave keeps at least two 32-key steps.
+            # with small heads, two otherwise: 3-5 % faster at 384 blocks of the 135M sizes than one block a unit;
+            # from 512 blocks on a split costs 3-8 %); a wave keeps at least two 32-key steps.
             target = 768 if head_dim <= 64 else 512
-            splits = int(max(1, min(steps // (waves * 2), -(-target // blocks), 64)))
+            per = target // blocks if head_dim <= 64 and blocks > 256 else -(-target // blocks)
+            splits = int(max(1, min(steps // (waves * 2), per, 64)))
         return waves, splits

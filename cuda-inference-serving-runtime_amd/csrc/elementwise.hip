@@ -289,16 +289,73 @@ __global__ void rope_scatter_kernel(T* __restrict__ qkv, const int* __restrict__
     }
 }
 
-// The same for bf16 rows whose whole heads turn (rot == dim) with dim a multiple of 16: one wavefront a
-// row, every lane turns 8 pairs at a time with 16-byte loads and stores.
+// The values of a prompt portion, 16 consecutive rows by 512 value columns a block, through LDS into the
+// transposed pages.  Rows that follow each other in a request lie side by side in a coordinate's run of a page:
+// when the 16 rows are one such run (inside one page, from a multiple of 8 on), a thread writes a coordinate's
+// 16 positions as 32 contiguous bytes and a wave 2 KB; otherwise lane j of every 16 writes row j's elements one
+// by one, which still puts neighbouring rows into one sector.  (One row at a time, every element is a 2-byte
+// store into a sector of its own: 20 of 29 us at 2,048 rows of 2,048 value columns.)
+__device__ __forceinline__ void rope_scatter_value_tile(const bf16_t* __restrict__ qkv, const int* __restrict__ slots,
+                                                        bf16_t* __restrict__ vcache, int rows, int heads, int kv_heads,
+                                                        int dim, int page_size, int tile) {
+    typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+    constexpr int TR = 16, CH = 512, PITCH = CH + 8;
+    __shared__ __attribute__((aligned(16))) bf16_t vs[TR * PITCH];
+    const int tid = threadIdx.x;
+    const int vcols = kv_heads * dim, col_chunks = (vcols + CH - 1) / CH;
+    const int row0 = (tile / col_chunks) * TR, c0 = (tile % col_chunks) * CH;
+    const int row_width = (heads + 2 * kv_heads) * dim;
+    const bf16_t* vbase = qkv + (size_t)(heads + kv_heads) * dim;
+    for (int i = tid; i < TR * (CH / 8); i += 256) {
+        const int rr = i / (CH / 8), cc = (i % (CH / 8)) * 8;
+        u32x4 v = {0u, 0u, 0u, 0u};
+        if (row0 + rr < rows && c0 + cc < vcols) v = *(const u32x4*)(vbase + (size_t)(row0 + rr) * row_width + c0 + cc);
+        *(u32x4*)(&vs[rr * PITCH + cc]) = v;
+    }
+    // one run?  (every thread looks at all 16 slots: the answer is the same for the whole block)
+    const int s0 = slots[row0];
+    bool run = s0 >= 0 && row0 + TR <= rows && (s0 % page_size) % 8 == 0 && s0 % page_size + TR <= page_size;
+    for (int j = 1; j < TR && run; ++j) run = slots[row0 + j] == s0 + j;
+    __syncthreads();
+    if (run) {
+        const int page = s0 / page_size, off = s0 % page_size;
+        for (int c = tid; c < CH && c0 + c < vcols; c += 256) {
+            const int col = c0 + c, h = col / dim, d = col % dim;
+            uint32_t w[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                w[j] = (uint32_t)vs[(2 * j) * PITCH + c] | ((uint32_t)vs[(2 * j + 1) * PITCH + c] << 16);
+            bf16_t* dst = vcache + (((size_t)page * kv_heads + h) * dim + d) * page_size + off;
+            *(u32x4*)dst = (u32x4){w[0], w[1], w[2], w[3]};
+            *(u32x4*)(dst + 8) = (u32x4){w[4], w[5], w[6], w[7]};
+        }
+        return;
+    }
+    const int j = tid % TR;
+    const int slot = row0 + j < rows ? slots[row0 + j] : -1;
+    if (slot < 0) return;
+    const int page = slot / page_size, off = slot % page_size;
+    for (int c = tid / TR; c < CH && c0 + c < vcols; c += 256 / TR) {
+        const int col = c0 + c, h = col / dim, d = col % dim;
+        vcache[(((size_t)page * kv_heads + h) * dim + d) * page_size + off] = vs[j * PITCH + c];
+    }
+}
+
+// The same for bf16 rows whose whole heads turn (rot == dim) with dim a multiple of 16: `lanes` (64, 128 or
+// 256) lanes of a block a row, every lane turns 8 pairs at a time with 16-byte loads and stores.
 __global__ void __launch_bounds__(256)
 rope_scatter_wave_kernel(bf16_t* __restrict__ qkv, const int* __restrict__ positions, const int* __restrict__ slots,
                          const float* __restrict__ cos_tab, const float* __restrict__ sin_tab,
                          bf16_t* __restrict__ kcache, bf16_t* __restrict__ vcache, int rows, int heads, int kv_heads,
-                         int dim, int page_size, int max_pos, int has_kv) {
+                         int dim, int page_size, int max_pos, int has_kv, int lanes, int qk_blocks) {
     typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
-    const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
-    const int row = blockIdx.x * 4 + wave;
+    if ((int)blockIdx.x >= qk_blocks) {                  // the blocks after the turning ones carry the values of a portion
+        rope_scatter_value_tile(qkv, slots, vcache, rows, heads, kv_heads, dim, page_size, blockIdx.x - qk_blocks);
+        return;
+    }
+    const bool values_here = qk_blocks == (int)gridDim.x;   // no value blocks: every row writes its own
+    const int lane = threadIdx.x % lanes;
+    const int row = blockIdx.x * (256 / lanes) + threadIdx.x / lanes;
     if (row >= rows) return;
     const int half = dim / 2, per_head = half / 8;   // 8-pair chunks of a head
     int pos = positions[row];
@@ -310,7 +367,7 @@ rope_scatter_wave_kernel(bf16_t* __restrict__ qkv, const int* __restrict__ posit
     const int slot = (has_kv && slots) ? slots[row] : -1;
     const int page = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot % page_size : 0;
     const int turning = heads + (slot >= 0 ? kv_heads : 0);   // q heads, then k heads if they have a place to go
-    for (int i = lane; i < turning * per_head; i += WAVE) {
+    for (int i = lane; i < turning * per_head; i += lanes) {
         const int h = i / per_head, d = (i % per_head) * 8;
         const bf16_t* p = base + h * dim + d;
         const u32x4 av = *(const u32x4*)p, bv = *(const u32x4*)(p + half);
@@ -331,10 +388,10 @@ rope_scatter_wave_kernel(bf16_t* __restrict__ qkv, const int* __restrict__ posit
         *(u32x4*)dst = (u32x4){lo[0], lo[1], lo[2], lo[3]};
         *(u32x4*)(dst + half) = (u32x4){hi[0], hi[1], hi[2], hi[3]};
     }
-    if (slot < 0) return;
+    if (slot < 0 || !values_here) return;
     // v heads: 8 coordinates a lane, written to the transposed page one by one
     const bf16_t* vb = base + (heads + kv_heads) * dim;
-    for (int i = lane; i < kv_heads * (dim / 8); i += WAVE) {
+    for (int i = lane; i < kv_heads * (dim / 8); i += lanes) {
         const int h = i / (dim / 8), d = (i % (dim / 8)) * 8;
         const u32x4 v = *(const u32x4*)(vb + h * dim + d);
         bf16_t* dst = vcache + (((size_t)page * kv_heads + h) * dim + d) * page_size + off;
@@ -356,8 +413,16 @@ extern "C" int cisr_rope_scatter(void* qkv, const int* positions, const int* slo
             (float*)kcache, (float*)vcache, heads, kv_heads, dim, rot, page_size, max_pos, has_kv);
     } else if (rot == dim && dim % 16 == 0 && (uintptr_t)qkv % 16 == 0 && (uintptr_t)cos_tab % 16 == 0 &&
                (uintptr_t)sin_tab % 16 == 0 && (!has_kv || (uintptr_t)kcache % 16 == 0)) {
-        rope_scatter_wave_kernel<<<(rows + 3) / 4, 256, 0, stream>>>((bf16_t*)qkv, positions, slots, cos_tab, sin_tab,
-            (bf16_t*)kcache, (bf16_t*)vcache, rows, heads, kv_heads, dim, page_size, max_pos, has_kv);
+        // lanes a row: as many as it has 8-pair chunks to turn, so that every lane's loads are in flight at once
+        const int chunks = (heads + (has_kv ? kv_heads : 0)) * (dim / 16);
+        const int lanes = chunks > 128 ? 256 : chunks > 64 ? 128 : 64, rows_a_block = 256 / lanes;
+        const int qk_blocks = (rows + rows_a_block - 1) / rows_a_block;
+        // a portion of 32 rows and more: further blocks carry the values, 16 rows by 512 columns each
+        const long long value_blocks = (rows >= 32 && has_kv && slots) ? (long long)((rows + 15) / 16) * ((kv_heads * dim + 511) / 512) : 0;
+        if (qk_blocks + value_blocks > 0x7fffffffLL) return (int)hipErrorInvalidValue;
+        rope_scatter_wave_kernel<<<(unsigned)(qk_blocks + value_blocks), 256, 0, stream>>>((bf16_t*)qkv, positions, slots,
+            cos_tab, sin_tab, (bf16_t*)kcache, (bf16_t*)vcache, rows, heads, kv_heads, dim, page_size, max_pos, has_kv, lanes,
+            qk_blocks);
     } else {
         rope_scatter_kernel<bf16_t><<<rows, 256, 0, stream>>>((bf16_t*)qkv, positions, slots, cos_tab, sin_tab,
             (bf16_t*)kcache, (bf16_t*)vcache, heads, kv_heads, dim, rot, page_size, max_pos, has_kv);

@@ -140,6 +140,55 @@ def test_rope_scatter(ops, dtype, heads, kv_heads, dim, theta):
             assert (kc64[s // P_, :, s % P_] == 7).all() and (vc64[s // P_, :, :, s % P_] == 7).all()
 
 
+@pytest.mark.parametrize("heads, kv_heads, dim, page_size, T, start", [
+    (9, 3, 64, 16, 100, None), (4, 4, 16, 4, 37, None), (3, 1, 128, 16, 33, None), (34, 34, 32, 8, 50, None),
+    (9, 3, 64, 16, 100, 0), (34, 34, 32, 16, 70, 16), (3, 1, 128, 32, 64, 8), (4, 2, 64, 16, 48, 5), (32, 32, 64, 16, 64, 0)])
+def test_rope_scatter_of_portions(ops, heads, kv_heads, dim, page_size, T, start):
+    """Portions of 32 rows and more (bf16, whole heads turn) write their values through LDS, 16 rows a block: runs of
+    consecutive slots, slots that jump between pages and requests, rows without a slot, more value columns than one
+    pass holds, a last block that is not full; nothing but the slots given is written.  With `start` the rows are one
+    request's positions from there on, page after page (tiles that are one run inside a page are written 32 bytes a
+    coordinate), with a few rows without a slot among them."""
+    from runtime.parts import RotaryEmbedding
+    theta = 1e4
+    rope = RotaryEmbedding(dim, theta, 700)
+    rope.prepare(DEV, torch.bfloat16)
+    cos, sin = rope.tables()
+    rng = np.random.default_rng(T)
+    pages = T + 5             # a run takes a page of its own
+    free = rng.permutation(pages).tolist()
+    slots, pos = [], []
+    if start is not None:
+        own = [free.pop() for _ in range(-(-(start + T) // page_size))]
+        slots = [own[(start + i) // page_size] * page_size + (start + i) % page_size for i in range(T)]
+        pos = [start + i for i in range(T)]
+    while len(slots) < T:      # runs of consecutive slots of random length, each from the start of a free page or inside it
+        run = int(rng.integers(1, 2 * page_size))
+        page, off, p0 = free.pop(), int(rng.integers(0, page_size)), int(rng.integers(0, 600))
+        for i in range(min(run, page_size - off, T - len(slots))):
+            slots.append(page * page_size + off + i); pos.append(p0 + i)
+    for i in rng.choice(T, 3, replace=False):
+        slots[i] = -1
+    qkv = rnd(T, (heads + 2 * kv_heads) * dim, dtype=torch.bfloat16, seed=5)
+    ref = f64(qkv)
+    kc = torch.full((pages, kv_heads, page_size, dim), 7.0, dtype=torch.bfloat16, device=DEV)
+    vc = torch.full((pages, kv_heads, dim, page_size), 7.0, dtype=torch.bfloat16, device=DEV)
+    ops.rope_scatter(qkv, torch.tensor(pos, dtype=torch.int32, device=DEV), torch.tensor(slots, dtype=torch.int32, device=DEV),
+                     cos, sin, kc, vc, heads, kv_heads, dim, page_size)
+    q_ref = P.rope(ref[:, :heads * dim].reshape(T, heads, dim), pos, theta)
+    k_ref = P.rope(ref[:, heads * dim:(heads + kv_heads) * dim].reshape(T, kv_heads, dim), pos, theta)
+    v_ref = ref[:, (heads + kv_heads) * dim:].reshape(T, kv_heads, dim)
+    np.testing.assert_allclose(f64(qkv)[:, :heads * dim].reshape(T, heads, dim), q_ref, **tol(torch.bfloat16))
+    kc64, vc64 = f64(kc), f64(vc)
+    want_k, want_v = np.full(kc64.shape, 7.0), np.full(vc64.shape, 7.0)
+    for t, s in enumerate(slots):
+        if s >= 0:
+            want_k[s // page_size, :, s % page_size] = k_ref[t]
+            want_v[s // page_size, :, :, s % page_size] = v_ref[t]
+    np.testing.assert_array_equal(vc64, want_v)
+    np.testing.assert_allclose(kc64, want_k, **tol(torch.bfloat16))
+
+
 def test_rope_partial_rotation_and_identity(ops):
     from runtime.parts import RotaryEmbedding, NoPosition
     dim, rot = 16, 8

@@ -110,6 +110,90 @@ extern "C" int cisr_rmsnorm(const float* x, const float* w, void* y, const int* 
     return launch_rmsnorm<bf16_t>(x, w, (bf16_t*)y, rows, n_out, dim, eps, stream);
 }
 
+// x += sum of `slices` partial sums (parts[s][row][dim], added in slice order, then to x), and with w also
+// y = rmsnorm(x): what follows a product that was cut along its inner size and left unfinished, so that the sum,
+// the residual and the norm are one kernel.  One block a row (these are steps of few rows: a row's loads have to
+// be spread over many lanes and in flight together), R chunks of four floats a thread, four slices at a time.
+template <typename T, int R>
+__global__ void __launch_bounds__(256)
+rmsnorm_partials_kernel(float* x, const float* __restrict__ parts, int slices, const float* __restrict__ w,
+                        T* __restrict__ y, int n_rows, int dim, float eps) {
+    __shared__ float red[4];
+    const int row = blockIdx.x, tid = threadIdx.x;
+    const int n4 = dim / 4;
+    float4* xr = (float4*)(x + (size_t)row * dim);
+    const size_t slice4 = (size_t)n_rows * n4;
+    const float4* pr = (const float4*)parts + (size_t)row * n4;
+    const float4* w4 = (const float4*)w;
+    float4 v[R], r[R], g[R];
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+        const int c = min(tid + 256 * i, n4 - 1);     // past the row: a copy of its last chunk, not counted or stored
+        r[i] = xr[c];
+        if (w) g[i] = w4[c];
+        v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    for (int s0 = 0; s0 < slices; s0 += 4) {
+        float4 p[R][4];
+#pragma unroll
+        for (int i = 0; i < R; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                p[i][j] = pr[(size_t)min(s0 + j, slices - 1) * slice4 + min(tid + 256 * i, n4 - 1)];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if (s0 + j >= slices) break;
+#pragma unroll
+            for (int i = 0; i < R; ++i) { v[i].x += p[i][j].x; v[i].y += p[i][j].y; v[i].z += p[i][j].z; v[i].w += p[i][j].w; }
+        }
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+        v[i] = make_float4(v[i].x + r[i].x, v[i].y + r[i].y, v[i].z + r[i].z, v[i].w + r[i].w);
+        if (tid + 256 * i >= n4) continue;
+        xr[tid + 256 * i] = v[i];
+        ss += v[i].x * v[i].x + v[i].y * v[i].y + v[i].z * v[i].z + v[i].w * v[i].w;
+    }
+    if (!w) return;
+    const float scale = 1.0f / sqrtf(block_sum<256>(ss, red) / (float)dim + eps);
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+        const int c = tid + 256 * i;
+        if (c >= n4) continue;
+        const float a = v[i].x * scale * g[i].x, b = v[i].y * scale * g[i].y;
+        const float cc = v[i].z * scale * g[i].z, d = v[i].w * scale * g[i].w;
+        if (sizeof(T) == 4) {
+            ((float4*)((float*)y + (size_t)row * dim))[c] = make_float4(a, b, cc, d);
+        } else {
+            ((uint2*)((bf16_t*)y + (size_t)row * dim))[c] = make_uint2(pack_bf16x2(a, b), pack_bf16x2(cc, d));
+        }
+    }
+}
+
+template <typename T>
+static int launch_rmsnorm_partials(float* x, const float* parts, int slices, const float* w, T* y, int n_rows, int dim,
+                                   float eps, hipStream_t stream) {
+    const int chunks = (dim / 4 + 255) / 256;
+    if (chunks <= 1) rmsnorm_partials_kernel<T, 1><<<n_rows, 256, 0, stream>>>(x, parts, slices, w, y, n_rows, dim, eps);
+    else if (chunks <= 2) rmsnorm_partials_kernel<T, 2><<<n_rows, 256, 0, stream>>>(x, parts, slices, w, y, n_rows, dim, eps);
+    else if (chunks <= 4) rmsnorm_partials_kernel<T, 4><<<n_rows, 256, 0, stream>>>(x, parts, slices, w, y, n_rows, dim, eps);
+    else rmsnorm_partials_kernel<T, 8><<<n_rows, 256, 0, stream>>>(x, parts, slices, w, y, n_rows, dim, eps);
+    return CISR_LAUNCH_CHECK();
+}
+
+// x[n_rows, dim] += the partial sums parts[slices][n_rows][dim]; y = rmsnorm(x) with weights w (w null: the sum only,
+// y unused).  dim % 4 == 0, dim <= 8192, 16-byte aligned operands.
+extern "C" int cisr_rmsnorm_partials(float* x, const float* parts, int slices, const float* w, void* y, int n_rows, int dim,
+                                     float eps, int out_dtype, hipStream_t stream) {
+    if (n_rows <= 0) return 0;
+    if (slices < 1 || dim <= 0 || dim % 4 || dim > 8192 || (uintptr_t)x % 16 || (uintptr_t)parts % 16 || (uintptr_t)w % 16 ||
+        (w && (!y || (uintptr_t)y % 16)))
+        return (int)hipErrorInvalidValue;
+    if (out_dtype == DT_F32) return launch_rmsnorm_partials<float>(x, parts, slices, w, (float*)y, n_rows, dim, eps, stream);
+    return launch_rmsnorm_partials<bf16_t>(x, parts, slices, w, (bf16_t*)y, n_rows, dim, eps, stream);
+}
+
 // x += delta, then y = rmsnorm(x) (reference: kernels/execution.cu:12-24; here
 // the sum stays float so nothing is rounded before the norm reads it).
 template <typename TD, typename T>

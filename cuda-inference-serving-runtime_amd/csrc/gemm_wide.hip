@@ -35,6 +35,7 @@ struct WideArgs {
     int units;                  // 16-row units of W
     int slices;                 // slices of K: SPW / 2 rounds of NW pairs of 32-wide k-steps each
     int dual_off;               // two blocks of W this many rows apart (SwiGLU), or 0
+    int leave_partials;         // several slices: no second kernel, the caller's next kernel adds the partial sums
     // the fused q/k/v projection (head_dim > 0): C is q, bf16 [M, heads * head_dim]
     const int* positions; const int* slots; const float* cos_tab; const float* sin_tab;
     bf16_t* kcache; bf16_t* vcache; int heads, kv_heads, head_dim, page_size, max_pos;
@@ -244,7 +245,7 @@ static int wide_launch(WideArgs a, size_t workspace_floats, bool plan_only, long
     const size_t partial = a.slices > 1 ? (size_t)a.slices * a.M * a.N * NB : 0;
     if (need) *need = (long long)partial;
     if (plan_only) return 0;
-    if (partial > workspace_floats || (partial && !a.P)) return (int)hipErrorInvalidValue;
+    if (partial > workspace_floats || (partial && !a.P) || (a.leave_partials && !partial)) return (int)hipErrorInvalidValue;
     const long long items = (long long)a.units * a.slices;
     const int cus = wide_cus();
     const size_t shmem = (size_t)NW * NB * MT * 4 * WAVE * sizeof(float);
@@ -256,7 +257,7 @@ static int wide_launch(WideArgs a, size_t workspace_floats, bool plan_only, long
     // one block a compute unit, each with an equal run of the work items
     gemm_wide_kernel<MT, NW, SPW, NB, ROPE><<<(unsigned)(items < cus ? items : cus), NW * 64, shmem, stream>>>(a);
     int err = CISR_LAUNCH_CHECK();
-    if (err || a.slices == 1) return err;
+    if (err || a.slices == 1 || a.leave_partials) return err;
     const size_t cells = (size_t)a.M * a.N;
     gemm_wide_finish_kernel<NB, ROPE><<<(unsigned)((cells + 255) / 256), 256, 0, stream>>>(a);
     return CISR_LAUNCH_CHECK();
@@ -320,14 +321,15 @@ static bool wide_aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 
 static int wide_entry(const void* A, int lda, const void* W, int ldw, void* C, int ldc, const float* R, int ldr, int M, int N,
                       int K, int out_dtype, int dual_off, float* workspace, long long workspace_floats, bool plan_only,
-                      long long* need, hipStream_t stream) {
+                      long long* need, hipStream_t stream, bool leave_partials = false) {
     if (need) *need = 0;
     if (M <= 0 || N <= 0) return 0;
     if (M > 64 || K < 8 || K % 8 || lda % 8 || ldw % 8 || dual_off < 0 || workspace_floats < 0 ||
         (out_dtype != DT_F32 && out_dtype != DT_BF16) || (R && out_dtype != DT_F32) || (dual_off > 0 && R))
         return (int)hipErrorInvalidValue;
-    if (!plan_only && (!wide_aligned16(A) || !wide_aligned16(W) || !C)) return (int)hipErrorInvalidValue;
+    if (!plan_only && (!wide_aligned16(A) || !wide_aligned16(W) || (!C && !leave_partials))) return (int)hipErrorInvalidValue;
     WideArgs a = {};
+    a.leave_partials = leave_partials;
     a.A = (const bf16_t*)A; a.lda = lda; a.W = (const bf16_t*)W; a.ldw = ldw; a.C = C; a.ldc = ldc; a.out_dtype = out_dtype;
     a.R = R; a.ldr = ldr; a.P = workspace; a.M = M; a.N = N; a.K = K; a.units = (N + 15) / 16; a.dual_off = dual_off;
     return dual_off > 0 ? wide_dispatch<2, false>(a, (size_t)workspace_floats, plan_only, need, stream)
@@ -372,4 +374,13 @@ extern "C" int cisr_gemm_wide_bf16(const void* A, int lda, const void* W, int ld
                                    long long workspace_floats, hipStream_t stream) {
     return wide_entry(A, lda, W, ldw, C, ldc, R, ldr, M, N, K, out_dtype, dual_off, workspace, workspace_floats, false,
                       nullptr, stream);
+}
+
+// The first pass alone, for a product that is cut into several slices (cisr_gemm_wide_workspace(M, N, K, 0) > 0; an
+// error otherwise): workspace[s][M][N] holds the slices' partial sums of A . W^T, which the caller's next kernel
+// adds in slice order (cisr_rmsnorm_partials, cisr_add_partials) instead of a second kernel here.
+extern "C" int cisr_gemm_wide_partials_bf16(const void* A, int lda, const void* W, int ldw, int M, int N, int K,
+                                            float* workspace, long long workspace_floats, hipStream_t stream) {
+    return wide_entry(A, lda, W, ldw, nullptr, 0, nullptr, 0, M, N, K, DT_F32, 0, workspace, workspace_floats, false,
+                      nullptr, stream, true);
 }

@@ -64,6 +64,10 @@ class StepContext:
         self.tasks = {}           # rows per tile -> int32 [n, 4] task list on the device
         self.single_rows = None   # int32 [S]: the rows of the one-token segments of a mixed step, then -1
         self.n_single = 0         # host: how many entries of single_rows a launch of their own covers (0: none)
+        # A product whose partial sums are still to be added to the residual stream: (rows tensor, partials), set by a
+        # part that was told it may (`next_norm`), taken by the norm that reads the rows next (or settled)
+        self.unfinished = None
+        self.next_norm = None     # the norm that reads the residual stream after the block that runs now, if known
         self.capturing = False    # the step is being recorded into a graph: launches only
         self.owner = None         # key of the captured program this step belongs to, if any
 
@@ -89,6 +93,37 @@ class StepContext:
             if rows_per_tile not in self.runner.task_tilings:
                 self.runner.task_tilings.append(rows_per_tile)
         return tasks
+
+    def add_product(self, a, w, residual):
+        """residual += a . w^T, in place.  Where the product is cut along its inner size and the norm that reads the
+        residual next can add the slices itself (`next_norm`), they are left to it: one kernel fewer."""
+        if getattr(self.next_norm, "adds_partials", False):
+            partials = ops.gemm_unfinished(a, w, residual)
+            if partials is not None:
+                self.leave_unfinished(residual, partials)
+                return residual
+        return ops.gemm(a, w, residual, residual=residual)
+
+    def leave_unfinished(self, rows, partials):
+        """`rows` lack the partial sums `partials` (ops.gemm_unfinished); whoever reads them next adds them."""
+        if self.unfinished is not None:
+            raise RuntimeError("a second unfinished product before the first was added")
+        self.unfinished = (rows, partials)
+
+    def take_unfinished(self, rows):
+        """The partial sums that `rows` lack, for a kernel that adds them itself; None if there are none."""
+        if self.unfinished is None:
+            return None
+        if self.unfinished[0].data_ptr() != rows.data_ptr():
+            raise RuntimeError("the unfinished product belongs to other rows")
+        partials, self.unfinished = self.unfinished[1], None
+        return partials
+
+    def settle(self, rows):
+        """Add what `rows` lack, if anything: before a reader that cannot do it itself."""
+        partials = self.take_unfinished(rows)
+        if partials is not None:
+            ops.add_partials(rows, partials)
 
     def attend(self, q, q_row_stride, kcache, vcache, view, out, heads, kv_heads, head_dim, window, scale):
         """out[r] = attention of row r's queries over its request's cache."""

@@ -58,6 +58,8 @@ def _declare(h):
         "cisr_sample": [p, p, p, p, p, p, i, i, i, p],
         "cisr_take_tokens": [p, p, p, i, i, p],
         "cisr_gemm_wide_bf16": [p, i, p, i, p, i, p, i, i, i, i, i, i, p, C.c_longlong, p],
+        "cisr_gemm_wide_partials_bf16": [p, i, p, i, i, i, i, p, C.c_longlong, p],
+        "cisr_rmsnorm_partials": [p, p, i, p, p, i, i, f, i, p],
         "cisr_qkv_rope_wide": [p, i, p, i, p, i, i, i, p, p, p, p, p, p, i, i, i, i, i, p, C.c_longlong, p],
     }
     for name, args in sig.items():
@@ -143,6 +145,35 @@ def rmsnorm(x, weight, out, eps, rows=None):
     _check(lib().cisr_rmsnorm(_dev(x, "x", torch.float32), _dev(weight, "weight", torch.float32, (dim,)),
                               _dev(out, "out", None, (n_out, dim)), rp, n_out, dim, float(eps),
                               _storage(out, "out"), _stream()), "rmsnorm")
+    return out
+
+
+def partials_ok(x):
+    """Whether add_partials / rmsnorm_partials take the float rows x."""
+    return (x.dtype == torch.float32 and x.is_contiguous() and x.shape[1] % 4 == 0 and x.shape[1] <= 8192
+            and x.data_ptr() % 16 == 0)
+
+
+def add_partials(x, partials):
+    """x += the partial sums that gemm_unfinished left, in slice order (float rows, in place)."""
+    parts, slices = partials
+    rows, dim = x.shape
+    if not partials_ok(x) or parts.numel() < slices * rows * dim:
+        raise KernelError("add_partials: contiguous float rows of a multiple of 4 (at most 8192) and their partial sums")
+    _check(lib().cisr_rmsnorm_partials(x.data_ptr(), _dev(parts, "partials", torch.float32), int(slices), None, None, rows, dim,
+                                       0.0, _DT[torch.float32], _stream()), "add_partials")
+    return x
+
+
+def rmsnorm_partials(x, partials, weight, out, eps):
+    """x += the partial sums that gemm_unfinished left (in place), out = rmsnorm(x) * weight: one kernel."""
+    parts, slices = partials
+    rows, dim = x.shape
+    if not partials_ok(x) or parts.numel() < slices * rows * dim or out.data_ptr() % 16:
+        raise KernelError("rmsnorm_partials: contiguous float rows of a multiple of 4 (at most 8192) and their partial sums")
+    _check(lib().cisr_rmsnorm_partials(x.data_ptr(), _dev(parts, "partials", torch.float32), int(slices),
+                                       _dev(weight, "weight", torch.float32, (dim,)), _dev(out, "out", None, (rows, dim)),
+                                       rows, dim, float(eps), _storage(out, "out"), _stream()), "rmsnorm_partials")
     return out
 
 
@@ -403,6 +434,26 @@ def _gemm_wide(a, w, out, residual, swiglu, what):
                                      None if work is None else work.data_ptr(), 0 if work is None else work.numel(),
                                      _stream()), what)
     return out
+
+
+def gemm_unfinished(a, w, residual):
+    """The product a . w^T that is to be added to the float rows `residual`, left unfinished where the wide kernel
+    cuts it into slices and would need a second kernel to add them: returns (partial sums [slices, M, N], slices)
+    for rmsnorm_partials or add_partials, which then are that second kernel; None (nothing done) for every other
+    product: call gemm."""
+    m, k = a.shape
+    n = w.shape[0]
+    if (a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or w.shape[1] != k or not 0 < m <= SKINNY_ROWS
+            or library_ok(m, w) or not _skinny_ok(a, w) or not wide_ok(m, w) or tuple(residual.shape) != (m, n)
+            or not partials_ok(residual)):
+        return None
+    need = _wide_plan(m, n, k, False)
+    if need <= 0:
+        return None
+    work = _wide_workspace(a.device, need)
+    _check(lib().cisr_gemm_wide_partials_bf16(a.data_ptr(), a.stride(0), w.data_ptr(), w.stride(0), m, n, k,
+                                              work.data_ptr(), work.numel(), _stream()), "gemm_unfinished")
+    return work, need // (m * n)
 
 
 def _skinny_ok(a, w):

@@ -94,8 +94,15 @@ class Model:
         """Logits [R, vocab] (float) at ctx.logit_rows; None if no row is wanted
         (the layers still run: they fill the cache)."""
         x = self.embedding.forward(ctx)
+        last = len(self.schedule) - 1
         for index, entry in enumerate(self.schedule):
+            # a block may leave its last product to the norm that reads the residual stream next, if that block names one
+            following = self.layers[self.schedule[index + 1].layer] if index < last else None
+            ctx.next_norm = following.first_norm() if hasattr(following, "first_norm") else None
             x = self.layers[entry.layer].forward(x, ctx, self.site_of(index))
+            ctx.next_norm = None
+            if following is None or not hasattr(following, "first_norm"):
+                ctx.settle(x)
         if ctx.logit_rows.shape[0] == 0:
             return None
         if self.head.fuses_norm(self.final_norm, x, ctx.logit_rows):

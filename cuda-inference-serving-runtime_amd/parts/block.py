@@ -22,14 +22,29 @@ class PreNormBlock(Part):
         for p in self.parts():
             p.prepare(device, dtype)
 
+    def first_norm(self):
+        """The norm that reads the residual stream first: the block before may leave its last product to it."""
+        return self.mixer_norm
+
     def forward(self, residual, ctx, site):
+        # ctx.next_norm names the norm that reads the residual stream after the part that runs: a part's last
+        # product may be left to it (ctx.add_product); on entry it is the norm after this block
+        after = ctx.next_norm
+        ffn_fuses = self.ffn.fuses_norm(self.ffn_norm, residual, ctx)
+        ctx.next_norm = None if ffn_fuses else self.ffn_norm
         if self.mixer.fuses_norm(self.mixer_norm, residual, ctx):
+            ctx.settle(residual)
             residual = self.mixer.forward(None, residual, ctx, site, norm=self.mixer_norm)
         else:
             residual = self.mixer.forward(self.mixer_norm.forward(residual, ctx), residual, ctx, site)
-        if self.ffn.fuses_norm(self.ffn_norm, residual, ctx):
+        if ffn_fuses:
+            ctx.settle(residual)
+            ctx.next_norm = after
             return self.ffn.forward(None, residual, ctx, norm=self.ffn_norm)
-        return self.ffn.forward(self.ffn_norm.forward(residual, ctx), residual, ctx)
+        h = self.ffn_norm.forward(residual, ctx)
+        ctx.settle(residual)       # (a norm that adds no partial sums)
+        ctx.next_norm = after
+        return self.ffn.forward(h, residual, ctx)
 
 
 register_part("block", "prenorm", PreNormBlock)

@@ -38,7 +38,7 @@ class GatedMLP(FeedForward):
             ops.gemm_swiglu(h, self.w_gate_up, act)   # one kernel: product and activation
         else:
             ops.gemm_swiglu(h, self.w_gate_up, act, scratch=ctx.buffer("ffn.gate_up", (T, 2 * self.intermediate), ctx.dtype))
-        return ops.gemm(act, self.w_down, residual, residual=residual)
+        return ctx.add_product(act, self.w_down, residual)
 
 
 register_part("ffn", "gated_mlp", GatedMLP)

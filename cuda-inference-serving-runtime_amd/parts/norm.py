@@ -7,6 +7,8 @@ from .base import Part, TensorSpec, register_part
 
 
 class RMSNorm(Part):
+    adds_partials = True    # forward adds the partial sums of a product left unfinished before it (ctx.add_product)
+
     def __init__(self, name, dim, eps):
         self.name, self.dim, self.eps = name, dim, float(eps)
         self.weight = None
@@ -20,6 +22,12 @@ class RMSNorm(Part):
     def forward(self, x, ctx, rows=None, tag="norm"):
         n_out = x.shape[0] if rows is None else rows.shape[0]
         out = ctx.buffer(tag, (n_out, self.dim), ctx.dtype)
+        partials = ctx.take_unfinished(x)
+        if partials is not None:
+            # the product before was left as partial sums: they, the residual and the norm are one kernel
+            if rows is None and ops.partials_ok(x):
+                return ops.rmsnorm_partials(x, partials, self.weight, out, self.eps)
+            ops.add_partials(x, partials)
         return ops.rmsnorm(x, self.weight, out, self.eps, rows)
 
 

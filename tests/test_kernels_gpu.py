@@ -681,6 +681,44 @@ def test_gemm_wide_at_the_sizes_that_choose_it(ops, M):
     torch.testing.assert_close(y, x.float() @ w_n.float().T, rtol=1e-4, atol=1e-4)
 
 
+@pytest.mark.parametrize("M", [4, 8, 40, 64])
+def test_product_left_unfinished_is_added_by_the_norm_that_follows(ops, M, monkeypatch):
+    """A product that the wide kernel cuts along its inner size may leave its slices' partial sums to the kernel that
+    reads the rows next: sum + residual + norm in one kernel, or the sum alone; the rows are bit for bit what the
+    product's own second kernel gives, the norm differs by the order of its sum of squares only.  Products that are
+    not cut (or not wide) are not taken."""
+    torch.manual_seed(M)
+    N, K = 2048, 8192                       # the down projection of the 1.7B sizes
+    w = (torch.randn(N, K, device=DEV) * 0.02).bfloat16()
+    a = (torch.randn(M, K, device=DEV) * 0.5).bfloat16()
+    r = torch.randn(M, N, device=DEV)
+    nw = 1 + 0.1 * torch.randn(N, device=DEV)
+    assert ops.wide_ok(M, w)
+    want_x = r.clone()
+    ops.gemm(a, w, want_x, residual=want_x)
+    for out_dtype in (torch.bfloat16, torch.float32):
+        want_y = ops.rmsnorm(want_x, nw, torch.empty(M, N, dtype=out_dtype, device=DEV), 1e-5)
+        x = r.clone()
+        partials = ops.gemm_unfinished(a, w, x)
+        assert partials is not None and partials[1] > 1
+        assert torch.equal(x, r)            # nothing added yet
+        y = ops.rmsnorm_partials(x, partials, nw, torch.empty(M, N, dtype=out_dtype, device=DEV), 1e-5)
+        assert torch.equal(x, want_x)
+        torch.testing.assert_close(y.float(), want_y.float(), rtol=1e-2 if out_dtype == torch.bfloat16 else 1e-5, atol=1e-5)
+    x = r.clone()
+    ops.add_partials(x, ops.gemm_unfinished(a, w, x))
+    assert torch.equal(x, want_x)
+    torch.testing.assert_close(x, r + a.float() @ w.float().T, rtol=1e-4, atol=1e-4)
+    # not taken: small weights (another kernel), a product of one slice, rows that are no contiguous floats
+    small = (torch.randn(64, 128, device=DEV) * 0.02).bfloat16()
+    assert ops.gemm_unfinished(a[:, :128].contiguous(), small, torch.zeros(M, 64, device=DEV)) is None
+    for limit in ("WIDE_MIN_BYTES", "WIDE_MIN_BYTES_FEW_ROWS", "WIDE_MIN_BYTES_MANY_ROWS"):
+        monkeypatch.setattr(ops, limit, 0)
+    assert ops.wide_ok(M, small) and ops.gemm_unfinished(a[:, :128].contiguous(), small, torch.zeros(M, 64, device=DEV)) is None
+    assert ops.gemm_unfinished(a, w, torch.zeros(M, N, dtype=torch.bfloat16, device=DEV)) is None
+    assert ops.gemm_unfinished(a, w, torch.zeros(M, 2 * N, device=DEV)[:, :N]) is None
+
+
 def test_library_products_of_many_rows_also_in_captured_graphs(ops, monkeypatch):
     """Large bf16 products of many rows may go to the vendor's library, with the residual sum and the activation
     as kernels after it.  Checked against float products, eagerly and in a captured graph that is replayed with

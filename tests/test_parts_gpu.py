@@ -109,6 +109,57 @@ def test_block_part(setup):
     runner.cache.check()
 
 
+def test_product_left_to_the_next_norm_only_if_that_norm_adds_it(folders, monkeypatch):
+    """ctx.add_product leaves a product that the wide kernel cuts into slices to the norm named in ctx.next_norm, if
+    that norm says it adds partial sums; RMSNorm.forward then gives the norm of the finished rows and finishes them;
+    any other reader (no norm named, a norm of another kind, ctx.settle) gets finished rows."""
+    from runtime.engine import load_model, ModelRunner, StepEntry
+    from runtime.kernels import ops
+    from runtime.parts import RMSNorm
+    for limit in ("WIDE_MIN_BYTES", "WIDE_MIN_BYTES_FEW_ROWS", "WIDE_MIN_BYTES_MANY_ROWS"):
+        monkeypatch.setattr(ops, limit, 0)
+    model = load_model(folders["a"], dtype="bfloat16")
+    runner = ModelRunner(model, n_pages=16, page_size=8)
+    runner.create("u")
+    ctx = runner._context([StepEntry("u", [1] * 6, [])], runner.cache.append_many([("u", 6)]))
+    torch.manual_seed(0)
+    M, N, K = 6, 64, 8192
+    a = (torch.randn(M, K, device=DEV) * 0.5).bfloat16()
+    w = (torch.randn(N, K, device=DEV) * 0.02).bfloat16()
+    r = torch.randn(M, N, device=DEV)
+    assert ops._wide_plan(M, N, K, False) > 0, "this shape was meant to be cut into slices"
+    want = ops.gemm(a, w, r.clone(), residual=None) + r
+
+    class OtherNorm:                  # knows nothing of partial sums
+        def forward(self, x, ctx):
+            return x * 2
+
+    norm = RMSNorm("n", N, 1e-5)
+    norm.weight = 1 + 0.1 * torch.randn(N, device=DEV)
+    for reader in (None, OtherNorm()):
+        ctx.next_norm = reader
+        x = ctx.add_product(a, w, r.clone())
+        assert ctx.unfinished is None
+        torch.testing.assert_close(x, want, rtol=1e-5, atol=1e-5)
+    ctx.next_norm = norm
+    x = ctx.add_product(a, w, r.clone())
+    assert ctx.unfinished is not None and torch.equal(x, r)
+    y = norm.forward(x, ctx)
+    assert ctx.unfinished is None
+    torch.testing.assert_close(x, want, rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(y.float(), ops.rmsnorm(want, norm.weight, torch.empty(M, N, device=DEV), 1e-5), rtol=2e-2, atol=2e-2)
+    x = ctx.add_product(a, w, r.clone())
+    with pytest.raises(RuntimeError):
+        ctx.add_product(a, w, r.clone())          # a second one before the first was added
+    with pytest.raises(RuntimeError):
+        ctx.settle(torch.zeros(M, N, device=DEV))  # other rows
+    ctx.settle(x)
+    torch.testing.assert_close(x, want, rtol=1e-5, atol=1e-5)
+    ctx.settle(x)                                  # nothing left: no change
+    torch.testing.assert_close(x, want, rtol=1e-5, atol=1e-5)
+    runner.release("u")
+
+
 def test_head_part_tied_and_untied(folders):
     from runtime.engine import load_model
     tied = load_model(folders["a"], dtype="bfloat16")

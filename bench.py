@@ -97,7 +97,7 @@ def main():
         keys = [f"b{batch}-{i}" for i in range(batch)]
         last, prefill_times = [], []
         for key in keys:
-            tokens = rng.integers(0, V, size=args.prompt).tolist()
+            tokens = rng.integers(0, V, size=args.prompt, dtype=np.int32)   # token ids as they come from a tokenizer: an array
             first, dt = timed_prefill(key, tokens)
             last.append(first)
             prefill_times.append(dt)

@@ -17,6 +17,8 @@ per layer) and an append may bring many tokens.
 from dataclasses import dataclass
 from typing import Optional
 
+import numpy as np
+
 
 class OutOfPages(MemoryError):
     pass
@@ -135,7 +137,11 @@ class CacheGroup:
         while len(table) * P < length + n_new:
             table.append(self.pool.allocate())
             self._touch(request)
-        slots = [table[(length + i) // P] * P + (length + i) % P for i in range(n_new)]
+        if n_new > 32:      # a prompt portion: the same, vectorised
+            at = np.arange(length, length + n_new, dtype=np.int64)
+            slots = (np.asarray(table, dtype=np.int64)[at // P] * P + at % P).tolist()
+        else:
+            slots = [table[(length + i) // P] * P + (length + i) % P for i in range(n_new)]
         return slots, copies
 
     def create(self, request):

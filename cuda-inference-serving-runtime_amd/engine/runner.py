@@ -148,8 +148,12 @@ class ModelRunner:
             elif n == 1:
                 if not 0 <= int(e.tokens[0]) < vocab:
                     raise ValueError(f"request {e.request!r} has a token outside the vocabulary")
-            elif min(e.tokens) < 0 or max(e.tokens) >= vocab:
-                raise ValueError(f"request {e.request!r} has a token outside the vocabulary")
+            else:
+                # a portion: checked as an array, which the metadata then takes as it is (a list is converted once)
+                ids = np.asarray(e.tokens)
+                if ids.ndim != 1 or ids.dtype.kind not in "iu" or ids.min() < 0 or ids.max() >= vocab:
+                    raise ValueError(f"request {e.request!r} has a token outside the vocabulary")
+                e.tokens = ids.astype(np.int32, copy=False)
             for w in e.want:
                 if not 0 <= int(w) < n:
                     raise ValueError(f"request {e.request!r} wants a place outside its tokens")

@@ -39,8 +39,8 @@ def main():
                          "requests with prompts of 128..--prompt tokens and --new-tokens each through the scheduler")
     ap.add_argument("--requests", type=int, default=64)
     ap.add_argument("--new-tokens", type=int, default=256)
-    ap.add_argument("--token-budget", type=int, default=1024)
-    ap.add_argument("--prefill-chunk", type=int, default=512)
+    ap.add_argument("--token-budget", type=int, default=2112, help="serving: rows a step (a whole prompt beside 64 decoded tokens)")
+    ap.add_argument("--prefill-chunk", type=int, default=2048)
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU only; --gpus {args.gpus} is not run")

@@ -215,6 +215,76 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ x, const TD* __restrict__
     for (int d = threadIdx.x; d < dim; d += 256) store_f32(dst + d, xr[d] * scale * w[d]);
 }
 
+// The same for a bf16 delta and rows of a multiple of four, 16-byte aligned (8 for the delta): one wavefront a
+// row, as rmsnorm_wave_kernel, which it equals bit for bit on the summed rows.
+template <typename T, int R>
+__global__ void __launch_bounds__(256)
+add_rmsnorm_wave_kernel(float* x, const bf16_t* __restrict__ delta, const float* __restrict__ w, T* __restrict__ y,
+                        int n_rows, int dim, float eps) {
+    const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+    const int row = blockIdx.x * 4 + wave;
+    if (row >= n_rows) return;
+    const int n4 = dim / 4;
+    float4* xr = (float4*)(x + (size_t)row * dim);
+    const uint2* dr = (const uint2*)(delta + (size_t)row * dim);
+    const float4* w4 = (const float4*)w;
+    float4 v[R], g[R];
+    uint2 d[R];
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+        const int c = min(lane + WAVE * i, n4 - 1);   // past the row: a copy of its last chunk, not counted or stored
+        v[i] = xr[c];
+        d[i] = dr[c];
+        g[i] = w4[c];
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+        v[i].x += __uint_as_float(d[i].x << 16); v[i].y += __uint_as_float(d[i].x & 0xffff0000u);
+        v[i].z += __uint_as_float(d[i].y << 16); v[i].w += __uint_as_float(d[i].y & 0xffff0000u);
+        if (lane + WAVE * i >= n4) continue;
+        xr[lane + WAVE * i] = v[i];
+        ss += v[i].x * v[i].x + v[i].y * v[i].y + v[i].z * v[i].z + v[i].w * v[i].w;
+    }
+    const float scale = 1.0f / sqrtf(wave_sum(ss) / (float)dim + eps);
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+        const int c = lane + WAVE * i;
+        if (c >= n4) continue;
+        const float a = v[i].x * scale * g[i].x, b = v[i].y * scale * g[i].y;
+        const float cc = v[i].z * scale * g[i].z, e = v[i].w * scale * g[i].w;
+        if (sizeof(T) == 4) {
+            ((float4*)((float*)y + (size_t)row * dim))[c] = make_float4(a, b, cc, e);
+        } else {
+            ((uint2*)((bf16_t*)y + (size_t)row * dim))[c] = make_uint2(pack_bf16x2(a, b), pack_bf16x2(cc, e));
+        }
+    }
+}
+
+template <typename T>
+static int launch_add_rmsnorm_wave(float* x, const bf16_t* delta, const float* w, T* y, int rows, int dim, float eps,
+                                   hipStream_t stream) {
+    const int blocks = (rows + 3) / 4, chunks = (dim / 4 + WAVE - 1) / WAVE;
+    if (chunks <= 1) add_rmsnorm_wave_kernel<T, 1><<<blocks, 256, 0, stream>>>(x, delta, w, y, rows, dim, eps);
+    else if (chunks <= 2) add_rmsnorm_wave_kernel<T, 2><<<blocks, 256, 0, stream>>>(x, delta, w, y, rows, dim, eps);
+    else if (chunks <= 4) add_rmsnorm_wave_kernel<T, 4><<<blocks, 256, 0, stream>>>(x, delta, w, y, rows, dim, eps);
+    else if (chunks <= 8) add_rmsnorm_wave_kernel<T, 8><<<blocks, 256, 0, stream>>>(x, delta, w, y, rows, dim, eps);
+    else if (chunks <= 16) add_rmsnorm_wave_kernel<T, 16><<<blocks, 256, 0, stream>>>(x, delta, w, y, rows, dim, eps);
+    else add_rmsnorm_wave_kernel<T, 32><<<blocks, 256, 0, stream>>>(x, delta, w, y, rows, dim, eps);
+    return CISR_LAUNCH_CHECK();
+}
+
+// x[rows, dim] (float) += delta (bf16); y = rmsnorm(x) with weights w, float or bf16 (out_dtype): dim % 4 == 0,
+// dim <= 8192, 16-byte aligned x, w, y, 8-byte aligned delta.
+extern "C" int cisr_add_rmsnorm_bf16(float* x, const void* delta, const float* w, void* y, int rows, int dim, float eps,
+                                     int out_dtype, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    if (dim <= 0 || dim % 4 || dim > 8192 || (uintptr_t)x % 16 || (uintptr_t)delta % 8 || (uintptr_t)w % 16 || (uintptr_t)y % 16)
+        return (int)hipErrorInvalidValue;
+    if (out_dtype == DT_F32) return launch_add_rmsnorm_wave<float>(x, (const bf16_t*)delta, w, (float*)y, rows, dim, eps, stream);
+    return launch_add_rmsnorm_wave<bf16_t>(x, (const bf16_t*)delta, w, (bf16_t*)y, rows, dim, eps, stream);
+}
+
 extern "C" int cisr_add_rmsnorm(float* x, const void* delta, const float* w, void* y, int rows, int dim,
                                 float eps, int dtype, hipStream_t stream) {
     if (rows <= 0) return 0;

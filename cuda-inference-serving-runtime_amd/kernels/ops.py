@@ -60,6 +60,7 @@ def _declare(h):
         "cisr_gemm_wide_bf16": [p, i, p, i, p, i, p, i, i, i, i, i, i, p, C.c_longlong, p],
         "cisr_gemm_wide_partials_bf16": [p, i, p, i, i, i, i, p, C.c_longlong, p],
         "cisr_rmsnorm_partials": [p, p, i, p, p, i, i, f, i, p],
+        "cisr_add_rmsnorm_bf16": [p, p, p, p, i, i, f, i, p],
         "cisr_qkv_rope_wide": [p, i, p, i, p, i, i, i, p, p, p, p, p, p, i, i, i, i, i, p, C.c_longlong, p],
     }
     for name, args in sig.items():
@@ -155,9 +156,12 @@ def partials_ok(x):
 
 
 def add_partials(x, partials):
-    """x += the partial sums that gemm_unfinished left, in slice order (float rows, in place)."""
+    """x += what gemm_unfinished left (float rows, in place): the partial sums in slice order, or (slices 0) the
+    bf16 product."""
     parts, slices = partials
     rows, dim = x.shape
+    if slices == 0:
+        return residual_add(x, parts)
     if not partials_ok(x) or parts.numel() < slices * rows * dim:
         raise KernelError("add_partials: contiguous float rows of a multiple of 4 (at most 8192) and their partial sums")
     _check(lib().cisr_rmsnorm_partials(x.data_ptr(), _dev(parts, "partials", torch.float32), int(slices), None, None, rows, dim,
@@ -166,13 +170,19 @@ def add_partials(x, partials):
 
 
 def rmsnorm_partials(x, partials, weight, out, eps):
-    """x += the partial sums that gemm_unfinished left (in place), out = rmsnorm(x) * weight: one kernel."""
+    """x += what gemm_unfinished left (in place), out = rmsnorm(x) * weight: one kernel."""
     parts, slices = partials
     rows, dim = x.shape
-    if not partials_ok(x) or parts.numel() < slices * rows * dim or out.data_ptr() % 16:
-        raise KernelError("rmsnorm_partials: contiguous float rows of a multiple of 4 (at most 8192) and their partial sums")
-    _check(lib().cisr_rmsnorm_partials(x.data_ptr(), _dev(parts, "partials", torch.float32), int(slices),
-                                       _dev(weight, "weight", torch.float32, (dim,)), _dev(out, "out", None, (rows, dim)),
+    if not partials_ok(x) or out.data_ptr() % 16:
+        raise KernelError("rmsnorm_partials: contiguous float rows of a multiple of 4 (at most 8192)")
+    wp, op = _dev(weight, "weight", torch.float32, (dim,)), _dev(out, "out", None, (rows, dim))
+    if slices == 0:
+        _check(lib().cisr_add_rmsnorm_bf16(x.data_ptr(), _dev(parts, "product", torch.bfloat16, (rows, dim)), wp, op, rows, dim,
+                                           float(eps), _storage(out, "out"), _stream()), "rmsnorm_partials")
+        return out
+    if parts.numel() < slices * rows * dim:
+        raise KernelError("rmsnorm_partials: too few partial sums")
+    _check(lib().cisr_rmsnorm_partials(x.data_ptr(), _dev(parts, "partials", torch.float32), int(slices), wp, op,
                                        rows, dim, float(eps), _storage(out, "out"), _stream()), "rmsnorm_partials")
     return out
 
@@ -294,9 +304,11 @@ def attention_rowwise(q, q_row_stride, kcache, vcache, tables, seg_of_row, posit
 # 39.9 ms); at 65-255 rows with weights streamed from HBM it is up to 2.5 times as fast on narrow outputs with
 # a long inner size, which leave the tiled kernel few tiles (it does not cut K).  With at most 64 rows the
 # weight-streaming kernels here are as fast or faster (8 rows: 50 against 67 us for gate and up of the 8B
-# sizes), as are all products of small weights, and both save the kernel after the product.  0 rows: never.
+# sizes), as are all products of small weights, and both save the kernel after the product.  The least weights are
+# those of the 1.7B sizes' output projection (8 MB: 10.7 against 13.9 us at 128 rows, 29 against 33 at 2,048, the
+# residual sum included; the products of the 135M sizes, 0.7 to 3.5 MB, are as fast or faster here).  0 rows: never.
 LIBRARY_MIN_ROWS = int(os.environ.get("CISR_LIBRARY_MIN_ROWS", "65"))
-LIBRARY_MIN_BYTES = int(float(os.environ.get("CISR_LIBRARY_MIN_MB", "16")) * (1 << 20))
+LIBRARY_MIN_BYTES = int(float(os.environ.get("CISR_LIBRARY_MIN_MB", "8")) * (1 << 20))
 _library_scratch = {}   # (device, elements) -> bf16 buffers, never freed: captured programs keep their addresses
 
 
@@ -437,15 +449,22 @@ def _gemm_wide(a, w, out, residual, swiglu, what):
 
 
 def gemm_unfinished(a, w, residual):
-    """The product a . w^T that is to be added to the float rows `residual`, left unfinished where the wide kernel
-    cuts it into slices and would need a second kernel to add them: returns (partial sums [slices, M, N], slices)
-    for rmsnorm_partials or add_partials, which then are that second kernel; None (nothing done) for every other
-    product: call gemm."""
+    """The product a . w^T that is to be added to the float rows `residual`, left unfinished where adding it takes a
+    kernel of its own: the wide kernel's partial sums of a product cut into slices, (partial sums [slices, M, N],
+    slices), or the library's bf16 product, (product [M, N], 0); rmsnorm_partials or add_partials then are that
+    kernel.  None (nothing done) for every other product: call gemm."""
     m, k = a.shape
     n = w.shape[0]
-    if (a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or w.shape[1] != k or not 0 < m <= SKINNY_ROWS
-            or library_ok(m, w) or not _skinny_ok(a, w) or not wide_ok(m, w) or tuple(residual.shape) != (m, n)
+    if (a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or w.shape[1] != k or tuple(residual.shape) != (m, n)
             or not partials_ok(residual)):
+        return None
+    if library_ok(m, w):
+        if not a.is_contiguous():
+            return None
+        product = _scratch_bf16(a.device, m, n)
+        torch.mm(a, w.t(), out=product)
+        return product, 0
+    if not 0 < m <= SKINNY_ROWS or not _skinny_ok(a, w) or not wide_ok(m, w):
         return None
     need = _wide_plan(m, n, k, False)
     if need <= 0:

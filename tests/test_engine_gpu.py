@@ -263,8 +263,8 @@ def test_layers_of_real_sizes_match_the_plain_model(tmp_path_factory, sizes, exe
     """Layers of real sizes: the sizes at which products choose other kernels by themselves (the wide
     weight-streaming product for decode steps, with the fused projection finishing in it; the vendor's library
     for portions of more than 64 rows).  Whole prompts, portions, decode steps of several requests and mixed
-    steps against the plain model.  Between the two layers of the 1.7B sizes the down projection of few rows is left
-    as partial sums to the next layer's norm."""
+    steps against the plain model.  Products that end a part are left to the norm that follows: the slices of
+    the wide product with few rows, the library's result with many."""
     from runtime.engine import load_model, ModelRunner, StepEntry
     from runtime.kernels import ops
     from conftest import write_folder, plain_logits, assert_close
@@ -308,9 +308,9 @@ def test_layers_of_real_sizes_match_the_plain_model(tmp_path_factory, sizes, exe
     if execution == "graph":
         replayed = [key for key, p in runner.programs.items() if p["graph"] is not None and p["runs"] >= 3]
         assert any(key[0] > 64 for key in replayed) and any(key[3] for key in replayed)
-    if sizes == "1.7b":
-        assert sum(u is not None for u in left) >= 3, "no product was left to the norm that follows"
-    assert sum(u is None for u in left) >= 1 or sizes != "1.7b"      # (many rows: not taken)
+    if sizes == "1.7b":     # few rows: the wide product's slices; many rows: the library's bf16 product
+        assert sum(u is not None and u[1] > 1 for u in left) >= 3, "no cut product was left to the norm that follows"
+        assert sum(u is not None and u[1] == 0 for u in left) >= 3, "no library product was left to the norm that follows"
     runner.cache.check()
 
 

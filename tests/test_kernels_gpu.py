@@ -681,34 +681,39 @@ def test_gemm_wide_at_the_sizes_that_choose_it(ops, M):
     torch.testing.assert_close(y, x.float() @ w_n.float().T, rtol=1e-4, atol=1e-4)
 
 
-@pytest.mark.parametrize("M", [4, 8, 40, 64])
+@pytest.mark.parametrize("M", [4, 8, 40, 64, 100, 300])
 def test_product_left_unfinished_is_added_by_the_norm_that_follows(ops, M, monkeypatch):
     """A product that the wide kernel cuts along its inner size may leave its slices' partial sums to the kernel that
     reads the rows next: sum + residual + norm in one kernel, or the sum alone; the rows are bit for bit what the
     product's own second kernel gives, the norm differs by the order of its sum of squares only.  Products that are
-    not cut (or not wide) are not taken."""
+    not cut (or not wide) are not taken.  With more than 64 rows the product is the library's and what is left to
+    the next kernel is its bf16 result (slices 0): the same rows and the same norm, bit for bit."""
     torch.manual_seed(M)
     N, K = 2048, 8192                       # the down projection of the 1.7B sizes
     w = (torch.randn(N, K, device=DEV) * 0.02).bfloat16()
     a = (torch.randn(M, K, device=DEV) * 0.5).bfloat16()
     r = torch.randn(M, N, device=DEV)
     nw = 1 + 0.1 * torch.randn(N, device=DEV)
-    assert ops.wide_ok(M, w)
+    assert ops.wide_ok(M, w) if M <= 64 else ops.library_ok(M, w)
     want_x = r.clone()
     ops.gemm(a, w, want_x, residual=want_x)
     for out_dtype in (torch.bfloat16, torch.float32):
         want_y = ops.rmsnorm(want_x, nw, torch.empty(M, N, dtype=out_dtype, device=DEV), 1e-5)
         x = r.clone()
         partials = ops.gemm_unfinished(a, w, x)
-        assert partials is not None and partials[1] > 1
+        assert partials is not None and (partials[1] > 1 if M <= 64 else partials[1] == 0)
         assert torch.equal(x, r)            # nothing added yet
         y = ops.rmsnorm_partials(x, partials, nw, torch.empty(M, N, dtype=out_dtype, device=DEV), 1e-5)
         assert torch.equal(x, want_x)
+        if M > 64:
+            assert torch.equal(y, want_y)
         torch.testing.assert_close(y.float(), want_y.float(), rtol=1e-2 if out_dtype == torch.bfloat16 else 1e-5, atol=1e-5)
     x = r.clone()
     ops.add_partials(x, ops.gemm_unfinished(a, w, x))
     assert torch.equal(x, want_x)
-    torch.testing.assert_close(x, r + a.float() @ w.float().T, rtol=1e-4, atol=1e-4)
+    torch.testing.assert_close(x, r + a.float() @ w.float().T, rtol=1e-4 if M <= 64 else 2e-2, atol=1e-4 if M <= 64 else 2e-2)
+    if M > 64:
+        return
     # not taken: small weights (another kernel), a product of one slice, rows that are no contiguous floats
     small = (torch.randn(64, 128, device=DEV) * 0.02).bfloat16()
     assert ops.gemm_unfinished(a[:, :128].contiguous(), small, torch.zeros(M, 64, device=DEV)) is None

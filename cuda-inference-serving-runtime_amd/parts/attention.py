@@ -81,7 +81,7 @@ class PagedAttention(Mixer):
             ops.rope_scatter(q, ctx.positions, slots, cos, sin, kcache_w, vcache_w, nh, nkv, D, view.page_size)
         out = ctx.buffer("attn.out", (T, nh * D), ctx.dtype)
         ctx.attend(q, q_stride, kcache, vcache, view, out, nh, nkv, D, self.window, self.scale)
-        return ops.gemm(out, self.w_out, residual, residual=residual)
+        return ctx.add_product(out, self.w_out, residual)
 
 
 register_part("mixer", "attention", PagedAttention)

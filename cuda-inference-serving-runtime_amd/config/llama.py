@@ -6,7 +6,7 @@ key of its own (the reference requires it to equal hidden/heads,
 runtime/checkpoint.py:17; here any even size up to 256 in the projections'
 shapes is allowed).
 """
-from dataclasses import dataclass, fields, asdict
+from dataclasses import dataclass, asdict
 from typing import Optional, Tuple
 
 from .base import ConfigError

@@ -18,7 +18,7 @@ and the norm part, and the part applies the norm inside its first kernel.
 A mixer states what it keeps between steps: `cache_need()` (pages of keys and
 values) and/or `state_need()` (a fixed-size state per request), or neither.
 """
-from ..weights.loader import TensorSpec
+from ..weights.loader import TensorSpec  # noqa: F401  (parts import it from here)
 
 _PARTS = {}
 

@@ -5,7 +5,7 @@ import pytest
 import torch
 
 import plain_llama as P
-from conftest import TINY
+
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"

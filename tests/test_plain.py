@@ -2,7 +2,6 @@
 special cases that reduce to a library routine, and invariants, each chosen so
 that a plausible mistake fails it."""
 import numpy as np
-import pytest
 import torch
 
 import plain_llama as P

@@ -5,13 +5,13 @@ with so few pages that they are used again; long decoding; the first tokens."""
 import os
 import subprocess
 import sys
-from pathlib import Path
+
 
 import numpy as np
 import pytest
 
 from conftest import ROOT, TINY, random_tokens
-from trace_tools import Trace, ceil64
+from trace_tools import Trace
 
 pytestmark = pytest.mark.gpu
 DTYPES = ["float32", "bfloat16"]

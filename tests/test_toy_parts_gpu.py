@@ -112,9 +112,9 @@ def plain_toy(raw, w, tokens):
 
 
 def test_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path):
-    import json
+
     import plain_llama as P
-    from runtime.engine import load_model, write_random_model, ModelRunner, StepEntry
+    from runtime.engine import load_model, ModelRunner, StepEntry
     cleanup = build_toy()
     try:
         raw = {"model_type": "toy-decay-lm", "vocab_size": 61, "hidden_size": 24, "decay": 0.7,

@@ -27,6 +27,23 @@ def test_append_slots_follow_the_block_table():
     m.check()
 
 
+def test_report_counts_resident_peak_free_and_shared_pages():
+    # reference runtime/cache.py:109-118 (pool, resident, peak, free, shared, sequences)
+    m = manager(pages=8, page_size=4, sites=2)
+    m.create("a")
+    m.append_many([("a", 9)])                      # three pages
+    m.fork("a", "b")                               # shared by two requests
+    m.append_many([("b", 1)])                      # copy-on-write of the partly filled last page
+    (r,) = m.report()
+    assert r["sites"] == 2 and r["pages"] == 8 and r["requests"] == 2 and r["window"] is None
+    assert r["resident_pages"] == 4 and r["free_pages"] == 4 and r["shared_pages"] == 2 and r["peak_pages"] == 4
+    assert r["elements_per_token"] == 2 * 2 * 16 * 2
+    m.release("a"); m.release("b")
+    (r,) = m.report()
+    assert r["resident_pages"] == 0 and r["free_pages"] == 8 and r["peak_pages"] == 4 and r["requests"] == 0
+    m.check()
+
+
 def test_sites_with_equal_needs_share_one_group():
     m = manager(sites=3, window=5)
     assert len(m.groups) == 2 and len(m.groups[0].sites) == 3 and m.groups[1].need.window == 5

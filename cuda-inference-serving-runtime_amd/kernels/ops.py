@@ -631,8 +631,8 @@ def attention_mfma(q, q_row_stride, kcache, vcache, tables, seg_of_row, position
     if q.numel() < (rows - 1) * q_row_stride + heads * dim:
         raise KernelError("attention: q buffer too small for its stride")
     pages = kcache.shape[0]
-    if kcache.numel() >= 2 ** 32 or vcache.numel() >= 2 ** 32:
-        raise KernelError("attention_mfma: a layer's keys (or values) must be fewer than 2^32 elements (32-bit offsets)")
+    if kcache.numel() >= 2 ** 31 or vcache.numel() >= 2 ** 31:
+        raise KernelError("attention_mfma: a layer's keys (or values) must be fewer than 2^31 elements (32-bit byte offsets)")
     dpad = -(-dim // 32) * 32
     fn = _attention_entry(dpad)
     po = pm = tp = None

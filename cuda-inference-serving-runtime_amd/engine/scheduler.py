@@ -272,6 +272,9 @@ class Engine:
         if not pages:
             free, _ = torch.cuda.mem_get_info(torch.device(device))
             addressable = max_requests * -(-model.max_positions // page_size)
+            # (the attention kernels address a site's keys with 32-bit byte offsets: fewer than 2^31 elements)
+            widest = max(need.kv_heads * need.head_dim for need in model.cache_needs().values() if need is not None)
+            addressable = min(addressable, (2 ** 31 - 1) // (widest * page_size))
             pages = pages_that_fit(model.cache_needs(), page_size, 2 if dtype == "bfloat16" else 4, free, most=addressable)
         runner = ModelRunner(model, n_pages=pages, page_size=page_size, max_requests=max_requests, device=device,
                              execution=execution)

@@ -149,7 +149,7 @@ gemm_bf16_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict
     __shared__ __attribute__((aligned(16))) bf16_t As[2][BM * BK];
     __shared__ __attribute__((aligned(16))) bf16_t Ws[2][BN * BK];
 
-    const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / WAVE), lane = tid % WAVE;   // (uniform: scalar loop control)
     const int wm = wave / 2, wn = wave % 2;
     const int r = lane % 16, g = lane / 16;
     // The hardware deals consecutive workgroups round-robin to the 8 XCDs, each with an L2 of its own.

@@ -92,7 +92,7 @@ __global__ void __launch_bounds__(NW * 64)
 gemm_wide_kernel(WideArgs p) {
     extern __shared__ float smem[];
     float (*red)[NB][MT][4][WAVE] = reinterpret_cast<float (*)[NB][MT][4][WAVE]>(smem);   // [wave][block][tile][e][lane]
-    const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / WAVE), lane = tid % WAVE;   // (uniform: scalar loop control)
     const int r = lane % 16, g = lane / 16;
     const int M = p.M, N = p.N, K = p.K;
     constexpr int TSTEP = NW / 4;                                 // NW is a multiple of 4

@@ -53,7 +53,7 @@ template <typename T, int R>
 __global__ void __launch_bounds__(256)
 rmsnorm_wave_kernel(const float* __restrict__ x, const float* __restrict__ w, T* __restrict__ y,
                     const int* __restrict__ rows, int n_out, int dim, float eps) {
-    const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE), lane = threadIdx.x % WAVE;   // (uniform: the row's loads of indices are scalar)
     const int orow = blockIdx.x * 4 + wave;
     if (orow >= n_out) return;
     const int irow = rows ? rows[orow] : orow;
@@ -221,7 +221,7 @@ template <typename T, int R>
 __global__ void __launch_bounds__(256)
 add_rmsnorm_wave_kernel(float* x, const bf16_t* __restrict__ delta, const float* __restrict__ w, T* __restrict__ y,
                         int n_rows, int dim, float eps) {
-    const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE), lane = threadIdx.x % WAVE;   // (uniform: the row's loads of indices are scalar)
     const int row = blockIdx.x * 4 + wave;
     if (row >= n_rows) return;
     const int n4 = dim / 4;
@@ -509,7 +509,7 @@ rope_scatter_wave_kernel(bf16_t* __restrict__ qkv, const int* __restrict__ posit
     }
     const bool values_here = qk_blocks == (int)gridDim.x;   // no value blocks: every row writes its own
     const int lane = threadIdx.x % lanes;
-    const int row = blockIdx.x * (256 / lanes) + threadIdx.x / lanes;
+    const int row = blockIdx.x * (256 / lanes) + __builtin_amdgcn_readfirstlane(threadIdx.x / lanes);   // lanes is a multiple of 64: uniform in a wave
     if (row >= rows) return;
     const int half = dim / 2, per_head = half / 8;   // 8-pair chunks of a head
     int pos = positions[row];

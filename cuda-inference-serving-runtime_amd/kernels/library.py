@@ -98,9 +98,9 @@ def library_path(unit=CORE, create=False):
     for d in _build_dirs():
         try:
             d.mkdir(parents=True, exist_ok=True)
-            probe = d / f".w{os.getpid()}"
-            probe.write_text("")
-            probe.unlink()
+            fd, probe = tempfile.mkstemp(prefix=".w", dir=str(d))   # (a name of its own: units are built side by side)
+            os.close(fd)
+            os.unlink(probe)
             return d / name
         except OSError:
             continue

@@ -5,6 +5,9 @@
 // what else is in the batch.  One block of 256 threads per row; every thread
 // owns one contiguous slice of the vocabulary, which fixes the summation order.
 #include "common.h"
+#include "cisr_noalloc.h"
+#include <stdio.h>
+#include <mutex>
 
 __device__ __forceinline__ uint64_t splitmix64(uint64_t x) {
     x += 0x9E3779B97F4A7C15ull;
@@ -87,6 +90,58 @@ extern "C" int cisr_argmax(const float* logits, int* out, const int* index, int 
     int err = CISR_LAUNCH_CHECK();
     if (err) return err;
     argmax_final_kernel<<<rows, 64, 0, stream>>>(scratch_val, scratch_idx, out, index, index ? out_n : rows, ARGMAX_CHUNKS);
+    return CISR_LAUNCH_CHECK();
+}
+
+// The slice winners of cisr_argmax_noalloc: values (float) then indices (int), 32 of each a row.  In host code
+// this name is only a stand-in for the symbol, not a device address; the address on each device comes from
+// hipGetSymbolAddress and is kept in noalloc_scratch[].
+static __device__ __align__(256) unsigned char scratch[CISR_ARGMAX_NOALLOC_MAX_ROWS * ARGMAX_CHUNKS * (sizeof(float) + sizeof(int))];
+
+#define NOALLOC_MAX_DEVICES 64
+static void* noalloc_scratch[NOALLOC_MAX_DEVICES];     // per device: each GPU holds its own copy at its own address
+static std::mutex noalloc_lock;
+
+static int noalloc_scratch_of_current_device(void** ptr) {
+    int device = -1;
+    hipError_t e = hipGetDevice(&device);
+    if (e != hipSuccess) return (int)e;
+    if (device < 0 || device >= NOALLOC_MAX_DEVICES) return (int)hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> guard(noalloc_lock);
+    if (noalloc_scratch[device] == nullptr) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return (int)e;
+        if (p == nullptr) return (int)hipErrorInvalidSymbol;
+        noalloc_scratch[device] = p;
+    }
+    *ptr = noalloc_scratch[device];
+    return 0;
+}
+
+extern "C" int cisr_noalloc_init(void) {
+    void* p = nullptr;
+    return noalloc_scratch_of_current_device(&p);
+}
+
+extern "C" int cisr_argmax_noalloc_max_rows(void) { return CISR_ARGMAX_NOALLOC_MAX_ROWS; }
+
+extern "C" int cisr_argmax_noalloc(const float* logits, int* out, int rows, int vocab, hipStream_t stream) {
+    if (rows == 0) return 0;
+    if (rows < 0 || rows > CISR_ARGMAX_NOALLOC_MAX_ROWS || vocab <= 0 || logits == nullptr || out == nullptr) {
+        fprintf(stderr, "cisr_argmax_noalloc: %d rows of %d logits refused (1 to %d rows, a vocabulary of at least 1, "
+                        "no null pointers)\n", rows, vocab, CISR_ARGMAX_NOALLOC_MAX_ROWS);
+        return (int)hipErrorInvalidValue;
+    }
+    void* base = nullptr;
+    int err = noalloc_scratch_of_current_device(&base);
+    if (err) return err;
+    float* pval = (float*)base;
+    int* pidx = (int*)((unsigned char*)base + (size_t)CISR_ARGMAX_NOALLOC_MAX_ROWS * ARGMAX_CHUNKS * sizeof(float));
+    argmax_partial_kernel<<<dim3(rows, ARGMAX_CHUNKS), 256, 0, stream>>>(logits, pval, pidx, vocab, ARGMAX_CHUNKS);
+    err = CISR_LAUNCH_CHECK();
+    if (err) return err;
+    argmax_final_kernel<<<rows, 64, 0, stream>>>(pval, pidx, out, nullptr, rows, ARGMAX_CHUNKS);
     return CISR_LAUNCH_CHECK();
 }
 

@@ -28,12 +28,14 @@ def build_from_config_dict(raw):
     return arch, config, arch.build(config)
 
 
-def load_model(folder, dtype="bfloat16", device="cuda:0"):
-    """The model of `folder` with its weights on `device`, ready to step."""
+def load_model(folder, dtype="bfloat16", device="cuda:0", strict=False):
+    """The model of `folder` with its weights on `device`, ready to step.  Tensors that the model does not
+    declare are left alone unless `strict`."""
     dtype = parse_dtype(dtype)
     raw = read_config_json(folder)
     _, _, model = build_from_config_dict(raw)
-    tensors = load_folder(folder, model.tensor_specs(), dtype, torch.device(device), ignored=model.ignored_tensors())
+    tensors = load_folder(folder, model.tensor_specs(), dtype, torch.device(device), ignored=model.ignored_tensors(),
+                          strict=strict)
     model.bind(tensors, dtype, torch.device(device))
     return model
 

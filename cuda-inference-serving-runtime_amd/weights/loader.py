@@ -6,12 +6,20 @@ may appear once: runtime/checkpoint.py:18-19,36 in the reference), checks the
 whole set at once and raises ONE error that lists missing tensors, unexpected
 tensors and wrong shapes.  Nothing is renamed.
 
+A tensor that the model does not declare is no fault by itself: the reference
+checks the expected names and shapes only (runtime/checkpoint.py:44-58), and
+checkpoints carry buffers such as ``...rotary_emb.inv_freq``.  Such a folder
+loads, with one line on stderr that names the extras; they are listed in the
+error when something else is wrong (a misspelt name shows as one missing and
+one unexpected tensor), and ``strict=True`` makes them an error of their own.
+
 Dtype rule.  ``dtype=bfloat16``: bfloat16 tensors stay bfloat16, a tensor that
 the file stores in 32 bits stays in 32 bits, float16 is widened to float32
 first, integer tables become int32.  ``dtype=float32``: every floating tensor
 is widened to float32 (exact).  What a kernel then needs (a bf16 matrix operand,
 a float norm weight) is the business of the part that owns the tensor.
 """
+import sys
 from dataclasses import dataclass
 from pathlib import Path
 from typing import Tuple
@@ -51,8 +59,9 @@ def open_folder(folder):
     return index
 
 
-def check_against(specs, index, ignored=()):
-    """Raise one WeightError naming every missing, unexpected and mis-shaped tensor.
+def check_against(specs, index, ignored=(), strict=False):
+    """Raise one WeightError naming every missing, unexpected and mis-shaped tensor, if a tensor is
+    missing or mis-shaped (or, with `strict`, unexpected).  Returns the unexpected names otherwise.
     `ignored` names tensors a checkpoint may carry without the model using them."""
     expected = {s.name: s for s in specs}
     missing = sorted(n for n in expected if n not in index)
@@ -63,7 +72,7 @@ def check_against(specs, index, ignored=()):
             _, shape = index[name].info(name)
             if tuple(shape) != tuple(spec.shape):
                 wrong.append(f"{name}: file has {list(shape)}, model expects {list(spec.shape)}")
-    if missing or unexpected or wrong:
+    if missing or wrong or (strict and unexpected):
         lines = ["checkpoint does not match the model:"]
         if missing:
             lines.append(f"  missing ({len(missing)}): " + ", ".join(missing))
@@ -72,6 +81,7 @@ def check_against(specs, index, ignored=()):
         if wrong:
             lines.append(f"  wrong shape ({len(wrong)}): " + "; ".join(sorted(wrong)))
         raise WeightError("\n".join(lines))
+    return unexpected
 
 
 def _kept_dtype(stored, integer, dtype):
@@ -84,10 +94,13 @@ def _kept_dtype(stored, integer, dtype):
     return torch.float32  # stored in 32 bits (or float16/float64): kept in 32 bits
 
 
-def load_folder(folder, specs, dtype, device, ignored=()):
+def load_folder(folder, specs, dtype, device, ignored=(), strict=False):
     """{name: tensor on `device`} for every spec, after the whole-set check."""
     index = open_folder(folder)
-    check_against(specs, index, ignored)
+    extras = check_against(specs, index, ignored, strict)
+    if extras:
+        shown = ", ".join(extras[:8]) + (f", ... ({len(extras)} in all)" if len(extras) > 8 else "")
+        print(f"[runtime.weights] {folder}: tensors that the model does not use are left alone: {shown}", file=sys.stderr)
     out = {}
     for spec in specs:
         t = index[spec.name].tensor(spec.name)

@@ -140,6 +140,23 @@ def test_loader_lists_everything_wrong_in_one_error(tmp_path):
     assert untied.ignored_tensors() == ()
 
 
+def test_loader_leaves_extra_tensors_alone(tmp_path, capsys):
+    """A tensor the model does not declare is no fault by itself (the reference checks the expected set only,
+    runtime/checkpoint.py:44-58): the folder loads, the extra is named on stderr; strict mode refuses it."""
+    from safetensors.torch import load_file, save_file
+    folder = write_folder(tmp_path / "m", TINY["a"], 0)
+    tensors = load_file(str(folder / "model.safetensors"))
+    tensors["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.zeros(8)
+    save_file(tensors, str(folder / "model.safetensors"))
+    _, _, model = build_from_config_dict(raw("a"))
+    got = load_folder(folder, model.tensor_specs(), torch.bfloat16, "cpu", ignored=model.ignored_tensors())
+    assert set(got) == {s.name for s in model.tensor_specs()}
+    assert "rotary_emb.inv_freq" in capsys.readouterr().err
+    assert check_against(model.tensor_specs(), open_folder(folder)) == ["model.layers.0.self_attn.rotary_emb.inv_freq"]
+    with pytest.raises(WeightError, match="unexpected \\(1\\)"):
+        load_folder(folder, model.tensor_specs(), torch.bfloat16, "cpu", ignored=model.ignored_tensors(), strict=True)
+
+
 def test_loader_duplicate_across_shards_and_empty_folder(tmp_path):
     from safetensors.torch import save_file
     with pytest.raises(FileNotFoundError):

@@ -7,8 +7,10 @@ zeroing of a fresh state slot) goes through two callbacks.
 
 Per step the step function calls `append_many([(request, n_tokens), ...])`,
 which is atomic: either every request gets its slots in every group, or
-OutOfPages is raised and nothing has changed (the reference preflights every
-layer before mutating any, runtime/model.py:98-102).
+OutOfPages is raised and no request has gained a token, a slot or a page (the
+reference preflights every layer before mutating any, runtime/model.py:98-102);
+the only thing a refused step may have done is to give back pages that a window
+had passed, which no later query reads.
 """
 from dataclasses import dataclass, field
 
@@ -124,6 +126,13 @@ class CacheManager:
             seen.add(request)
         if self.fast_decode and all(n == 1 for _, n in items) and all(g.need.window is None for g in self.groups):
             return self._append_one_each(items)
+        # Windows first give back, for every request of the step, the pages that no later query can see; only then
+        # are fresh pages counted and taken.  (Trimmed one request at a time, a request that needs a page could
+        # come before the one whose window frees it, and run out in the middle of the step.)  Giving such a page
+        # back changes nothing that a retry of the step would read.
+        for request, _ in items:
+            for group in self.groups:
+                group.trim(request, self.lengths[request])
         if not self.can_append(items):
             raise OutOfPages("not enough free KV pages for this step")
         result = []
@@ -131,7 +140,6 @@ class CacheManager:
             length = self.lengths[request]
             done = Appended(request, length, n, state_slot=self.slots.slot_of(request))
             for gid, group in enumerate(self.groups):
-                group.trim(request, length)
                 slots, copies = group.append(request, length, n)
                 done.slots[gid] = slots
                 if copies and self._copy_pages is not None:

@@ -127,6 +127,35 @@ def test_window_gives_pages_back_once_passed():
     m.check()
 
 
+def test_window_step_is_atomic_whatever_the_order_of_its_requests():
+    """No free page, one request of the step needs a page and a LATER one frees one through its window: the step
+    is served (pages are given back for all requests before any is taken).  And when it cannot be served, no
+    request has moved."""
+    def fill(order):
+        m = manager(pages=4, page_size=4, sites=0, window=4)
+        for r in "abc":
+            m.create(r)
+        m.append_many([("a", 4)])              # a: one full page, its next token needs a fresh one
+        m.append_many([("b", 7)])              # b: two pages; its next token (position 7) sees 4..7: page 0 is dead
+        m.append_many([("c", 2)])              # c: one page, partly filled
+        assert m.free_pages() == [0]
+        return m, [(r, 1) for r in order]
+    for order in ("cab", "abc", "bca"):
+        m, items = fill(order)
+        assert m.can_append(items)
+        done = {d.request: d for d in m.append_many(items)}
+        assert (m.length("a"), m.length("b"), m.length("c")) == (5, 8, 3)
+        assert m.table(0, "b")[0] == -1 and done["a"].slots[0][0] % 4 == 0
+        m.check()
+    # without b in the step nothing is freed: the step is refused and nobody has moved
+    m, _ = fill("ca")
+    before = ({r: m.length(r) for r in "abc"}, {r: list(m.table(0, r)) for r in "abc"})
+    with pytest.raises(OutOfPages):
+        m.append_many([("c", 1), ("a", 1)])
+    assert before == ({r: m.length(r) for r in "abc"}, {r: list(m.table(0, r)) for r in "abc"})
+    m.check()
+
+
 def test_window_group_never_needs_more_than_window_plus_portion():
     m = manager(pages=4, page_size=4, sites=0, window=8)
     m.create("a")

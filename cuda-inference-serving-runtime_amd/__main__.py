@@ -3,7 +3,8 @@
 Options keep the names and meanings of the reference's command line
 (runtime/__main__.py:13-26); `--device cpu` does not exist here (there is no CPU
 path), `--dtype float16` is not built, `--execution buffered` is what `eager`
-already is (stable buffers, explicit kernels).  Added: `--model` (a named
+already is (stable buffers, explicit kernels), and `--execution` defaults to
+`graph` (the reference's default, eager, is the slow path in both).  Added: `--model` (a named
 configuration with seeded random weights when no checkpoint is given),
 `--seed`, `--temperature`, `--max-active`.
 """
@@ -18,7 +19,9 @@ def main(argv=None):
     parser = argparse.ArgumentParser(prog="python -m runtime", description=__doc__)
     parser.add_argument("--device", choices=["hip", "cuda"], default="hip", help="the MI355X (both names mean it)")
     parser.add_argument("--dtype", choices=["float32", "bfloat16"], default="bfloat16")
-    parser.add_argument("--execution", choices=["eager", "buffered", "graph"], default="eager")
+    parser.add_argument("--execution", choices=["eager", "buffered", "graph"], default="graph",
+                        help="graph: every step as a captured program (the default here: it is the fast path); "
+                             "eager or buffered: kernels launched one by one")
     parser.add_argument("--checkpoint", type=Path, help="folder with config.json and *.safetensors")
     parser.add_argument("--model", default="tiny-a", help="named configuration for random weights (no --checkpoint)")
     parser.add_argument("--seed", type=int, default=0, help="seed of random weights and of sampling")

@@ -113,8 +113,10 @@ class CacheManager:
     def can_append(self, items):
         return all(need <= len(group.pool.free) for need, group in zip(self.pages_needed(items), self.groups))
 
-    def append_many(self, items):
-        """items: [(request, n_new)], each request at most once.  Returns [Appended]."""
+    def append_many(self, items, commit=True):
+        """items: [(request, n_new)], each request at most once.  Returns [Appended].
+        With commit=False the slots are placed but the requests' lengths stay: the caller calls `commit(done)`
+        once the step that writes the slots is launched, or `abandon(done)` if it could not be."""
         seen = set()
         for request, n in items:
             if request not in self.lengths:
@@ -125,7 +127,7 @@ class CacheManager:
                 raise ValueError("a request must bring at least one token")
             seen.add(request)
         if self.fast_decode and all(n == 1 for _, n in items) and all(g.need.window is None for g in self.groups):
-            return self._append_one_each(items)
+            return self._append_one_each(items, commit)
         # Windows first give back, for every request of the step, the pages that no later query can see; only then
         # are fresh pages counted and taken.  (Trimmed one request at a time, a request that needs a page could
         # come before the one whose window frees it, and run out in the middle of the step.)  Giving such a page
@@ -144,11 +146,32 @@ class CacheManager:
                 done.slots[gid] = slots
                 if copies and self._copy_pages is not None:
                     self._copy_pages(group, copies)
-            self.lengths[request] = length + n
+            if commit:
+                self.lengths[request] = length + n
             result.append(done)
         return result
 
-    def _append_one_each(self, items):
+    def commit(self, done):
+        """The step that fills the slots of `done` (append_many with commit=False) is on its way: the tokens count."""
+        for d in done:
+            if self.lengths[d.request] != d.start:
+                raise RuntimeError(f"request {d.request!r} moved between its append and its commit")
+            self.lengths[d.request] = d.start + d.count
+        return done
+
+    def abandon(self, done):
+        """The step of `done` (append_many with commit=False) was never launched: pages taken for its tokens go
+        back, the requests stand where they stood.  (A page copied for a write stays copied, pages that a window
+        had passed stay given back: neither changes what a later step reads.)"""
+        for d in done:
+            keep = -(-self.lengths[d.request] // self.page_size)
+            for group in self.groups:
+                table = group.tables[d.request]
+                while len(table) > keep:
+                    group.pool.drop(table.pop())
+                    group._touch(d.request)
+
+    def _append_one_each(self, items, commit=True):
         """append_many for the common step in which every request brings one token and no group has a
         window: the same pages in the same order, with the counting and the placing done in line."""
         P = self.page_size
@@ -174,7 +197,8 @@ class CacheManager:
                     if copies and self._copy_pages is not None:
                         self._copy_pages(group, copies)
                 done.slots[gid] = [table[-1] * P + length % P]
-            lengths[request] = length + 1
+            if commit:
+                lengths[request] = length + 1
             result.append(done)
         return result
 
@@ -207,6 +231,24 @@ class CacheManager:
 
     def free_pages(self):
         return [len(g.pool.free) for g in self.groups]
+
+    def capacity(self):
+        """Pages of each group's pool."""
+        return [g.pool.n_pages for g in self.groups]
+
+    def most_pages_held(self, tokens, portion):
+        """Per group, the most pages one request holds at any time while it grows to `tokens` cached tokens in
+        steps of at most `portion`: all of them where every key is kept; where only a window is kept, the pages
+        that a window and a portion can touch (a portion is placed after the pages behind its first token's
+        window went back)."""
+        P = self.page_size
+        out = []
+        for group in self.groups:
+            pages = -(-tokens // P)
+            if group.need.window is not None:
+                pages = min(pages, (group.need.window + max(1, portion) - 1) // P + 2)
+            out.append(pages)
+        return out
 
     def report(self):
         out = []

@@ -40,10 +40,10 @@ def load_model(folder, dtype="bfloat16", device="cuda:0", strict=False):
     return model
 
 
-def write_random_model(folder, config, seed, dtype="bfloat16"):
+def write_random_model(folder, config, seed, dtype="bfloat16", std=None):
     """Write config.json and model.safetensors for `config` (a config.json dict or
-    the name of a preset) with seeded random weights."""
+    the name of a preset) with seeded random weights: N(0, std), norms 1 + N(0, std); std 0.02 unless given."""
     raw = preset(config) if isinstance(config, str) else dict(config)
     _, typed, model = build_from_config_dict(raw)
     return write_model_folder(folder, typed.to_dict() if hasattr(typed, "to_dict") else raw,
-                              model.tensor_specs(), seed, parse_dtype(dtype))
+                              model.tensor_specs(), seed, parse_dtype(dtype), **({} if std is None else {"std": std}))

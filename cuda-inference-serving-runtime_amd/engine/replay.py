@@ -26,12 +26,14 @@ PAGE_SIZE = 16          # divides 64, so a request rounded up to 64 tokens never
 MAX_LIVE = 4
 
 
-def replay(model_dir, dtype, out_dir, max_tokens, lines, page_size=PAGE_SIZE, echo=print):
+def replay(model_dir, dtype, out_dir, max_tokens, lines, page_size=PAGE_SIZE, echo=print, execution="eager"):
+    """`execution`: "eager" launches every step's kernels one by one; "graph" runs every step as a captured program
+    (the way serving decodes), padded to its bucket of rows, segments and wanted rows."""
     out_dir = Path(out_dir)
     out_dir.mkdir(parents=True, exist_ok=True)
     model = load_model(model_dir, dtype=dtype)
     pages = max(1, -(-int(max_tokens) // page_size))
-    runner = ModelRunner(model, n_pages=pages, page_size=page_size, max_requests=4 * MAX_LIVE)
+    runner = ModelRunner(model, n_pages=pages, page_size=page_size, max_requests=4 * MAX_LIVE, execution=execution)
     for line in lines:
         line = line.strip()
         if not line:
@@ -62,10 +64,12 @@ def main(argv=None):
     parser.add_argument("--out", required=True, help="folder for <step>.f32 files")
     parser.add_argument("--max-tokens", type=int, required=True,
                         help="most tokens live requests hold at any time (each rounded up to 64)")
+    parser.add_argument("--execution", choices=["eager", "graph"], default="eager",
+                        help="eager: kernels launched one by one; graph: every step as a captured program")
     args = parser.parse_args(argv)
 
     def echo(text):
         print(text, flush=True)
 
-    replay(args.model, args.dtype, args.out, args.max_tokens, sys.stdin, echo=echo)
+    replay(args.model, args.dtype, args.out, args.max_tokens, sys.stdin, echo=echo, execution=args.execution)
     return 0

@@ -161,12 +161,21 @@ class ModelRunner:
     def step(self, entries: List[StepEntry]):
         """Float logits [sum(len(want)), vocab] on the GPU (valid until the next step)."""
         self.check(entries)
-        done = self.cache.append_many([(e.request, len(e.tokens)) for e in entries])  # OutOfPages changes nothing
+        # slots first, the requests' lengths only once the step is launched (the reference commits after it has
+        # submitted the work, runtime/execution.py:125-126): a step that fails on the way (a shape that a kernel
+        # refuses, no memory for a buffer) leaves every request where it stood, and can be tried again
+        done = self.cache.append_many([(e.request, len(e.tokens)) for e in entries], commit=False)  # OutOfPages changes nothing
+        try:
+            if self.execution == "graph":
+                logits = self._run_program(self._program_key(entries, done), entries, done)
+            else:
+                ctx = self._context(entries, done)
+                logits = self._forward(ctx, any(e.pending for e in entries))
+        except BaseException:
+            self.cache.abandon(done)
+            raise
+        self.cache.commit(done)
         self.steps += 1
-        if self.execution == "graph":
-            return self._run_program(self._program_key(entries, done), entries, done)
-        ctx = self._context(entries, done)
-        logits = self._forward(ctx, any(e.pending for e in entries))
         if logits is None:
             return torch.empty((0, self.model.vocab_size), dtype=torch.float32, device=self.device)
         return logits
@@ -195,16 +204,22 @@ class ModelRunner:
 
     _FIXED = 10   # arrays of the metadata before the cache groups'
 
-    def _layout(self, T, S, R):
+    def _width(self, context):
+        """Block-table entries a step carries per request: what its longest context needs, in steps of 16 entries,
+        not what the context limit would need (at a limit of 128k that would be megabytes a step)."""
+        need = -(-int(context) // self.page_size)
+        return min(self.table_width, -(-need // 16) * 16)
+
+    def _layout(self, T, S, R, W):
         """Offsets of the packed int32 metadata: tokens, positions, seg_of_row, seg_start, seg_first_pos,
         state_slots, logit_rows, token_source, logit_slots, single_rows, then per group slots and tables, then one
         attention task list per known tiling (its length is the most tiles that T rows in S segments can make)."""
-        W, G = self.table_width, len(self.cache.groups)
+        G = len(self.cache.groups)
         sizes = [T, T, T, S + 1, S, S, R, T, R, S] + [T, S * W] * G + [4 * (-(-T // r) + S) for r in self.task_tilings]
         return np.concatenate(([0], np.cumsum(sizes))).astype(np.int64)
 
-    def _table_rows(self, g, done):
-        """int32 [len(done), W]: the block tables of the step's requests in group g.  A host copy of every
+    def _table_rows(self, g, done, W):
+        """int32 [len(done), W]: the first W entries of the block tables of the step's requests in group g.  A host copy of every
         live request's table is kept by state slot and rewritten only when the table has changed (a new
         page, a page the window has passed, a copy-on-write), so a step costs one gather."""
         group = self.cache.groups[g]
@@ -216,7 +231,7 @@ class ModelRunner:
                 mirror[d.state_slot, :len(table)] = table
                 mirror[d.state_slot, len(table):] = -1
                 stamps[d.state_slot] = stamp
-        return mirror[[d.state_slot for d in done]]
+        return mirror[[d.state_slot for d in done], :W]
 
     def _single_segments(self, done):
         """How many one-token segments of a mixed step get an attention launch of their own: all of them, if
@@ -226,7 +241,7 @@ class ModelRunner:
             return 0
         return len(singles)
 
-    def _context(self, entries, done, pad=None, device_buffer=None, n_single=None):
+    def _context(self, entries, done, pad=None, device_buffer=None, n_single=None, context=None):
         """Build the step's metadata on the host, upload it in one copy and wrap it.
         `pad` = (T, S, R) pads the batch with inert rows (for captured programs):
         token 0 at position 0, no segment, no cache slot."""
@@ -235,11 +250,13 @@ class ModelRunner:
         n_rows, n_seg = sum(counts), len(entries)
         n_want = sum(len(e.want) for e in entries)
         T, S, R = pad if pad is not None else (n_rows, n_seg, n_want)
-        W, G, F = self.table_width, len(self.cache.groups), self._FIXED
-        layout = (T, S, R, tuple(self.task_tilings))
+        # the longest context of the step (a captured program brings the bound of its bucket) sizes the block tables
+        longest = max(s + c for s, c in zip(starts, counts))
+        W, G, F = self._width(longest if context is None else context), len(self.cache.groups), self._FIXED
+        layout = (T, S, R, W, tuple(self.task_tilings))
         offsets = self._layouts.get(layout)
         if offsets is None:
-            offsets = self._layouts[layout] = [int(x) for x in self._layout(T, S, R)]
+            offsets = self._layouts[layout] = [int(x) for x in self._layout(T, S, R, W)]
         total = offsets[-1]
         host = self._stage(total)
         arr = host.numpy()
@@ -292,7 +309,7 @@ class ModelRunner:
                 slots[:n_rows] = [d.slots[g][0] for d in done]
             else:
                 slots[:n_rows] = np.concatenate([np.asarray(d.slots[g], dtype=np.int32) for d in done])
-            tables[:n_seg] = self._table_rows(g, done)
+            tables[:n_seg] = self._table_rows(g, done, W)
             if pad is not None:
                 slots[n_rows:] = -1
                 tables[n_seg:] = -1
@@ -327,7 +344,7 @@ class ModelRunner:
         ctx.tasks = {r: view(F + 2 * G + i, (-1, 4)) for i, r in enumerate(tilings)}
         self._last_wanted = ([entries[s].request for s in wanted_seg], wanted_slots, view(8)[:n_want])
         ctx.segments = [(d.request, d.start, d.count) for d in done]
-        ctx.max_context = ctx.span_hint = max(s + c for s, c in zip(starts, counts))
+        ctx.max_context = ctx.span_hint = longest
         ctx.decode_only = decode_only
         return ctx
 
@@ -385,9 +402,9 @@ class ModelRunner:
         if program["tilings"] != self.task_tilings:
             # a mixer asked for a task list that the metadata did not hold yet: lay it out again
             torch.cuda.synchronize()
-            program.update(meta=torch.zeros(int(self._layout(T, S, R)[-1]), dtype=torch.int32, device=self.device),
+            program.update(meta=torch.zeros(int(self._layout(T, S, R, self._width(context))[-1]), dtype=torch.int32, device=self.device),
                            graph=None, runs=0, tilings=list(self.task_tilings))
-        ctx = self._context(entries, done, pad=(T, S, R), device_buffer=program["meta"], n_single=n_single)
+        ctx = self._context(entries, done, pad=(T, S, R), device_buffer=program["meta"], n_single=n_single, context=context)
         ctx.owner = key
         ctx.span_hint = context   # launch shapes inside a captured program depend on the key only
         ctx.decode_only = decode_only

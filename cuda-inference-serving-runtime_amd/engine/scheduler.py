@@ -21,7 +21,7 @@ there, and the host prepares step N+1 while the GPU runs step N.  The tokens
 are the same; a request that ends on an end-of-sequence token is found out one
 step late, and the token it decoded meanwhile is dropped.
 """
-import math
+import enum
 import time
 from collections import deque
 from dataclasses import dataclass, field
@@ -32,32 +32,98 @@ from .runner import StepEntry
 POLICIES = ("serial", "chunked", "decode_first")
 
 
+class Phase(str, enum.Enum):
+    """Where a request stands.  A member compares equal to its name in lower case ("finished")."""
+    WAITING = "waiting"        # submitted, holds nothing
+    PREFILL = "prefill"        # admitted, its prompt is being cached
+    DECODE = "decode"          # one token a step
+    DRAINING = "draining"      # overlapped ticks: its last token is picked on the device and not read yet
+    FINISHED = "finished"
+    CANCELLED = "cancelled"
+
+    def __str__(self):
+        return self.value
+
+    @property
+    def over(self):
+        return self in (Phase.FINISHED, Phase.CANCELLED)
+
+
 @dataclass
 class Request:
+    """A request and its progress (the fields of the reference's Request, runtime/engine.py:13-26, and the
+    sampling parameters)."""
     key: str
     prompt: list
     max_new_tokens: int = 16
-    eos_token_id: Optional[int] = None
+    eos_token_id: Optional[int] = None     # one id, or a collection of them
     arrival_s: float = 0.0
     temperature: float = 0.0
     seed: int = 0
     generated: list = field(default_factory=list)
-    cursor: int = 0
+    cursor: int = 0          # prompt tokens cached so far
     launched: int = 0        # tokens picked for it so far, read by the host or not (overlapped ticks)
-    status: str = "waiting"  # waiting, prefill, decode, draining (its last token is picked, not read), finished, cancelled
+    status: Phase = Phase.WAITING
     submitted_at: float = 0.0
     first_token_at: Optional[float] = None
     token_times: list = field(default_factory=list)
     finished_at: Optional[float] = None
 
+    @property
+    def cached_tokens(self):
+        """Tokens that will ever sit in the cache: the last generated token is never fed back."""
+        return len(self.prompt) + max(0, self.max_new_tokens - 1)
+
+    def ends_with(self, token):
+        eos = self.eos_token_id
+        if eos is None:
+            return False
+        return token in eos if isinstance(eos, (list, tuple, set, frozenset)) else token == eos
+
+    def take(self, token, when):
+        """Record a generated token; True if it is the request's last."""
+        self.generated.append(int(token))
+        self.token_times.append(when)
+        if self.first_token_at is None:
+            self.first_token_at = when
+        return len(self.generated) >= self.max_new_tokens or self.ends_with(token)
+
+
+class PageLedger:
+    """Pages promised to admitted requests, group by group of the cache.
+
+    A request is admitted only if every group can promise it the most pages it will ever hold there (all its
+    tokens in a group that keeps every key; a window and a portion in a group that keeps a window), so a step of
+    admitted requests cannot run out of pages.  The numbers come from the cache manager."""
+
+    def __init__(self, cache, portion):
+        self.cache, self.portion, self.promised = cache, portion, {}
+
+    def need(self, tokens):
+        return self.cache.most_pages_held(tokens, self.portion)
+
+    def ever_fits(self, need):
+        return all(n <= cap for n, cap in zip(need, self.cache.capacity()))
+
+    def fits_now(self, need):
+        taken = [sum(p[g] for p in self.promised.values()) for g in range(len(need))]
+        return all(n <= cap - t for n, cap, t in zip(need, self.cache.capacity(), taken))
+
+    def promise(self, key, need):
+        self.promised[key] = list(need)
+
+    def withdraw(self, key):
+        return self.promised.pop(key, None) is not None
+
 
 class Engine:
     def __init__(self, runner, max_active=8, token_budget=32, prefill_chunk=8, policy="chunked", sampler=None,
                  overlap=False):
-        if min(max_active, token_budget, prefill_chunk) <= 0:
-            raise ValueError("invalid scheduler limits")
+        for name, value in (("max_active", max_active), ("token_budget", token_budget), ("prefill_chunk", prefill_chunk)):
+            if value <= 0:
+                raise ValueError(f"{name} must be positive, not {value}")
         if policy not in POLICIES:
-            raise ValueError(f"invalid policy {policy!r}; one of {POLICIES}")
+            raise ValueError(f"policy {policy!r} is none of {POLICIES}")
         self.runner = runner
         self.max_active = 1 if policy == "serial" else min(max_active, runner.max_requests)
         self.token_budget, self.prefill_chunk, self.policy = token_budget, prefill_chunk, policy
@@ -65,70 +131,80 @@ class Engine:
             from ..sampling import Sampler
             sampler = Sampler()
         self.sampler = sampler
-        self.waiting, self.active, self.requests, self.reserved = deque(), [], {}, {}
+        self.ledger = PageLedger(runner.cache, min(prefill_chunk, token_budget))
+        self.waiting, self.active, self.requests = deque(), [], {}
         self.trace, self.start, self.rotation = [], time.perf_counter(), 0
         self.overlap, self.inflight = overlap, None
 
-    # -- page accounting ----------------------------------------------------------
-    def _pool_pages(self):
-        return min(g.pool.n_pages for g in self.runner.cache.groups) if self.runner.cache.groups else 1 << 30
+    @property
+    def reserved(self):
+        """{request key: pages promised to it, summed over the cache groups}."""
+        return {key: sum(need) for key, need in self.ledger.promised.items()}
 
-    def _pages_for(self, r):
-        # the last generated token is never fed back, so it needs no cache entry
-        return math.ceil((len(r.prompt) + max(0, r.max_new_tokens - 1)) / self.runner.page_size)
-
-    # -- requests -------------------------------------------------------------------
-    def submit(self, request):
-        r = request
+    # -- requests come and go -------------------------------------------------------------
+    def _refusal(self, r):
+        """Why `r` cannot be taken, or None (what the reference checks at submit, runtime/engine.py:38-50)."""
         if r.key in self.requests:
-            raise ValueError("duplicate request ID")
-        if not r.prompt or r.max_new_tokens < 0 or r.arrival_s < 0:
-            raise ValueError("invalid request")
-        if r.status != "waiting" or r.cursor or r.generated:
-            raise ValueError("request already used")
-        if any((not 0 <= t < self.runner.model.vocab_size) for t in r.prompt):
-            raise ValueError("invalid prompt token")
-        if len(r.prompt) + max(0, r.max_new_tokens - 1) > self.runner.max_context:
-            raise ValueError("request exceeds context limit")
-        if self._pages_for(r) > self._pool_pages():
-            raise ValueError("request cannot fit in page pool")
-        r.submitted_at = self.start + r.arrival_s
-        self.requests[r.key] = r
-        self.waiting.append(r)
+            return f"the key {r.key!r} is already in use"
+        if r.status is not Phase.WAITING or r.cursor or r.launched or r.generated:
+            return f"request {r.key!r} has run before: submit a fresh Request"
+        if len(r.prompt) == 0:
+            return f"request {r.key!r} has an empty prompt"
+        if r.max_new_tokens < 0 or r.arrival_s < 0:
+            return f"request {r.key!r}: max_new_tokens and arrival_s cannot be negative"
+        vocab = self.runner.model.vocab_size
+        stray = next((t for t in r.prompt if not 0 <= t < vocab), None)
+        if stray is not None:
+            return f"request {r.key!r}: token {stray} is outside the vocabulary of {vocab}"
+        if r.cached_tokens > self.runner.max_context:
+            return f"request {r.key!r} would cache {r.cached_tokens} tokens, the context limit is {self.runner.max_context}"
+        need = self.ledger.need(r.cached_tokens)
+        if not self.ledger.ever_fits(need):
+            return f"request {r.key!r} needs {need} pages, the pools hold {self.runner.cache.capacity()}: it can never run"
+        return None
 
-    def _finish(self, r, status="finished"):
-        if r.key in self.reserved:
+    def submit(self, request):
+        reason = self._refusal(request)
+        if reason is not None:
+            raise ValueError(reason)
+        request.submitted_at = self.start + request.arrival_s
+        self.requests[request.key] = request
+        self.waiting.append(request)
+
+    def _close(self, r, phase=Phase.FINISHED):
+        """End a request: whatever it holds (cache pages, state slot, promised pages) goes back."""
+        if self.ledger.withdraw(r.key):
             self.runner.release(r.key)
-            del self.reserved[r.key]
             self.active.remove(r)
-        r.status, r.finished_at = status, time.perf_counter()
+        r.status, r.finished_at = phase, time.perf_counter()
 
     def cancel(self, key):
         r = self.requests[key]
-        if r.status in ("finished", "cancelled"):
+        if r.status.over:
             return
-        if r in self.waiting:
+        if r.status is Phase.WAITING:
             self.waiting.remove(r)
-        self._finish(r, "cancelled")
+        self._close(r, Phase.CANCELLED)
 
     def _admit(self):
-        available = self._pool_pages() - sum(self.reserved.values())
-        for r in list(self.waiting):  # scan all: a large request does not block smaller ones
+        """Take waiting requests in while there is room: the whole queue is looked at, so a request that does
+        not fit now does not hold up a later one that does (runtime/engine.py:65-76)."""
+        now = time.perf_counter()
+        for r in tuple(self.waiting):
             if len(self.active) >= self.max_active:
-                break
-            if time.perf_counter() < r.submitted_at:
-                continue
-            pages = self._pages_for(r)
-            if pages > available:
+                return
+            if r.submitted_at > now:
+                continue                      # not arrived yet
+            need = self.ledger.need(r.cached_tokens)
+            if not self.ledger.fits_now(need):
                 continue
             self.waiting.remove(r)
             if r.max_new_tokens == 0:
-                self._finish(r)
+                self._close(r)                # nothing to generate: it never touches the cache
                 continue
             self.runner.create(r.key)
-            self.reserved[r.key] = pages
-            available -= pages
-            r.status = "prefill"
+            self.ledger.promise(r.key, need)
+            r.status = Phase.PREFILL
             self.active.append(r)
 
     # -- one tick = one step --------------------------------------------------------
@@ -137,130 +213,112 @@ class Engine:
         order = self.active[self.rotation:] + self.active[:self.rotation]
         self.rotation = (self.rotation + 1) % max(1, len(self.active))
         if self.policy == "decode_first":
-            order.sort(key=lambda r: r.status != "decode")
+            order.sort(key=lambda r: r.status is not Phase.DECODE)
         remaining, plan = self.token_budget, []
         for r in order:
             if remaining == 0:
                 break
-            if r.status == "draining":
+            if r.status is Phase.DRAINING:
                 continue
-            n = 1 if r.status == "decode" else min(self.prefill_chunk, len(r.prompt) - r.cursor, remaining)
+            n = 1 if r.status is Phase.DECODE else min(self.prefill_chunk, len(r.prompt) - r.cursor, remaining)
             plan.append((r, n))
             remaining -= n
         return plan
 
-    def tick(self):
-        if self.overlap:
-            return self._tick_overlapped()
-        self._admit()
-        if not self.active:
-            return bool(self.waiting)
-        now = time.perf_counter()
-        plan = self.plan()
-        entries, sampled = [], []
+    def _entries(self, plan):
+        """The step's entries, and the requests whose logits are wanted (a token is picked for them)."""
+        entries, picking = [], []
         for r, n in plan:
-            if r.status == "decode":
-                entries.append(StepEntry(r.key, [r.generated[-1]], [0]))
-                sampled.append(r)
+            if r.status is Phase.DECODE:
+                on_device = r.launched > len(r.generated)     # its last token is picked but not read yet
+                entries.append(StepEntry(r.key, [0] if on_device else [r.generated[-1]], [0], pending=on_device))
+                picking.append(r)
             else:
+                portion = r.prompt[r.cursor:r.cursor + n]
                 last = r.cursor + n == len(r.prompt)
-                entries.append(StepEntry(r.key, r.prompt[r.cursor:r.cursor + n], [n - 1] if last else []))
+                entries.append(StepEntry(r.key, portion, [n - 1] if last else []))
                 if last:
-                    sampled.append(r)
-        logits = self.runner.step(entries)
-        choices = self.sampler.pick(logits, [(r.temperature, r.seed, len(r.generated)) for r in sampled])
-        completed = time.perf_counter()
-        picked = dict(zip((r.key for r in sampled), choices))
-        for r, n in plan:
-            if r.status == "prefill":
-                r.cursor += n
-                if r.cursor < len(r.prompt):
-                    continue
-                r.status = "decode"
-            token = int(picked[r.key])
-            r.generated.append(token)
-            r.token_times.append(completed)
-            if r.first_token_at is None:
-                r.first_token_at = completed
-            if len(r.generated) >= r.max_new_tokens or self._is_eos(r, token):
-                self._finish(r)
-        cache = self.runner.cache
-        self.trace.append({"elapsed_s": time.perf_counter() - self.start, "step_s": time.perf_counter() - now,
-                           "processed_tokens": sum(n for _, n in plan), "active": len(self.active),
-                           "resident_pages": sum(g.pool.used for g in cache.groups)})
-        return bool(self.active or self.waiting)
+                    picking.append(r)
+        return entries, picking
 
-    def _tick_overlapped(self):
+    @staticmethod
+    def _fed(r, n):
+        """Account for n tokens of `r` having been stepped; True if the step picks a token for it."""
+        if r.status is Phase.PREFILL:
+            r.cursor += n
+            if r.cursor < len(r.prompt):
+                return False
+            r.status = Phase.DECODE
+        return True
+
+    def _record(self, began, plan):
+        now = time.perf_counter()
+        self.trace.append({"elapsed_s": now - self.start, "step_s": now - began,
+                           "processed_tokens": sum(n for _, n in plan), "active": len(self.active),
+                           "resident_pages": sum(g.pool.used for g in self.runner.cache.groups)})
+
+    def tick(self):
+        """Admit, run one step, hand out its tokens.  False when nothing is left to do."""
         self._admit()
         if not self.active and self.inflight is None:
             return bool(self.waiting)
-        now = time.perf_counter()
+        began = time.perf_counter()
         plan = self.plan()
-        entries, sampled = [], []
-        for r, n in plan:
-            if r.status == "decode":
-                if r.launched > len(r.generated):     # its last token is still only on the device
-                    entries.append(StepEntry(r.key, [0], [0], pending=True))
-                else:
-                    entries.append(StepEntry(r.key, [r.generated[-1]], [0]))
-                sampled.append(r)
-            else:
-                last = r.cursor + n == len(r.prompt)
-                entries.append(StepEntry(r.key, r.prompt[r.cursor:r.cursor + n], [n - 1] if last else []))
-                if last:
-                    sampled.append(r)
+        entries, picking = self._entries(plan)
+        if self.overlap:
+            self._step_ahead(plan, entries, picking)
+        else:
+            logits = self.runner.step(entries)
+            tokens = dict(zip((r.key for r in picking),
+                              self.sampler.pick(logits, [(r.temperature, r.seed, len(r.generated)) for r in picking])))
+            when = time.perf_counter()
+            for r, n in plan:
+                if self._fed(r, n) and r.take(tokens[r.key], when):
+                    self._close(r)
+        self._record(began, plan)
+        return bool(self.active or self.waiting or self.inflight)
+
+    def _step_ahead(self, plan, entries, picking):
+        """Overlapped ticks: launch this step, then read the tokens of the step before.  What is known without
+        the token is settled at launch (the prompt cursor, the count of tokens); what needs the token (an
+        end-of-sequence) one step late."""
         launched = None
         if entries:
             logits = self.runner.step(entries)
-            if sampled:
-                picked = self.runner.pick(self.sampler, logits, [(r.temperature, r.seed, r.launched) for r in sampled])
-                launched = (picked, sampled)
+            if picking:
+                picked = self.runner.pick(self.sampler, logits, [(r.temperature, r.seed, r.launched) for r in picking])
+                launched = (picked, picking)
             for r, n in plan:
-                if r.status == "prefill":
-                    r.cursor += n
-                    if r.cursor < len(r.prompt):
-                        continue
-                    r.status = "decode"
-                r.launched += 1
-                if r.launched >= r.max_new_tokens:
-                    r.status = "draining"     # nothing more to decode; it ends when this token is read
+                if self._fed(r, n):
+                    r.launched += 1
+                    if r.launched >= r.max_new_tokens:
+                        r.status = Phase.DRAINING     # nothing more to decode; it ends when this token is read
         previous, self.inflight = self.inflight, launched
-        if previous is not None:
-            picked, requests = previous
-            tokens = picked.tokens()
-            completed = time.perf_counter()
-            for r, token in zip(requests, tokens):
-                if r.status in ("finished", "cancelled"):
-                    continue                  # ended by an earlier token, or cancelled: this one is dropped
-                r.generated.append(int(token))
-                r.token_times.append(completed)
-                if r.first_token_at is None:
-                    r.first_token_at = completed
-                if len(r.generated) >= r.max_new_tokens or self._is_eos(r, token):
-                    self._finish(r)
-        cache = self.runner.cache
-        self.trace.append({"elapsed_s": time.perf_counter() - self.start, "step_s": time.perf_counter() - now,
-                           "processed_tokens": sum(n for _, n in plan), "active": len(self.active),
-                           "resident_pages": sum(g.pool.used for g in cache.groups)})
-        return bool(self.active or self.waiting or self.inflight)
-
-    @staticmethod
-    def _is_eos(r, token):
-        eos = r.eos_token_id
-        return eos is not None and (token in eos if isinstance(eos, (list, tuple, set, frozenset)) else token == eos)
+        if previous is None:
+            return
+        picked, requests = previous
+        tokens = picked.tokens()
+        when = time.perf_counter()
+        for r, token in zip(requests, tokens):
+            if r.status.over:
+                continue                  # ended by an earlier token, or cancelled: this one is dropped
+            if r.take(token, when):
+                self._close(r)
 
     def run(self):
+        """Tick until every request is over; sleeps (at most 10 ms at a time) while only future arrivals wait."""
         while self.tick():
             if not self.active and self.waiting:
-                delay = min(r.submitted_at for r in self.waiting) - time.perf_counter()
-                if delay > 0:
-                    time.sleep(min(delay, 0.01))
+                pause = min(r.submitted_at for r in self.waiting) - time.perf_counter()
+                if pause > 0:
+                    time.sleep(min(pause, 0.01))
         return list(self.requests.values())
 
     # -- conveniences ---------------------------------------------------------------
     @classmethod
-    def from_folder(cls, folder, dtype="bfloat16", pages=128, page_size=16, execution="eager", device="cuda:0", **limits):
-        """An engine for the model in `folder` (config.json + safetensors).  pages None (or 0): as many as fit
+    def from_folder(cls, folder, dtype="bfloat16", pages=128, page_size=16, execution="graph", device="cuda:0", **limits):
+        """An engine for the model in `folder` (config.json + safetensors).  Steps run as captured programs unless
+        execution="eager" (kernels launched one by one).  pages None (or 0): as many as fit
         into four fifths of the GPU memory that is free once the weights are loaded, at most what the
         requests can address."""
         import torch
@@ -272,9 +330,11 @@ class Engine:
         if not pages:
             free, _ = torch.cuda.mem_get_info(torch.device(device))
             addressable = max_requests * -(-model.max_positions // page_size)
-            # (the attention kernels address a site's keys with 32-bit byte offsets: fewer than 2^31 elements)
-            widest = max(need.kv_heads * need.head_dim for need in model.cache_needs().values() if need is not None)
-            addressable = min(addressable, (2 ** 31 - 1) // (widest * page_size))
+            # (the attention kernels address a site's keys with 32-bit byte offsets: fewer than 2^31 elements;
+            # a model whose mixers keep no keys has nothing to size)
+            widths = [need.kv_heads * need.head_dim for need in model.cache_needs().values() if need is not None]
+            if widths:
+                addressable = min(addressable, (2 ** 31 - 1) // (max(widths) * page_size))
             pages = pages_that_fit(model.cache_needs(), page_size, 2 if dtype == "bfloat16" else 4, free, most=addressable)
         runner = ModelRunner(model, n_pages=pages, page_size=page_size, max_requests=max_requests, device=device,
                              execution=execution)

@@ -13,10 +13,11 @@ def build_llama(config):
     c = config
     embedding = TokenEmbedding("model.embed_tokens", c.vocab_size, c.hidden_size)
     layers = []
+    # one position part for the whole model: every layer turns by the same angles, so the tables exist once
+    position = make_part("position", "rotary", head_dim=c.head_dim, theta=c.rope_theta,
+                         max_positions=c.max_position_embeddings)
     for i in range(c.num_hidden_layers):
         p = f"model.layers.{i}"
-        position = make_part("position", "rotary", head_dim=c.head_dim, theta=c.rope_theta,
-                             max_positions=c.max_position_embeddings)
         mixer = make_part("mixer", "attention", name=p + ".self_attn", hidden=c.hidden_size,
                           heads=c.num_attention_heads, kv_heads=c.num_key_value_heads, head_dim=c.head_dim,
                           position=position)
@@ -29,7 +30,7 @@ def build_llama(config):
             ffn=ffn))
     final_norm = make_part("norm", "rmsnorm", name="model.norm", dim=c.hidden_size, eps=c.rms_norm_eps)
     head = LMHead("lm_head", c.vocab_size, c.hidden_size, tied_to=embedding if c.tie_word_embeddings else None)
-    return Model(c, embedding, layers, final_norm, head)
+    return Model(c, embedding, layers, final_norm, head, max_positions=c.max_position_embeddings, vocab_size=c.vocab_size)
 
 
 register_architecture(["LlamaForCausalLM", "llama"], LlamaConfig, build_llama)

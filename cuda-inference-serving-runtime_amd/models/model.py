@@ -19,8 +19,14 @@ class ScheduleEntry:
 
 
 class Model:
-    def __init__(self, config, embedding, layers, final_norm, head, schedule=None):
+    def __init__(self, config, embedding, layers, final_norm, head, schedule=None, max_positions=None, vocab_size=None):
+        """`max_positions` (the context limit) and `vocab_size`: given by the builder, or read from the
+        configuration's fields `max_position_embeddings` and `vocab_size` if it has them under these names."""
         self.config = config
+        self._max_positions = max_positions if max_positions is not None else getattr(config, "max_position_embeddings", None)
+        self._vocab_size = vocab_size if vocab_size is not None else getattr(config, "vocab_size", None)
+        if self._max_positions is None or self._vocab_size is None:
+            raise ValueError("a model needs max_positions and vocab_size (arguments, or fields of its configuration)")
         self.embedding, self.layers, self.final_norm, self.head = embedding, list(layers), final_norm, head
         self.schedule = list(schedule) if schedule is not None else [ScheduleEntry(i) for i in range(len(self.layers))]
         for index, entry in enumerate(self.schedule):
@@ -83,11 +89,11 @@ class Model:
 
     @property
     def max_positions(self):
-        return self.config.max_position_embeddings
+        return self._max_positions
 
     @property
     def vocab_size(self):
-        return self.config.vocab_size
+        return self._vocab_size
 
     # -- the forward pass over one step's rows ------------------------------------
     def forward(self, ctx):

@@ -17,7 +17,6 @@ import torch
 from ..cache.pages import KVNeed
 from ..kernels import ops
 from .base import Mixer, TensorSpec, matrix_operand, register_part
-from .norm import RMSNorm
 
 
 class PagedAttention(Mixer):
@@ -56,7 +55,7 @@ class PagedAttention(Mixer):
         return ops.qkv_rope_fused_ok(a, self.w_in, self.head_dim, cos, normed)
 
     def fuses_norm(self, norm, residual, ctx):
-        return isinstance(norm, RMSNorm) and self._fused_projection_ok(residual, True)
+        return getattr(norm, "fusable_as", None) == "rms" and self._fused_projection_ok(residual, True)
 
     def forward(self, h, residual, ctx, site, norm=None):
         T = residual.shape[0]

@@ -14,7 +14,9 @@ Mixers and feed-forwards add their result to the float residual stream
 themselves (their last matrix product does it in its epilogue) and return it.
 A mixer or feed-forward may take over the norm in front of it: if its
 `fuses_norm(norm, residual, ctx)` says so for a step, the block passes h=None
-and the norm part, and the part applies the norm inside its first kernel.
+and the norm part, and the part applies the norm inside its first kernel.  Which
+norms can be taken over is a capability the norm states (`fusable_as`: "rms"
+with `weight` and `eps`), not a class.
 A mixer states what it keeps between steps: `cache_need()` (pages of keys and
 values) and/or `state_need()` (a fixed-size state per request), or neither.
 """

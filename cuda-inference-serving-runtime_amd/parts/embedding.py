@@ -8,7 +8,6 @@ import torch
 
 from ..kernels import ops
 from .base import Part, TensorSpec, matrix_operand
-from .norm import RMSNorm
 
 
 class TokenEmbedding(Part):
@@ -39,7 +38,7 @@ class LMHead(Part):
         self.weight = self.tied_to.weight if self.tied_to is not None else matrix_operand(tensors[self.name + ".weight"], dtype)
 
     def fuses_norm(self, norm, residual, rows):
-        return isinstance(norm, RMSNorm) and ops.fused_norm_ok(residual, self.weight, rows.shape[0])
+        return getattr(norm, "fusable_as", None) == "rms" and ops.fused_norm_ok(residual, self.weight, rows.shape[0])
 
     def forward(self, h, ctx, norm=None, residual=None):
         """Logits of the normed rows h; or, with `norm`, of RMSNorm(residual[ctx.logit_rows]) in one kernel."""

@@ -5,7 +5,6 @@ import torch
 
 from ..kernels import ops
 from .base import FeedForward, TensorSpec, matrix_operand, register_part
-from .norm import RMSNorm
 
 
 class GatedMLP(FeedForward):
@@ -27,7 +26,7 @@ class GatedMLP(FeedForward):
         self.w_down = matrix_operand(tensors[f"{self.name}.down_proj.weight"], dtype)
 
     def fuses_norm(self, norm, residual, ctx):
-        return isinstance(norm, RMSNorm) and ops.fused_norm_ok(residual, self.w_gate_up, residual.shape[0])
+        return getattr(norm, "fusable_as", None) == "rms" and ops.fused_norm_ok(residual, self.w_gate_up, residual.shape[0])
 
     def forward(self, h, residual, ctx, norm=None):
         T = residual.shape[0]

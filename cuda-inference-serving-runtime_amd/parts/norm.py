@@ -7,6 +7,9 @@ from .base import Part, TensorSpec, register_part
 
 
 class RMSNorm(Part):
+    # What a kernel that takes over this norm must compute: "rms" = x * rsqrt(mean(x^2) + eps) * weight, with the
+    # attributes `weight` (float [dim]) and `eps`.  A mixer, feed-forward or head fuses any norm that says so.
+    fusable_as = "rms"
     adds_partials = True    # forward adds the partial sums of a product left unfinished before it (ctx.add_product)
 
     def __init__(self, name, dim, eps):

@@ -26,6 +26,8 @@ class RotaryEmbedding(Part):
         return np.arange(self.max_positions, dtype=np.float64)[:, None] * inv_freq[None, :]
 
     def prepare(self, device, dtype):
+        if self._tables is not None and self._tables[0].device == torch.device(device):
+            return                      # one part may serve many layers: its tables are built once
         a = self.angles()
         self._tables = (torch.from_numpy(np.cos(a).astype(np.float32)).to(device).contiguous(),
                         torch.from_numpy(np.sin(a).astype(np.float32)).to(device).contiguous())
@@ -42,6 +44,8 @@ class NoPosition(Part):
         self._tables = None
 
     def prepare(self, device, dtype):
+        if self._tables is not None and self._tables[0].device == torch.device(device):
+            return
         self._tables = (torch.ones(self.max_positions, 1, dtype=torch.float32, device=device),
                         torch.zeros(self.max_positions, 1, dtype=torch.float32, device=device))
 

@@ -18,26 +18,27 @@ from .safetensors_io import write_safetensors
 STD = 0.02
 
 
-def random_tensors(specs, seed, dtype=torch.bfloat16):
+def random_tensors(specs, seed, dtype=torch.bfloat16, std=STD):
+    """`std`: the spread of the normal draws (0.02 unless a caller wants layers that outweigh the embedding)."""
     rng = np.random.default_rng(seed)
     out = {}
     for spec in sorted(specs, key=lambda s: s.name):
         if spec.integer:
             raise ValueError(f"{spec.name}: integer tables have no random initialisation")
-        values = rng.standard_normal(size=spec.shape, dtype=np.float32) * np.float32(STD)
+        values = rng.standard_normal(size=spec.shape, dtype=np.float32) * np.float32(std)
         if spec.init == "one_plus_normal":
             values = values + np.float32(1.0)
         out[spec.name] = torch.from_numpy(values).to(dtype)
     return out
 
 
-def write_model_folder(folder, config_dict, specs, seed, dtype=torch.bfloat16):
+def write_model_folder(folder, config_dict, specs, seed, dtype=torch.bfloat16, std=STD):
     """config_dict is what goes into config.json; specs are the model's tensor specs."""
     folder = Path(folder)
     folder.mkdir(parents=True, exist_ok=True)
     raw = dict(config_dict)
     raw["torch_dtype"] = {torch.bfloat16: "bfloat16", torch.float32: "float32"}[dtype]
     (folder / "config.json").write_text(json.dumps(raw, indent=2) + "\n")
-    write_safetensors(folder / "model.safetensors", random_tensors(specs, seed, dtype),
+    write_safetensors(folder / "model.safetensors", random_tensors(specs, seed, dtype, std),
                       metadata={"format": "pt", "seed": seed})
     return folder

@@ -156,6 +156,30 @@ def test_window_step_is_atomic_whatever_the_order_of_its_requests():
     m.check()
 
 
+@pytest.mark.parametrize("fast", [True, False])
+def test_slots_without_commit_can_be_abandoned_or_committed(fast):
+    """A step places its slots first and counts its tokens only once it is launched; a step that is never
+    launched gives its pages back and leaves every request where it stood."""
+    m = manager(pages=6, page_size=4, sites=1)
+    m.fast_decode = fast
+    m.create("a"); m.create("b")
+    m.append_many([("a", 4), ("b", 3)])
+    before = ({r: m.length(r) for r in "ab"}, {r: list(m.table(0, r)) for r in "ab"}, m.free_pages())
+    for items in ([("a", 1), ("b", 1)], [("a", 9), ("b", 2)]):
+        done = m.append_many(items, commit=False)
+        assert (m.length("a"), m.length("b")) == (4, 3)          # not counted yet
+        assert [d.start for d in done] == [4, 3]
+        m.abandon(done)
+        assert before == ({r: m.length(r) for r in "ab"}, {r: list(m.table(0, r)) for r in "ab"}, m.free_pages())
+        m.check()
+    done = m.append_many([("a", 1), ("b", 1)], commit=False)
+    m.commit(done)
+    assert (m.length("a"), m.length("b")) == (5, 4) and len(m.table(0, "a")) == 2
+    m.check()
+    with pytest.raises(RuntimeError):
+        m.commit(done)                                            # the same step twice
+
+
 def test_window_group_never_needs_more_than_window_plus_portion():
     m = manager(pages=4, page_size=4, sites=0, window=8)
     m.create("a")

@@ -17,33 +17,37 @@ pytestmark = pytest.mark.gpu
 
 
 def plain_greedy_margin(cfg, w, prompt, steps):
-    """Greedy tokens and the smallest top-2 logit gap met on the way."""
-    tokens, out, margin = list(prompt), [], np.inf
+    """Greedy tokens, the gap between the two best logits at every step and those two tokens."""
+    tokens, out, gaps, top2 = list(prompt), [], [], []
     for _ in range(steps):
         logits = P.forward(cfg, w, tokens)[-1]
-        top = np.sort(logits)[-2:]
-        margin = min(margin, top[1] - top[0])
+        order = np.argsort(logits)[-2:]
+        gaps.append(float(logits[order[1]] - logits[order[0]]))
+        top2.append({int(order[0]), int(order[1])})
         out.append(int(np.argmax(logits)))
         tokens.append(out[-1])
-    return out, margin
+    return out, gaps, top2
 
 
+@pytest.mark.parametrize("execution", ["eager", "graph"])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["a", "b"])
-def test_greedy_generation_matches_plain(folders, name, dtype):
+def test_greedy_generation_matches_plain(folders, name, dtype, execution):
     from runtime.engine.scheduler import Engine
     cfg, w = P.read_folder(folders[name])
     V = TINY[name]["vocab_size"]
     prompts = [random_tokens(20 + i, n, V) for i, n in enumerate([5, 11, 17])]
     want = [plain_greedy_margin(cfg, w, p, 8) for p in prompts]
-    engine = Engine.from_folder(folders[name], dtype=dtype, pages=32, page_size=16, token_budget=16, prefill_chunk=7)
+    engine = Engine.from_folder(folders[name], dtype=dtype, pages=32, page_size=16, token_budget=16, prefill_chunk=7,
+                                execution=execution)
     got = engine.generate(prompts, max_new_tokens=8)
-    for g, (tokens, margin) in zip(got, want):
-        if dtype == "float32" or margin > 0.05:
+    for g, (tokens, gaps, top2) in zip(got, want):
+        if dtype == "float32" or min(gaps) > 0.05:
             assert g == tokens
-        else:   # a near tie may flip in bfloat16: equal up to the first such place
-            n = next((i for i, (x, y) in enumerate(zip(g, tokens)) if x != y), len(tokens))
-            assert n >= 1
+        else:   # a near tie may flip in bfloat16: equal up to the first place whose two best logits are that close
+            first_tie = next(i for i, gap in enumerate(gaps) if gap < 0.05)
+            assert g[:first_tie] == tokens[:first_tie]
+            assert g[first_tie] in top2[first_tie], "a flipped near tie picks the runner-up, nothing else"
     engine.runner.cache.check()
     assert engine.runner.cache.free_pages() == [32]
 
@@ -100,6 +104,69 @@ def test_graph_replays_match_eager_logits(folders):
     graph_runner = runners[1]
     decode_programs = [p for key, p in graph_runner.programs.items() if key[3] and p["graph"] is not None]
     assert len(decode_programs) >= 2 and all(p["runs"] >= 3 for p in decode_programs)
+
+
+@pytest.mark.parametrize("name,dtype", [("c", "bfloat16"), ("a", "float32")])
+def test_evicted_programs_are_built_again_and_stay_right(folders, name, dtype):
+    """More step shapes than the runner keeps captured programs for: the oldest are dropped (their buffers go
+    back) and, when their shape comes again, built, captured and replayed anew.  Every step, before and after, is
+    compared with the plain model."""
+    from runtime.engine import load_model, ModelRunner, StepEntry
+    from conftest import plain_logits, assert_close
+    V = TINY[name]["vocab_size"]
+    model = load_model(folders[name], dtype=dtype)
+    runner = ModelRunner(model, n_pages=80, page_size=8, max_requests=4, execution="graph")
+    seqs = {k: random_tokens(700 + i, 200, V) for i, k in enumerate("uvw")}
+    refs = {k: plain_logits(folders[name], seqs[k]) for k in seqs}
+    fed = {}
+
+    def restart():
+        for k in seqs:
+            if k in runner.cache:
+                runner.release(k)
+            runner.create(k)
+            fed[k] = 0
+
+    def feed(parts, wanted=True):
+        entries, places = [], []
+        for k, n in parts:
+            want = ([0, n - 1] if n > 1 else [0]) if wanted else []
+            entries.append(StepEntry(k, seqs[k][fed[k]:fed[k] + n], want))
+            places += [(k, fed[k] + j) for j in want]
+            fed[k] += n
+        logits = runner.step(entries).float().cpu().numpy()
+        assert logits.shape[0] == len(places)
+        for row, (k, pos) in zip(logits, places):
+            assert_close(row[None], refs[k][pos][None], dtype, f"request {k} position {pos}")
+
+    first = [("u", 5), ("v", 1)]
+    restart()
+    feed([("u", 3)]); feed([("v", 2)])
+    for _ in range(3):                      # built, captured, replayed
+        feed(first)
+    first_key = next(reversed(runner.programs))
+    assert runner.programs[first_key]["graph"] is not None
+    shapes = [[("u", n)] for n in (1, 2, 3, 5, 9, 17, 33)] + [[("u", n), ("v", m)] for n, m in ((1, 1), (2, 3), (9, 9), (17, 20))] \
+        + [[("u", 1), ("v", 1), ("w", 1)], [("u", 2), ("v", 1), ("w", 7)], [("u", 30), ("v", 1), ("w", 40)]]
+    seen = set()
+    for wanted in (True, False):
+        restart()
+        for parts in shapes:
+            for _ in range(2):              # the second run of a shape captures it
+                if max(fed[k] + n for k, n in parts) > 190:
+                    restart()
+                feed(parts, wanted)
+                seen.add(next(reversed(runner.programs)))
+            assert len(runner.programs) <= runner.program_capacity
+    assert len(seen) > runner.program_capacity, "not enough different shapes to push a program out"
+    assert first_key not in runner.programs, "the first program was never dropped"
+    restart()
+    feed([("u", 3)]); feed([("v", 2)])
+    for _ in range(3):                      # the dropped shape again: built, captured and replayed anew
+        feed(first)
+    again = runner.programs[first_key]
+    assert again["graph"] is not None and again["runs"] == 3
+    runner.cache.check()
 
 
 @pytest.mark.parametrize("name,dtype", [("d", "float32"), ("d", "bfloat16"), ("a", "bfloat16"), ("c", "bfloat16")])
@@ -359,6 +426,39 @@ def test_temperature_sampling_is_seeded_and_independent_of_the_batch(folders):
     assert e.generate(prompts[:2], max_new_tokens=12) != [together["0"], together["1"]]   # sampling is not greedy here
 
 
+@pytest.mark.parametrize("overlap,execution", [(False, "eager"), (True, "graph")])
+def test_sampled_tokens_are_those_of_a_plain_sampler(folders, overlap, execution):
+    """The tokens the engine samples (prompts of 1, 9, 33 and 64 tokens cut into portions of 7 beside decoding
+    requests, 12 tokens each at temperature 0.8) against float64 softmax(plain logits / T) drawn by inverse CDF at
+    uniform01(seed, index).  Each token is checked given the engine's own tokens before it; a draw that falls
+    within 2e-5 of an edge of its interval (the engine's softmax is 32-bit; a token's interval is about 2e-3 wide
+    with this vocabulary) may land on the neighbour and is only required to."""
+    import plain_sampling
+    from runtime.engine.scheduler import Engine, Request
+    cfg, w = P.read_folder(folders["b"])
+    V = TINY["b"]["vocab_size"]
+    prompts = [random_tokens(80 + i, n, V) for i, n in enumerate([1, 9, 33, 64])]
+    e = Engine.from_folder(folders["b"], dtype="float32", pages=64, page_size=8, token_budget=16, prefill_chunk=7,
+                           execution=execution, overlap=overlap)
+    for i, p in enumerate(prompts):
+        e.submit(Request(str(i), p, 12, temperature=0.8, seed=100 + i))
+    got = {r.key: r.generated for r in e.run()}
+    exact = 0
+    for i, p in enumerate(prompts):
+        tokens = got[str(i)]
+        assert len(tokens) == 12
+        for n, token in enumerate(tokens):
+            logits = P.forward(cfg, w, p + tokens[:n])[-1]
+            want, room = plain_sampling.draw(logits, 0.8, 100 + i, n)
+            if room > 2e-5:
+                assert token == want, f"request {i} token {n}: {token} instead of {want}"
+                exact += 1
+            else:
+                assert abs(token - want) <= 1, f"request {i} token {n}: {token} is no neighbour of {want}"
+    assert exact >= 40, "too few draws away from the edges to say anything"
+    assert any(t != g for i, p in enumerate(prompts) for t, g in zip(got[str(i)], P.greedy(cfg, w, p, 12))), "nothing was sampled"
+
+
 @pytest.mark.parametrize("execution", ["eager", "graph"])
 def test_overlapped_ticks_sample_and_stop_like_plain_ticks(folders, execution):
     """Steps launched before the tokens of the step before are read: the same sampled tokens, the same
@@ -385,6 +485,39 @@ def test_overlapped_ticks_sample_and_stop_like_plain_ticks(folders, execution):
     stopped = run(False, eos)
     assert len(stopped["0"]) <= 5 and stopped["0"][-1] == eos
     assert run(True, eos) == stopped
+
+
+@pytest.mark.parametrize("execution", ["eager", "graph"])
+def test_a_step_that_fails_leaves_its_requests_where_they_stood(folders, execution):
+    """Slots are placed before a step runs, the tokens are counted only once it is launched: a step that fails on
+    the way gives its pages back, and the same step, tried again, gives the right logits."""
+    from runtime.engine import load_model, ModelRunner, StepEntry
+    from conftest import plain_logits, assert_close
+    V = TINY["a"]["vocab_size"]
+    model = load_model(folders["a"], dtype="float32")
+    r = ModelRunner(model, n_pages=12, page_size=8, execution=execution)
+    a, b = random_tokens(31, 30, V), random_tokens(32, 12, V)
+    r.create("a"); r.create("b")
+    r.step([StepEntry("a", a[:5], []), StepEntry("b", b[:3], [])])
+    free = r.cache.free_pages()
+    real = model.forward
+
+    def broken(ctx):
+        raise RuntimeError("a kernel refused its shape")
+
+    model.forward = broken
+    try:
+        with pytest.raises(RuntimeError, match="refused"):
+            r.step([StepEntry("a", a[5:25], [19]), StepEntry("b", [b[3]], [0])])
+    finally:
+        model.forward = real
+    assert (r.length("a"), r.length("b")) == (5, 3) and r.cache.free_pages() == free
+    r.cache.check()
+    out = r.step([StepEntry("a", a[5:25], [19]), StepEntry("b", [b[3]], [0])]).cpu().numpy()
+    assert (r.length("a"), r.length("b")) == (25, 4)
+    assert_close(out[:1], plain_logits(folders["a"], a)[24:25], "float32", "the portion, tried again")
+    assert_close(out[1:], plain_logits(folders["a"], b)[3:4], "float32", "the decoded token, tried again")
+    r.cache.check()
 
 
 def test_fork_shares_a_prefix_and_copies_on_write(folders):

@@ -15,47 +15,51 @@ from trace_tools import Trace
 
 pytestmark = pytest.mark.gpu
 DTYPES = ["float32", "bfloat16"]
+EXECUTIONS = ["eager", "graph"]     # kernels launched one by one; every step as a captured program
 
 
-def run(folder, dtype, trace, out_dir, max_tokens=None, page_size=None):
+def run(folder, dtype, trace, out_dir, max_tokens=None, page_size=None, execution="eager"):
     from runtime.engine.replay import replay, PAGE_SIZE
     done = []
     runner = replay(folder, dtype, out_dir, max_tokens or trace.peak, trace.lines(), page_size=page_size or PAGE_SIZE,
-                    echo=done.append)
+                    echo=done.append, execution=execution)
     assert done == [f"done {i}" for i in range(len(trace.steps))]
     runner.cache.check()
     return runner
 
 
+@pytest.mark.parametrize("execution", EXECUTIONS)
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", ["a", "b", "c", "d"])
-def test_whole_requests_alone(folders, tmp_path, name, dtype):
+def test_whole_requests_alone(folders, tmp_path, name, dtype, execution):
     V = TINY[name]["vocab_size"]
     seqs = {f"r{i}": random_tokens(10 * i + 1, n, V) for i, n in enumerate([1, 5, 64, 65, 150])}
     trace = Trace()
     for rid, toks in seqs.items():
         trace.add([(rid, toks, list(range(len(toks))))], end=[rid])
-    runner = run(folders[name], dtype, trace, tmp_path)
+    runner = run(folders[name], dtype, trace, tmp_path, execution=execution)
     trace.check(folders[name], tmp_path, dtype, V, seqs)
     assert all(free == g.pool.n_pages for free, g in zip(runner.cache.free_pages(), runner.cache.groups))
 
 
+@pytest.mark.parametrize("execution", EXECUTIONS)
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", ["a", "b", "c", "d"])
-def test_prefix_then_last_32_one_by_one(folders, tmp_path, name, dtype):
+def test_prefix_then_last_32_one_by_one(folders, tmp_path, name, dtype, execution):
     V = TINY[name]["vocab_size"]
     toks = random_tokens(77, 131, V)
     trace = Trace()
     trace.add([("p", toks[:-32], list(range(len(toks) - 32)))])
     for t in toks[-32:]:
         trace.add([("p", [t], [0])])
-    run(folders[name], dtype, trace, tmp_path)
+    run(folders[name], dtype, trace, tmp_path, execution=execution)
     trace.check(folders[name], tmp_path, dtype, V, {"p": toks})
 
 
+@pytest.mark.parametrize("execution", EXECUTIONS)
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", ["a", "b", "c", "d"])
-def test_portions_of_changing_size(folders, tmp_path, name, dtype):
+def test_portions_of_changing_size(folders, tmp_path, name, dtype, execution):
     V = TINY[name]["vocab_size"]
     toks = random_tokens(5, 140, V)
     trace, at = Trace(), 0
@@ -68,7 +72,7 @@ def test_portions_of_changing_size(folders, tmp_path, name, dtype):
         trace.add([("q", toks[at:at + n], want)])
         at += n
     trace.add([("q", toks[at:], list(range(len(toks) - at)))], end=["q"])
-    run(folders[name], dtype, trace, tmp_path)
+    run(folders[name], dtype, trace, tmp_path, execution=execution)
     trace.check(folders[name], tmp_path, dtype, V, {"q": toks})
 
 
@@ -109,14 +113,15 @@ def mixed_trace(V, seed):
     return trace, seqs
 
 
+@pytest.mark.parametrize("execution", EXECUTIONS)
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", ["a", "b", "c", "d"])
-def test_mixed_requests_reuse_pages(folders, tmp_path, name, dtype):
+def test_mixed_requests_reuse_pages(folders, tmp_path, name, dtype, execution):
     V = TINY[name]["vocab_size"]
     trace, seqs = mixed_trace(V, seed=3)
     assert any(len(s["entries"]) == 4 for s in trace.steps)
     assert any(len(e["tokens"]) > 1 for s in trace.steps for e in s["entries"] if len(s["entries"]) > 1)
-    runner = run(folders[name], dtype, trace, tmp_path)          # pool = exactly the peak of rounded-up tokens
+    runner = run(folders[name], dtype, trace, tmp_path, execution=execution)   # pool = exactly the peak of rounded-up tokens
     pool = runner.cache.groups[0].pool
     assert pool.n_pages * 16 == trace.peak
     assert sum(-(-len(s) // 16) for s in seqs.values()) > pool.n_pages, "the trace must need more pages than exist"
@@ -124,15 +129,16 @@ def test_mixed_requests_reuse_pages(folders, tmp_path, name, dtype):
     trace.check(folders[name], tmp_path, dtype, V, seqs)
 
 
+@pytest.mark.parametrize("execution", EXECUTIONS)
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_long_decoding_and_first_tokens(folders, tmp_path, dtype):
+def test_long_decoding_and_first_tokens(folders, tmp_path, dtype, execution):
     name = "a"
     V = TINY[name]["vocab_size"]
     toks = random_tokens(9, 300, V)
     trace = Trace()
     for t in toks:                       # position 0 alone, then 299 single-token steps
         trace.add([("d", [t], [0])])
-    run(folders[name], dtype, trace, tmp_path)
+    run(folders[name], dtype, trace, tmp_path, execution=execution)
     got = trace.check(folders[name], tmp_path, dtype, V, {"d": toks})
     assert [p for p, _ in got["d"]][:3] == [0, 1, 2]
 
@@ -176,8 +182,8 @@ def test_out_of_pages_and_bad_input_fail_loudly(folders, tmp_path):
         run(folders["a"], "float32", over, tmp_path, max_tokens=1024)
 
 
-@pytest.mark.parametrize("dtype", DTYPES)
-def test_trace_run_program(folders, tmp_path, dtype):
+@pytest.mark.parametrize("dtype,execution", [("float32", None), ("bfloat16", None), ("bfloat16", "graph")])
+def test_trace_run_program(folders, tmp_path, dtype, execution):
     """The program itself, as a user runs it: reads steps from its input, writes
     <step>.f32 and prints `done <step>` after every step."""
     name = "b"
@@ -191,7 +197,8 @@ def test_trace_run_program(folders, tmp_path, dtype):
     out = tmp_path / "out"
     env = dict(os.environ, PYTHONPATH="")
     proc = subprocess.run([sys.executable, str(ROOT / "bin" / "trace_run"), "--model", str(folders[name]), "--dtype", dtype,
-                           "--out", str(out), "--max-tokens", str(trace.peak)], input="\n".join(trace.lines()) + "\n",
+                           "--out", str(out), "--max-tokens", str(trace.peak)] + (["--execution", execution] if execution else []),
+                          input="\n".join(trace.lines()) + "\n",
                           capture_output=True, text=True, timeout=300, env=env, cwd=str(tmp_path))
     assert proc.returncode == 0, proc.stderr[-2000:]
     assert proc.stdout.split("\n")[:len(trace.steps)] == [f"done {i}" for i in range(len(trace.steps))]

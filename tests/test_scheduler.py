@@ -179,6 +179,32 @@ def test_when_pages_run_out_requests_wait_and_none_fails():
     assert runner.cache.free_pages() == [6]
 
 
+def test_pages_are_promised_group_by_group():
+    """Two cache groups: one keeps every key (plenty of pages), one a window of 8 (few pages).  A request is
+    promised all its pages in the first and what a window and a portion can touch in the second, and the
+    scarcer group decides how many run together."""
+    runner = FakeRunner(pages=40, max_context=512)
+    window = KVNeed(1, 8, window=8)
+    runner.cache = CacheManager({0: KVNeed(1, 8), 1: window}, {KVNeed(1, 8): 40, window: 9}, 4, 8)
+    e = make_engine(runner, token_budget=8, prefill_chunk=4)
+    assert e.ledger.need(30) == [8, 4]               # ceil(30/4); (8 + 4 - 1)//4 + 2
+    assert e.ledger.need(5) == [2, 2]                # a short request never holds more than its tokens
+    for i in range(3):
+        e.submit(Request(str(i), [1] * 27, 4))       # 30 cached tokens each
+    e.tick()
+    assert [r.key for r in e.active] == ["0", "1"] and [r.key for r in e.waiting] == ["2"]   # 3 x 4 > 9 window pages
+    assert e.reserved == {"0": 12, "1": 12}
+    peak = [0, 0]
+    while e.tick():
+        peak = [max(p, g.pool.used) for p, g in zip(peak, runner.cache.groups)]
+        runner.cache.check()
+    assert peak[0] <= 16 and peak[1] <= 8
+    assert all(r.status == "finished" and len(r.generated) == 4 for r in e.requests.values())
+    assert runner.cache.free_pages() == [40, 9] and not e.reserved
+    with pytest.raises(ValueError, match="can never run"):
+        e.submit(Request("huge", [1] * 200, 1))      # 50 pages in the group that keeps everything
+
+
 def test_a_small_request_passes_a_large_one_that_does_not_fit_yet():
     runner = FakeRunner(pages=6)
     e = make_engine(runner, token_budget=8, prefill_chunk=8)

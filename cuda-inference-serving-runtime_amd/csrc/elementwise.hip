@@ -380,10 +380,12 @@ extern "C" int cisr_swiglu(const void* gu, void* act, int rows, int inter, int d
 // One block per token row of the fused projection buffer
 //   qkv[r] = [ q: heads*D | k: kv_heads*D | v: kv_heads*D ].
 // q is rotated in place; k is rotated and written to the cache; v is copied to
-// the cache.  Pairing is split-half over the first `rot` coordinates of a head:
-// (i, i + rot/2) turns by the angle whose cosine and sine sit in
-// cos_tab/sin_tab[pos, i] (tables are float, [max_pos, rot/2]).
-// (reference: kernels/ops.cu:21-33, kernels/execution.cu:28-40)
+// the cache.  Pair i of the first `rot` coordinates of a head turns by the angle
+// whose cosine and sine sit in cos_tab/sin_tab[pos, i] (tables are float,
+// [max_pos, rot/2]).  Which coordinates pair i is made of is a parameter:
+// split-half, (i, i + rot/2), the reference's rule (kernels/ops.cu:21-33,
+// kernels/execution.cu:28-40), or interleaved, (2i, 2i + 1).  The vectorised
+// kernel below and the fused projection kernels are the split-half rule only.
 // Cache layout per site: keys [pages, kv_heads, page_size, D], values transposed
 // inside a page, [pages, kv_heads, D, page_size] (so that the attention kernels
 // read runs of keys for one coordinate); slot = page*page_size + offset; a
@@ -393,9 +395,11 @@ __global__ void rope_scatter_kernel(T* __restrict__ qkv, const int* __restrict__
                                     const int* __restrict__ slots, const float* __restrict__ cos_tab,
                                     const float* __restrict__ sin_tab, T* __restrict__ kcache,
                                     T* __restrict__ vcache, int heads, int kv_heads, int dim, int rot,
-                                    int page_size, int max_pos, int has_kv) {
+                                    int page_size, int max_pos, int has_kv, int interleaved) {
     const int row = blockIdx.x;
     const int half = rot / 2;
+    // which two coordinates pair d turns: (d, d + rot/2) in the split-half rule, (2d, 2d + 1) in the interleaved one
+    const int lo_mul = interleaved ? 2 : 1, hi_add = interleaved ? 1 : half;
     int pos = positions[row];
     if (pos < 0) pos = 0;
     if (pos >= max_pos) pos = max_pos - 1;  // host rejects this before launch
@@ -410,10 +414,11 @@ __global__ void rope_scatter_kernel(T* __restrict__ qkv, const int* __restrict__
     for (int i = threadIdx.x; i < heads * half; i += blockDim.x) {
         int h = i / half, d = i % half;
         T* p = base + h * dim;
-        float a = load_f32(p + d), b = load_f32(p + d + half);
+        const int lo = d * lo_mul, hi = lo + hi_add;
+        float a = load_f32(p + lo), b = load_f32(p + hi);
         float c = cs[d], s = sn[d];
-        store_f32(p + d, a * c - b * s);
-        store_f32(p + d + half, b * c + a * s);
+        store_f32(p + lo, a * c - b * s);
+        store_f32(p + hi, b * c + a * s);
     }
     if (slot < 0) return;
     // k heads: rotate and scatter
@@ -421,11 +426,12 @@ __global__ void rope_scatter_kernel(T* __restrict__ qkv, const int* __restrict__
     for (int i = threadIdx.x; i < kv_heads * half; i += blockDim.x) {
         int h = i / half, d = i % half;
         const T* p = kb + h * dim;
-        float a = load_f32(p + d), b = load_f32(p + d + half);
+        const int lo = d * lo_mul, hi = lo + hi_add;
+        float a = load_f32(p + lo), b = load_f32(p + hi);
         float c = cs[d], s = sn[d];
         T* dst = kcache + (((size_t)page * kv_heads + h) * page_size + off) * dim;
-        store_f32(dst + d, a * c - b * s);
-        store_f32(dst + d + half, b * c + a * s);
+        store_f32(dst + lo, a * c - b * s);
+        store_f32(dst + hi, b * c + a * s);
     }
     // coordinates beyond the rotated part of k pass through
     if (rot < dim) {
@@ -560,12 +566,12 @@ rope_scatter_wave_kernel(bf16_t* __restrict__ qkv, const int* __restrict__ posit
 extern "C" int cisr_rope_scatter(void* qkv, const int* positions, const int* slots, const float* cos_tab,
                                  const float* sin_tab, void* kcache, void* vcache, int rows, int heads,
                                  int kv_heads, int dim, int rot, int page_size, int max_pos, int has_kv,
-                                 int dtype, hipStream_t stream) {
+                                 int interleaved, int dtype, hipStream_t stream) {
     if (rows <= 0) return 0;
     if (dtype == DT_F32) {
         rope_scatter_kernel<float><<<rows, 256, 0, stream>>>((float*)qkv, positions, slots, cos_tab, sin_tab,
-            (float*)kcache, (float*)vcache, heads, kv_heads, dim, rot, page_size, max_pos, has_kv);
-    } else if (rot == dim && dim % 16 == 0 && (uintptr_t)qkv % 16 == 0 && (uintptr_t)cos_tab % 16 == 0 &&
+            (float*)kcache, (float*)vcache, heads, kv_heads, dim, rot, page_size, max_pos, has_kv, interleaved);
+    } else if (!interleaved && rot == dim && dim % 16 == 0 && (uintptr_t)qkv % 16 == 0 && (uintptr_t)cos_tab % 16 == 0 &&
                (uintptr_t)sin_tab % 16 == 0 && (!has_kv || (uintptr_t)kcache % 16 == 0)) {
         // lanes a row: as many as it has 8-pair chunks to turn, so that every lane's loads are in flight at once
         const int chunks = (heads + (has_kv ? kv_heads : 0)) * (dim / 16);
@@ -579,7 +585,7 @@ extern "C" int cisr_rope_scatter(void* qkv, const int* positions, const int* slo
             qk_blocks);
     } else {
         rope_scatter_kernel<bf16_t><<<rows, 256, 0, stream>>>((bf16_t*)qkv, positions, slots, cos_tab, sin_tab,
-            (bf16_t*)kcache, (bf16_t*)vcache, heads, kv_heads, dim, rot, page_size, max_pos, has_kv);
+            (bf16_t*)kcache, (bf16_t*)vcache, heads, kv_heads, dim, rot, page_size, max_pos, has_kv, interleaved);
     }
     return CISR_LAUNCH_CHECK();
 }

@@ -44,7 +44,7 @@ def _declare(h):
         "cisr_add_rmsnorm": [p, p, p, p, i, i, f, i, p],
         "cisr_residual_add": [p, p, ll, i, p],
         "cisr_swiglu": [p, p, i, i, i, p],
-        "cisr_rope_scatter": [p, p, p, p, p, p, p, i, i, i, i, i, i, i, i, i, p],
+        "cisr_rope_scatter": [p, p, p, p, p, p, p, i, i, i, i, i, i, i, i, i, i, p],
         "cisr_page_copy": [p, p, p, i, i, ll, ll, p],
         "cisr_f32_to_bf16": [p, p, ll, p],
         "cisr_attn_rowwise": [p, i, p, p, p, p, p, p, p, p, i, i, i, i, i, i, i, f, i, i, p],
@@ -219,9 +219,10 @@ def swiglu(gate_up, out):
     return out
 
 
-def rope_scatter(qkv, positions, slots, cos, sin, kcache, vcache, heads, kv_heads, dim, page_size):
+def rope_scatter(qkv, positions, slots, cos, sin, kcache, vcache, heads, kv_heads, dim, page_size, interleaved=False):
     """Rotate q (in place) and k of the fused projection rows, write k and v into
     the cache at `slots`.  kcache/vcache None: q only (a layer reading another's cache).
+    Pair i of a head is coordinates (i, i + rot/2), or with `interleaved` (2i, 2i + 1).
     qkv [T, (heads + 2 kv_heads) * dim] (or [T, heads * dim] without a cache);
     cos/sin float [max_pos, rot/2]; keys [pages, kv_heads, page_size, dim],
     values transposed in a page: [pages, kv_heads, dim, page_size]."""
@@ -241,8 +242,8 @@ def rope_scatter(qkv, positions, slots, cos, sin, kcache, vcache, heads, kv_head
         sp = _dev(slots, "slots", torch.int32, (rows,))
     _check(lib().cisr_rope_scatter(_dev(qkv, "qkv", None, (rows, width)), _dev(positions, "positions", torch.int32, (rows,)),
                                    sp, _dev(cos, "cos", torch.float32), _dev(sin, "sin", torch.float32, (max_pos, half)),
-                                   kp, vp, rows, heads, kv_heads, dim, rot, page_size, max_pos, int(has_kv), dt,
-                                   _stream()), "rope_scatter")
+                                   kp, vp, rows, heads, kv_heads, dim, rot, page_size, max_pos, int(has_kv),
+                                   int(bool(interleaved)), dt, _stream()), "rope_scatter")
 
 
 def page_copy(pool, src, dst, slabs, pages_per_slab):

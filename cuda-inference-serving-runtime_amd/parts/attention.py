@@ -50,9 +50,14 @@ class PagedAttention(Mixer):
     def prepare(self, device, dtype):
         self.position.prepare(device, dtype)
 
+    @property
+    def _interleaved(self):
+        return getattr(self.position, "pairing", "split_half") == "interleaved"
+
     def _fused_projection_ok(self, a, normed):
         cos, _ = self.position.tables()
-        return ops.qkv_rope_fused_ok(a, self.w_in, self.head_dim, cos, normed)
+        # (the fused kernels turn split-half pairs only; another pairing takes the general rotary kernel)
+        return not self._interleaved and ops.qkv_rope_fused_ok(a, self.w_in, self.head_dim, cos, normed)
 
     def fuses_norm(self, norm, residual, ctx):
         return getattr(norm, "fusable_as", None) == "rms" and self._fused_projection_ok(residual, True)
@@ -77,7 +82,8 @@ class PagedAttention(Mixer):
             q_stride = (nh + (2 * nkv if self.own_kv else 0)) * D
             q = ctx.buffer("attn.qkv", (T, q_stride), ctx.dtype)
             ops.gemm(h, self.w_in, q)
-            ops.rope_scatter(q, ctx.positions, slots, cos, sin, kcache_w, vcache_w, nh, nkv, D, view.page_size)
+            ops.rope_scatter(q, ctx.positions, slots, cos, sin, kcache_w, vcache_w, nh, nkv, D, view.page_size,
+                             interleaved=self._interleaved)
         out = ctx.buffer("attn.out", (T, nh * D), ctx.dtype)
         ctx.attend(q, q_stride, kcache, vcache, view, out, nh, nkv, D, self.window, self.scale)
         return ctx.add_product(out, self.w_out, residual)

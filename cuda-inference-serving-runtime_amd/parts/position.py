@@ -5,6 +5,11 @@ RotaryEmbedding is the split-half rotary embedding: coordinate pair
 (reference: runtime/reference.py:9-15, kernels/ops.cu:21-33).  Angles are
 computed on the host in float64 and stored as float cosine/sine tables, so the
 kernels do no transcendental arithmetic.  NoPosition turns nothing.
+
+What a position part gives a mixer: `tables() -> (cos, sin)` float
+[max_positions, pairs], and `pairing`: which two coordinates of a head pair i
+is, "split_half" (i, i + pairs) or "interleaved" (2i, 2i + 1).  A part without
+the attribute is split-half.
 """
 import numpy as np
 import torch
@@ -13,7 +18,10 @@ from .base import Part, register_part
 
 
 class RotaryEmbedding(Part):
-    def __init__(self, head_dim, theta, max_positions, rotary_dim=None):
+    def __init__(self, head_dim, theta, max_positions, rotary_dim=None, pairing="split_half"):
+        if pairing not in ("split_half", "interleaved"):
+            raise ValueError(f"pairing {pairing!r} is neither split_half nor interleaved")
+        self.pairing = pairing
         self.head_dim, self.theta, self.max_positions = head_dim, float(theta), int(max_positions)
         self.rotary_dim = head_dim if rotary_dim is None else rotary_dim
         if self.rotary_dim % 2 or not 0 < self.rotary_dim <= head_dim:
@@ -38,6 +46,7 @@ class RotaryEmbedding(Part):
 
 class NoPosition(Part):
     """Identity: a one-pair table with angle zero."""
+    pairing = "split_half"
 
     def __init__(self, head_dim, max_positions=1, **_):
         self.head_dim, self.max_positions = head_dim, int(max_positions)

@@ -54,3 +54,32 @@ def test_family_layer_sizes(family_folders, name, dtype):
         assert fed[k] == len(seqs[k])
         assert_close(np.concatenate(got[k]), plain_logits(folder, seqs[k]), dtype, what=f"{name} request {k}")
     runner.cache.check()
+
+
+@pytest.mark.parametrize("name", ["smollm2-1.7b", "llama-3-8b"])
+def test_a_cut_across_the_library_threshold_changes_rounding_only(family_folders, name):
+    """With large weights a portion of more than 64 rows takes the vendor library's bf16 product, whose output
+    projection and down projection are rounded to bfloat16 before they are added to the float residual; 64 rows
+    and fewer add the float accumulator.  The same prompt cut at 65 + 35 and at 64 + 36 rows therefore differs by
+    that rounding, and by nothing more: the difference between the two runs stays far inside the bound that
+    either holds against the plain implementation."""
+    from runtime.engine import load_model, ModelRunner, StepEntry
+    from runtime.kernels import ops
+    from conftest import BF16_RMSE
+    folder = family_folders[name]
+    V = FAMILY[name]["vocab_size"]
+    tokens = random_tokens(5, 100, V)
+    model = load_model(folder, dtype="bfloat16")
+    assert ops.library_ok(65, model.layers[0].mixer.w_out) and not ops.library_ok(64, model.layers[0].mixer.w_out)
+    runs = []
+    for first in (65, 64):
+        runner = ModelRunner(model, n_pages=16, page_size=16, max_requests=2)
+        runner.create("p")
+        out = [runner.step([StepEntry("p", tokens[:first], list(range(first)))]).float().cpu().numpy(),
+               runner.step([StepEntry("p", tokens[first:], list(range(100 - first)))]).float().cpu().numpy()]
+        runs.append(np.concatenate(out))
+    ref = plain_logits(folder, tokens)
+    for got in runs:
+        assert_close(got, ref, "bfloat16", what=name)
+    between = np.linalg.norm(runs[0] - runs[1]) / np.linalg.norm(ref)
+    assert between < BF16_RMSE / 4, f"the two cuts differ by {between:.3e}"

@@ -140,6 +140,45 @@ def test_rope_scatter(ops, dtype, heads, kv_heads, dim, theta):
             assert (kc64[s // P_, :, s % P_] == 7).all() and (vc64[s // P_, :, :, s % P_] == 7).all()
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("heads, kv_heads, dim, rot", [(4, 2, 10, 10), (9, 3, 64, 64), (5, 1, 24, 16)])
+def test_rope_scatter_with_interleaved_pairs(ops, dtype, heads, kv_heads, dim, rot):
+    """The pairing rule is a parameter of the rotary kernel: pair i is coordinates (2i, 2i + 1) instead of
+    (i, i + rot/2); with rot < dim the coordinates from rot on pass through.  Checked against complex
+    multiplication of (x[2i] + j x[2i+1]) by exp(j angle); the split-half rule on the same rows must differ."""
+    from runtime.parts import RotaryEmbedding
+    theta = 1e4
+    rope = RotaryEmbedding(dim, theta, 600, rotary_dim=rot, pairing="interleaved")
+    rope.prepare(DEV, dtype)
+    cos, sin = rope.tables()
+    T, P_, pages = 4, 4, 5
+    qkv = rnd(T, (heads + 2 * kv_heads) * dim, dtype=dtype, seed=12)
+    ref = f64(qkv)
+    pos, slots = [0, 17, 500, 3], [6, 1, 19, 8]
+    kc = torch.zeros((pages, kv_heads, P_, dim), dtype=dtype, device=DEV)
+    vc = torch.zeros((pages, kv_heads, dim, P_), dtype=dtype, device=DEV)
+    split = qkv.clone()
+    ops.rope_scatter(qkv, torch.tensor(pos, dtype=torch.int32, device=DEV), torch.tensor(slots, dtype=torch.int32, device=DEV),
+                     cos, sin, kc, vc, heads, kv_heads, dim, P_, interleaved=True)
+
+    def turn(x):          # [T, heads, dim]
+        angle = np.asarray(pos, np.float64)[:, None] * (theta ** (-np.arange(rot // 2) * 2.0 / rot))[None, :]
+        z = (x[..., 0:rot:2] + 1j * x[..., 1:rot:2]) * np.exp(1j * angle)[:, None, :]
+        out = x.copy()
+        out[..., 0:rot:2], out[..., 1:rot:2] = z.real, z.imag
+        return out
+
+    q_ref = turn(ref[:, :heads * dim].reshape(T, heads, dim))
+    k_ref = turn(ref[:, heads * dim:(heads + kv_heads) * dim].reshape(T, kv_heads, dim))
+    np.testing.assert_allclose(f64(qkv)[:, :heads * dim].reshape(T, heads, dim), q_ref, **tol(dtype))
+    for t, s in enumerate(slots):
+        np.testing.assert_allclose(f64(kc)[s // P_, :, s % P_], k_ref[t], **tol(dtype))
+        np.testing.assert_array_equal(f64(vc)[s // P_, :, :, s % P_], ref[t, (heads + kv_heads) * dim:].reshape(kv_heads, dim))
+    ops.rope_scatter(split, torch.tensor(pos, dtype=torch.int32, device=DEV), torch.tensor(slots, dtype=torch.int32, device=DEV),
+                     cos, sin, torch.zeros_like(kc), torch.zeros_like(vc), heads, kv_heads, dim, P_)
+    assert np.abs(f64(split)[1:, :heads * dim] - f64(qkv)[1:, :heads * dim]).max() > 1e-2      # the other rule gives other rows
+
+
 @pytest.mark.parametrize("heads, kv_heads, dim, page_size, T, start", [
     (9, 3, 64, 16, 100, None), (4, 4, 16, 4, 37, None), (3, 1, 128, 16, 33, None), (34, 34, 32, 8, 50, None),
     (9, 3, 64, 16, 100, 0), (34, 34, 32, 16, 70, 16), (3, 1, 128, 32, 64, 8), (4, 2, 64, 16, 48, 5), (32, 32, 64, 16, 64, 0)])
@@ -442,6 +481,48 @@ def test_attention_mfma_window_and_far_key(ops):
     want = reference_attention(qt, kt, vt, tables, rows, 16)
     for mode, splits in (("rows", 1), ("rows", 8), ("tiles", 1), ("block", 1), ("block2", 1)):
         np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables, rows, 16, mode, splits), want, **MFMA_TOL)
+
+
+def test_attention_mfma_ignores_what_unseen_slots_hold(ops):
+    """Pages are not cleared when they change owners: the slots of a request's last page behind its last key, and
+    page 0 (read in place of a page that a window has passed), may hold anything, Inf and NaN included.  Keys there
+    have weight zero, and their values must not reach the output (0 x Inf is NaN)."""
+    heads, kv_heads, dim, P_ = 6, 2, 64, 16
+    plan = [(21, 14), (0, 5), (70, 1)]                       # last keys at 34, 4 and 70: none at a page's end
+    qt, kt, vt, tables, rows = portion_case(heads, kv_heads, dim, P_, plan, seed=77)
+    tab = tables.cpu().numpy()
+    poison = [float("inf"), float("-inf"), float("nan")]
+    want = {}
+    for window in (None, 16):
+        want[window] = reference_attention(qt, kt, vt, tables, rows, P_, window=window)
+    for s, (a, b) in enumerate(plan):
+        last = a + b - 1
+        page = tab[s, last // P_]
+        for off in range(last % P_ + 1, P_):                 # the rest of the last page
+            kt[page, :, off, :] = poison[off % 3]
+            vt[page, :, :, off] = poison[(off + 1) % 3]
+    used = {int(p) for p in tab.flatten() if p >= 0}
+    spare = next(p for p in range(kt.shape[0]) if p not in used)
+    kt[spare], vt[spare] = float("nan"), float("inf")        # a page of nobody's, standing in for page 0 below
+    for window in (None, 16):
+        t2 = tables.clone()
+        if window:                                           # request 2 (position 70, window 16 from 55): pages 0..2 passed
+            t2[2, :3] = -1
+        for mode, splits in (("tiles", 1), ("tiles2", 1), ("block", 1), ("block2", 1), ("rows", 1), ("rows", 3)):
+            got = run_mfma(ops, qt, kt, vt, t2, rows, P_, mode, splits, window=window)
+            assert np.isfinite(got).all(), f"{mode} window={window}: poison reached the output"
+            np.testing.assert_allclose(got, want[window], **MFMA_TOL, err_msg=f"{mode} window={window}")
+    # page 0 itself poisoned, with a table whose passed pages read it
+    if 0 not in {int(tab[2, j]) for j in range(3, 5)}:
+        k0, v0 = kt[0].clone(), vt[0].clone()
+        kt[0], vt[0] = float("nan"), float("nan")
+        t2 = tables.clone(); t2[2, :3] = -1
+        only = [i for i, (s, _) in enumerate(rows) if s == 2]
+        sub_rows = [rows[i] for i in only]
+        got = run_mfma(ops, qt[only].contiguous(), kt, vt, t2, sub_rows, P_, "rows", 2, window=16)
+        assert np.isfinite(got).all()
+        np.testing.assert_allclose(got, want[16][only], **MFMA_TOL)
+        kt[0], vt[0] = k0, v0
 
 
 def test_gemm_skinny_and_fused_swiglu(ops):

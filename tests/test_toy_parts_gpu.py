@@ -320,3 +320,116 @@ def test_toy_routed_feed_forward_and_position_encoding_are_registered_built_and_
         runner.cache.check()
     finally:
         cleanup()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_position_encoding_with_interleaved_pairs(tmp_path, dtype):
+    """A position encoding, defined here, whose pairs are neighbouring coordinates (2i, 2i + 1): it states its
+    pairing, the framework's attention turns queries and keys by that rule (the kernels that fuse the rotation
+    into the projection know the split-half rule only and step aside), and prompts cut into portions beside
+    decoded tokens match a plain implementation that multiplies complex numbers."""
+    import plain_llama as P
+    from conftest import assert_close
+    from runtime import register_part, make_part, register_architecture
+    from runtime.config import unregister_architecture
+    from runtime.engine import load_model, ModelRunner, StepEntry
+    from runtime.engine.loading import build_from_config_dict
+    from runtime.models import Model
+    from runtime.parts import Part, TokenEmbedding, LMHead, unregister_part
+    from runtime.weights import write_model_folder
+
+    class NeighbourPairs(Part):
+        pairing = "interleaved"
+
+        def __init__(self, head_dim, theta, max_positions):
+            self.head_dim, self.theta, self.max_positions, self._tables = head_dim, theta, max_positions, None
+
+        def prepare(self, device, dtype):
+            half = self.head_dim // 2
+            a = np.arange(self.max_positions, dtype=np.float64)[:, None] * self.theta ** (-np.arange(half) * 2.0 / self.head_dim)[None, :]
+            self._tables = (torch.from_numpy(np.cos(a).astype(np.float32)).to(device), torch.from_numpy(np.sin(a).astype(np.float32)).to(device))
+
+        def tables(self):
+            return self._tables
+
+    @dataclass(frozen=True)
+    class PairsConfig:
+        vocab_size: int
+        hidden_size: int
+        theta: float
+        max_position_embeddings: int
+        rms_norm_eps: float
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(*(raw[k] for k in ("vocab_size", "hidden_size", "theta", "max_position_embeddings", "rms_norm_eps")))
+
+    HEADS, KV, D = 4, 2, 16
+
+    def build(c):
+        def norm(n): return make_part("norm", "rmsnorm", name=n, dim=c.hidden_size, eps=c.rms_norm_eps)
+        position = make_part("position", "toy-neighbour-pairs", head_dim=D, theta=c.theta, max_positions=c.max_position_embeddings)
+        layers = [make_part("block", "prenorm", mixer_norm=norm(f"l{i}.n1"),
+                            mixer=make_part("mixer", "attention", name=f"l{i}.attn", hidden=c.hidden_size, heads=HEADS, kv_heads=KV,
+                                            head_dim=D, position=position),
+                            ffn_norm=norm(f"l{i}.n2"),
+                            ffn=make_part("ffn", "gated_mlp", name=f"l{i}.mlp", hidden=c.hidden_size, intermediate=40))
+                  for i in range(2)]
+        return Model(c, TokenEmbedding("embed", c.vocab_size, c.hidden_size), layers, norm("final"),
+                     LMHead("head", c.vocab_size, c.hidden_size))
+
+    def plain(raw, w, tokens):
+        T, eps = len(tokens), raw["rms_norm_eps"]
+        angle = np.arange(T)[:, None] * raw["theta"] ** (-np.arange(D // 2) * 2.0 / D)[None, :]
+
+        def turn(v):      # [T, heads, D]: (v[2i] + j v[2i+1]) * exp(j angle_i)
+            z = (v[..., 0::2] + 1j * v[..., 1::2]) * np.exp(1j * angle)[:, None, :]
+            out = np.empty_like(v)
+            out[..., 0::2], out[..., 1::2] = z.real, z.imag
+            return out
+
+        x = w["embed.weight"][tokens]
+        for i in range(2):
+            h = P.rmsnorm(x, w[f"l{i}.n1.weight"], eps)
+            q = turn(P.linear(h, w[f"l{i}.attn.q_proj.weight"]).reshape(T, HEADS, D))
+            k = turn(P.linear(h, w[f"l{i}.attn.k_proj.weight"]).reshape(T, KV, D))
+            v = P.linear(h, w[f"l{i}.attn.v_proj.weight"]).reshape(T, KV, D)
+            x = x + P.linear(P.causal_attention(q, k, v).reshape(T, HEADS * D), w[f"l{i}.attn.o_proj.weight"])
+            h = P.rmsnorm(x, w[f"l{i}.n2.weight"], eps)
+            x = x + P.linear(P.swiglu(P.linear(h, w[f"l{i}.mlp.gate_proj.weight"]), P.linear(h, w[f"l{i}.mlp.up_proj.weight"])),
+                             w[f"l{i}.mlp.down_proj.weight"])
+        return P.linear(P.rmsnorm(x, w["final.weight"], eps), w["head.weight"])
+
+    register_part("position", "toy-neighbour-pairs", NeighbourPairs)
+    register_architecture("toy-pairs-lm", PairsConfig, build)
+    try:
+        raw = {"model_type": "toy-pairs-lm", "vocab_size": 67, "hidden_size": 48, "theta": 50.0, "max_position_embeddings": 96,
+               "rms_norm_eps": 1e-5}
+        tmp_path.mkdir(exist_ok=True)
+        _, _, blueprint = build_from_config_dict(raw)
+        write_model_folder(tmp_path, raw, blueprint.tensor_specs(), seed=8, dtype=torch.bfloat16, std=0.15)
+        cfg, w = P.read_folder(tmp_path)
+        model = load_model(tmp_path, dtype=dtype)
+        runner = ModelRunner(model, n_pages=16, page_size=8, max_requests=2)
+        tokens = {"x": np.random.default_rng(4).integers(0, 67, 40).tolist(), "y": np.random.default_rng(5).integers(0, 67, 21).tolist()}
+        want = {k: plain(raw, w, v) for k, v in tokens.items()}
+        runner.create("x"); runner.create("y")
+        got, fed = {"x": [], "y": []}, {"x": 0, "y": 0}
+        for step in [[("x", 13), ("y", 2)], [("x", 1), ("y", 9)], [("x", 1), ("y", 1)], [("x", 25), ("y", 9)]]:
+            entries = [StepEntry(k, tokens[k][fed[k]:fed[k] + n], list(range(n))) for k, n in step]
+            out = runner.step(entries).float().cpu().numpy()
+            row = 0
+            for k, n in step:
+                got[k].append(out[row:row + n]); row += n; fed[k] += n
+        for k in tokens:
+            assert_close(np.concatenate(got[k]), want[k], dtype, f"request {k}")
+        # the pairing matters: the split-half rule on the same weights gives other logits
+        q = np.random.default_rng(0).standard_normal((3, 1, D))
+        assert np.abs(P.rope(q, [1, 2, 3], 50.0) - q).max() > 0.1
+        half_turned = P.rope(q, [1, 2, 3], 50.0)
+        z = (q[..., 0::2] + 1j * q[..., 1::2]) * np.exp(1j * (np.asarray([1, 2, 3])[:, None] * 50.0 ** (-np.arange(D // 2) * 2.0 / D)))[:, None, :]
+        assert np.abs(half_turned[..., 0::2] - z.real).max() > 0.1
+        runner.cache.check()
+    finally:
+        unregister_part("position", "toy-neighbour-pairs")
+        unregister_architecture("toy-pairs-lm")

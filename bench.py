@@ -17,72 +17,34 @@ PEAK_TFLOPS = {"bf16": 2500.0, "fp32": 157.3}
 REFERENCE_B1_TOKS = 203.9    # the reference's own graph-replay decode, batch 1, FP32, RTX 4060 Laptop
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=128)
-    ap.add_argument("--warmup", type=int, default=16)
-    ap.add_argument("--model", default="smollm2-135m")
-    ap.add_argument("--layers", type=int, default=None, help="fewer layers than the configuration (reported)")
-    ap.add_argument("--batch", type=int, default=8)
-    ap.add_argument("--prompt", type=int, default=2048)
-    ap.add_argument("--context", type=int, default=4096)
-    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
-    ap.add_argument("--page-size", type=int, default=16)
-    ap.add_argument("--points", default="1,64", help="other batch sizes to time (comma separated, empty for none)")
-    ap.add_argument("--execution", default="graph", choices=["graph", "eager"])
-    ap.add_argument("--overlap", type=int, default=1, choices=[0, 1],
-                    help="1: picked tokens stay on the device and a step is launched before the tokens of the one "
-                         "before are read, as the scheduler's overlapped ticks do; 0: every step waits for its tokens")
-    ap.add_argument("--workload", default="decode", choices=["decode", "serving"],
-                    help="decode: fixed batch after whole prompts (the default, timed per step); serving: --requests "
-                         "requests with prompts of 128..--prompt tokens and --new-tokens each through the scheduler")
-    ap.add_argument("--requests", type=int, default=64)
-    ap.add_argument("--new-tokens", type=int, default=256)
-    ap.add_argument("--token-budget", type=int, default=2112, help="serving: rows a step (a whole prompt beside 64 decoded tokens)")
-    ap.add_argument("--prefill-chunk", type=int, default=2048)
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print(f"bench.py measures one GPU only; --gpus {args.gpus} is not run")
-        return 2
+def sizes_of(config):
+    c = config
+    return (c.num_hidden_layers, c.hidden_size, c.head_dim, c.num_attention_heads, c.num_key_value_heads,
+            c.intermediate_size, c.vocab_size)
 
+
+def measure(model, args, batches, prompt, context, steps, warmup, repeats):
+    """Decode steps of every batch size in `batches` after whole prompts of `prompt` tokens, and the prompt steps
+    themselves.  Every batch is timed `repeats` times, `steps` decode steps each between synchronisations; the
+    median repeat counts.  Returns {batch: {...}}, the prompt step's median seconds and its flops."""
+    import statistics
     import numpy as np
     import torch
-    from runtime.config import preset
-    from runtime.engine import ModelRunner, StepEntry, load_model, write_random_model
+    from runtime.engine import ModelRunner, StepEntry
     from runtime.sampling import Sampler
-
-    raw = preset(args.model)
-    full_layers = raw["num_hidden_layers"]
-    if args.layers:
-        raw["num_hidden_layers"] = args.layers
-    raw["max_position_embeddings"] = max(raw["max_position_embeddings"], args.context)
-    folder = tempfile.mkdtemp(prefix="bench-model-")
-    write_random_model(folder, raw, seed=0, dtype="bfloat16")
-    model = load_model(folder, dtype=args.dtype)
     c = model.config
+    L, H, D, nh, nkv, I, V = sizes_of(c)
     itemsize = 2 if args.dtype == "bfloat16" else 4
     sampler = Sampler()
     rng = np.random.default_rng(0)
-    batches = [args.batch] + [int(b) for b in args.points.split(",") if b]
-    need_tokens = max(batches) * args.context
-    if args.workload == "serving":
-        return serving(args, model, full_layers)
-    runner = ModelRunner(model, n_pages=-(-need_tokens // args.page_size), page_size=args.page_size,
+    runner = ModelRunner(model, n_pages=-(-max(batches) * context // args.page_size), page_size=args.page_size,
                          max_requests=max(batches), execution=args.execution)
-
     # bytes a decode step has to read: every weight it uses once, and the cache of the live requests
-    L, H, D, nh, nkv, I, V = (c.num_hidden_layers, c.hidden_size, c.head_dim, c.num_attention_heads,
-                              c.num_key_value_heads, c.intermediate_size, c.vocab_size)
     layer_params = H * (nh + 2 * nkv) * D + nh * D * H + 3 * H * I + 2 * H
-    weight_bytes = (L * layer_params + V * H * (1 if c.tie_word_embeddings else 1) + H) * itemsize
+    weight_bytes = (L * layer_params + V * H + H) * itemsize     # (a tied head reads the embedding matrix; the gather reads rows)
     kv_bytes_per_token = L * 2 * nkv * D * itemsize
-
-    def prefill_flops(T):
-        gemm = 2 * T * L * (layer_params - 2 * H)
-        attn = L * nh * 4 * D * T * (T + 1) / 2
-        head = 2 * V * H  # one wanted row
-        return gemm + attn + head
+    prefill_flops = 2 * prompt * L * (layer_params - 2 * H) + L * nh * 4 * D * prompt * (prompt + 1) / 2 + 2 * V * H
+    prefill_times = []
 
     def timed_prefill(key, tokens):
         runner.create(key)
@@ -91,18 +53,15 @@ def main():
         logits = runner.step([StepEntry(key, tokens, [len(tokens) - 1])])
         first = sampler.pick(logits, [(0.0, 0, 0)])[0]
         torch.cuda.synchronize()
-        return first, time.perf_counter() - t0
+        prefill_times.append(time.perf_counter() - t0)
+        return first
 
-    def decode_run(batch, steps, warmup):
+    out = {}
+    for batch in batches:
         keys = [f"b{batch}-{i}" for i in range(batch)]
-        last, prefill_times = [], []
-        for key in keys:
-            tokens = rng.integers(0, V, size=args.prompt, dtype=np.int32)   # token ids as they come from a tokenizer: an array
-            first, dt = timed_prefill(key, tokens)
-            last.append(first)
-            prefill_times.append(dt)
+        # token ids as they come from a tokenizer: an array
+        last = [timed_prefill(key, rng.integers(0, V, size=prompt, dtype=np.int32)) for key in keys]
         params = [(0.0, 0, 0)] * batch
-
         unread = None
 
         def one():
@@ -122,38 +81,112 @@ def main():
 
         for _ in range(warmup):
             one()
-        torch.cuda.synchronize()
-        ctx0 = runner.length(keys[0])
-        t0 = time.perf_counter()
-        for _ in range(steps):
-            one()
+        timings = []
+        for _ in range(repeats):
+            torch.cuda.synchronize()
+            ctx0 = runner.length(keys[0])
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                one()
+            torch.cuda.synchronize()      # (overlapped: the tokens of the last step are read by the next repeat's first)
+            timings.append((time.perf_counter() - t0, ctx0 + steps / 2))
         if unread is not None:
-            last = unread.tokens()
-        torch.cuda.synchronize()
-        elapsed = time.perf_counter() - t0
-        ctx_mid = ctx0 + steps / 2
+            last, unread = unread.tokens(), None
         for key in keys:
             runner.release(key)
-        return elapsed, ctx_mid, prefill_times
+        elapsed, ctx_mid = sorted(timings)[len(timings) // 2]
+        step_bytes = weight_bytes + batch * ctx_mid * kv_bytes_per_token
+        out[batch] = {"ms_per_step": elapsed / steps * 1e3, "tokens_per_s": batch * steps / elapsed,
+                      "gbps": step_bytes / (elapsed / steps) / 1e9, "ms_all": [round(t / steps * 1e3, 4) for t, _ in timings]}
+    # the prompt step: the median of all timed ones but the very first (which pays one-time set-up)
+    pf = statistics.median(prefill_times[1:] if len(prefill_times) > 1 else prefill_times)
+    del runner
+    return out, pf, prefill_flops
 
-    steps = min(args.steps, args.context - args.prompt - args.warmup - 1)
-    results = {}
-    for batch in batches:
-        elapsed, ctx_mid, prefill_times = decode_run(batch, steps, args.warmup)
-        results[batch] = (elapsed, ctx_mid, prefill_times)
-    elapsed, ctx_mid, prefill_times = results[args.batch]
-    ms_per_step = elapsed / steps * 1e3
-    value = args.batch * steps / elapsed
-    step_bytes = weight_bytes + args.batch * ctx_mid * kv_bytes_per_token
-    achieved = step_bytes / (elapsed / steps) / 1e9
-    # prefill: the best of the timed prompt steps after the first (the first pays one-time set-up)
-    pf = min(prefill_times[1:]) if len(prefill_times) > 1 else prefill_times[0]
+
+def copy_bandwidth():
+    """GB/s of a plain device-to-device copy of 1 GiB (bytes read plus bytes written), the median of five: what
+    this GPU's memory gives a kernel that does nothing else, beside the published peak."""
+    import statistics
+    import torch
+    n = 1 << 30
+    a = torch.empty(n, dtype=torch.uint8, device="cuda"); b = torch.empty_like(a)
+    a.zero_(); b.copy_(a)
+    times = []
+    for _ in range(5):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        b.copy_(a)
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t0)
+    return 2 * n / statistics.median(times) / 1e9
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--repeats", type=int, default=3, help="timed repeats of --steps decode steps; the median counts")
+    ap.add_argument("--model", default="smollm2-135m")
+    ap.add_argument("--layers", type=int, default=None, help="fewer layers than the configuration (reported)")
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--prompt", type=int, default=2048)
+    ap.add_argument("--context", type=int, default=4096)
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--page-size", type=int, default=16)
+    ap.add_argument("--points", default="1,64", help="other batch sizes to time (comma separated, empty for none)")
+    ap.add_argument("--sizes", default="smollm2-1.7b:8:4096,llama-3-8b:8:8192",
+                    help="further layer sizes, measured with fewer layers than their configurations have: "
+                         "preset:layers:context, comma separated (empty for none); batches 1, 8 and 64 and a prompt step each")
+    ap.add_argument("--execution", default="graph", choices=["graph", "eager"])
+    ap.add_argument("--overlap", type=int, default=1, choices=[0, 1],
+                    help="1: picked tokens stay on the device and a step is launched before the tokens of the one "
+                         "before are read, as the scheduler's overlapped ticks do; 0: every step waits for its tokens")
+    ap.add_argument("--workload", default="decode", choices=["decode", "serving"],
+                    help="decode: fixed batch after whole prompts (the default, timed per step); serving: --requests "
+                         "requests with prompts of 128..--prompt tokens and --new-tokens each through the scheduler")
+    ap.add_argument("--requests", type=int, default=64)
+    ap.add_argument("--new-tokens", type=int, default=256)
+    ap.add_argument("--token-budget", type=int, default=2112, help="serving: rows a step (a whole prompt beside 64 decoded tokens)")
+    ap.add_argument("--prefill-chunk", type=int, default=2048)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU only; --gpus {args.gpus} is not run")
+        return 2
+
+    import torch
+    from runtime.config import preset
+    from runtime.engine import load_model, random_model, write_random_model
+
+    raw = preset(args.model)
+    full_layers = raw["num_hidden_layers"]
+    if args.layers:
+        raw["num_hidden_layers"] = args.layers
+    raw["max_position_embeddings"] = max(raw["max_position_embeddings"], args.context)
+    folder = tempfile.mkdtemp(prefix="bench-model-")
+    write_random_model(folder, raw, seed=0, dtype="bfloat16")
+    model = load_model(folder, dtype=args.dtype)
+    c = model.config
+    if args.workload == "serving":
+        return serving(args, model, full_layers)
+    batches = [args.batch] + [int(b) for b in args.points.split(",") if b]
+    repeats = max(1, args.repeats)
+
+    def steps_for(context, prompt):
+        return max(1, min(args.steps, (context - prompt - args.warmup - 1) // repeats))
+
+    steps = steps_for(args.context, args.prompt)
+    results, pf, pf_flops = measure(model, args, batches, args.prompt, args.context, steps, args.warmup, repeats)
+    L, H, D, nh, nkv, I, V = sizes_of(c)
+    main_r = results[args.batch]
     peak = PEAK_TFLOPS["bf16" if args.dtype == "bfloat16" else "fp32"] * 1e12
-    points = {f"decode_b{b}": round(b * steps / results[b][0], 1) for b in batches if b != args.batch}
+    copy_gbps = copy_bandwidth()
+    points = {f"decode_b{b}": round(results[b]["tokens_per_s"], 1) for b in batches if b != args.batch}
     line = {
         "metric": f"decode tokens/s, {args.model} layer sizes, batch {args.batch}, {args.prompt}-token prompts in a {args.context} context",
-        "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "value": round(main_r["tokens_per_s"], 1), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": args.warmup,
+        "ms_per_step": round(main_r["ms_per_step"], 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic (random weights N(0,0.02), uniform-random token ids)",
         "config": {"model": args.model, "global_batch": args.batch, "seq_len": args.context, "prompt_len": args.prompt,
                    "parallelism": "single-gpu", "layers": L, "layers_of_configuration": full_layers, "hidden": H,
@@ -161,12 +194,39 @@ def main():
                    "rope_theta": c.rope_theta, "rms_norm_eps": c.rms_norm_eps, "tied_head": c.tie_word_embeddings,
                    "page_size": args.page_size, "execution": args.execution + (", steps overlapped" if args.overlap else "")},
         "prefill": {"value": round(args.prompt / pf, 1), "tokens": args.prompt, "ms": round(pf * 1e3, 3),
-                    "frac": round(prefill_flops(args.prompt) / pf / peak, 5)},
-        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_GBPS, 5)},
+                    "frac": round(pf_flops / pf / peak, 5)},
+        "roofline": {"bound": "hbm", "achieved": round(main_r["gbps"], 1), "peak": HBM_GBPS, "unit": "GB/s",
+                     "frac": round(main_r["gbps"] / HBM_GBPS, 5), "measured_copy": round(copy_gbps, 1)},
         "points": points,
+        "points_roofline_frac": {f"decode_b{b}": round(results[b]["gbps"] / HBM_GBPS, 5) for b in batches if b != args.batch},
+        "method": {"repeats": repeats, "statistic": "median", "ms_per_step_of_repeats": main_r["ms_all"], "clock": "host, synchronised"},
         "reference_b1_tokens_per_s": REFERENCE_B1_TOKS,
     }
+    # further layer sizes, with fewer layers than their configurations have (both numbers named): random weights drawn
+    # on the device, batches 1, 8 and 64 after 2,048-token prompts, and the prompt step
+    del model
+    sizes = {}
+    for item in [x for x in args.sizes.split(",") if x]:
+        name, layers, context = item.split(":")
+        layers, context = int(layers), int(context)
+        raw = preset(name)
+        of_configuration = raw["num_hidden_layers"]
+        raw["num_hidden_layers"] = min(layers, of_configuration)
+        raw["max_position_embeddings"] = max(raw["max_position_embeddings"], context)
+        torch.cuda.empty_cache()
+        other = random_model(raw, seed=0, dtype=args.dtype)
+        n = steps_for(context, args.prompt)
+        r, pf2, flops2 = measure(other, args, [1, 8, 64], args.prompt, context, n, args.warmup, repeats)
+        sizes[name] = {"layers": raw["num_hidden_layers"], "layers_of_configuration": of_configuration, "context": context,
+                       "prompt_len": args.prompt, "steps": n,
+                       **{f"decode_b{b}": round(r[b]["tokens_per_s"], 1) for b in r},
+                       **{f"decode_b{b}_ms": round(r[b]["ms_per_step"], 4) for b in r},
+                       **{f"decode_b{b}_hbm_frac": round(r[b]["gbps"] / HBM_GBPS, 5) for b in r},
+                       "prefill_tokens_per_s": round(args.prompt / pf2, 1), "prefill_ms": round(pf2 * 1e3, 3),
+                       "prefill_frac": round(flops2 / pf2 / peak, 5)}
+        del other
+    if sizes:
+        line["sizes"] = sizes
     print(json.dumps(line))
     return 0
 

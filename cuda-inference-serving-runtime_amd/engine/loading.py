@@ -47,3 +47,24 @@ def write_random_model(folder, config, seed, dtype="bfloat16", std=None):
     _, typed, model = build_from_config_dict(raw)
     return write_model_folder(folder, typed.to_dict() if hasattr(typed, "to_dict") else raw,
                               model.tensor_specs(), seed, parse_dtype(dtype), **({} if std is None else {"std": std}))
+
+
+def random_model(config, seed=0, dtype="bfloat16", device="cuda:0", std=0.02):
+    """The model of `config` (a config.json dict or the name of a preset) with random weights drawn on the device:
+    matrices N(0, std), norm weights 1 + N(0, std), bound through the model's own declarations, without a folder.
+    For measurements at sizes whose files would take minutes to write; the draws are not those of
+    write_random_model (another generator), so results are not comparable token by token."""
+    dtype = parse_dtype(dtype)
+    raw = preset(config) if isinstance(config, str) else dict(config)
+    _, _, model = build_from_config_dict(raw)
+    generator = torch.Generator(device=device).manual_seed(seed)
+    tensors = {}
+    for spec in sorted(model.tensor_specs(), key=lambda s: s.name):
+        if spec.integer:
+            raise ValueError(f"{spec.name}: integer tables have no random initialisation")
+        values = torch.randn(spec.shape, generator=generator, device=device, dtype=torch.float32) * std
+        if spec.init == "one_plus_normal":
+            values += 1.0
+        tensors[spec.name] = values.to(torch.bfloat16 if dtype == torch.bfloat16 else torch.float32)
+    model.bind(tensors, dtype, torch.device(device))
+    return model

@@ -26,3 +26,9 @@ int cisr_skinny_launch_m1(const SkinnyArgs& a, int blocks, bool norm, int epi, i
 int cisr_skinny_launch_m2(const SkinnyArgs& a, int blocks, bool norm, int epi, int out_dtype, hipStream_t stream);
 int cisr_skinny_launch_m3(const SkinnyArgs& a, int blocks, bool norm, int epi, int out_dtype, hipStream_t stream);
 int cisr_skinny_launch_m4(const SkinnyArgs& a, int blocks, bool norm, int epi, int out_dtype, hipStream_t stream);
+
+// The narrow kernels (gemm_narrow.inc): four output columns a block, at most 16 rows of A, in tiles of four rows;
+// one function per number of tiles.  `units` = blocks: ceil(N / 4), or with EPI_ROPE (heads + 2 kv_heads) head_dim / 4.
+int cisr_narrow_launch_t1(const SkinnyArgs& a, int units, bool norm, int epi, int out_dtype, hipStream_t stream);
+int cisr_narrow_launch_t2(const SkinnyArgs& a, int units, bool norm, int epi, int out_dtype, hipStream_t stream);
+int cisr_narrow_launch_t4(const SkinnyArgs& a, int units, bool norm, int epi, int out_dtype, hipStream_t stream);

@@ -1,6 +1,7 @@
 // Entry points of the skinny (M <= 64) bf16 matrix products; the kernels live in gemm_skinny.inc,
 // compiled once per number of 16-row tiles (gemm_skinny_m1..m4.hip).
 #include "gemm_skinny.h"
+#include <stdlib.h>
 
 static int launch_rows(const SkinnyArgs& a, int blocks, bool norm, int epi, int out_dtype, hipStream_t stream) {
     if (a.M <= 16) return cisr_skinny_launch_m1(a, blocks, norm, epi, out_dtype, stream);
@@ -10,6 +11,24 @@ static int launch_rows(const SkinnyArgs& a, int blocks, bool norm, int epi, int 
 }
 
 static bool aligned16(const void* p) { return ((uintptr_t)p) % 16 == 0; }
+
+// Few rows against small weights with a narrow output: a block for every 16 columns would leave most compute
+// units idle, so the narrow kernels take over (a block for every 4 columns).  Measured on an MI355X in captured
+// chains: the down projection of the 135M sizes (8 rows, 576 x 1536) 4.3 us with 36 blocks of 16 columns.
+// CISR_NARROW=0 switches them off.
+static bool narrow_wanted(int M, int N, int K, bool norm) {
+    static const int enabled = getenv("CISR_NARROW") ? atoi(getenv("CISR_NARROW")) : 1;
+    const int rows = M <= 4 ? 4 : M <= 8 ? 8 : 16;
+    // with the norm fused, a block's rows must fit LDS and be one batch of loads: inner sizes up to 1024, 640, 576
+    if (norm && ((size_t)rows * (K + 8) * 2 > 40 * 1024 || K > (rows == 4 ? 1024 : rows == 8 ? 640 : 576))) return false;
+    return enabled && M <= 16 && (N + 15) / 16 < 256 && (long long)N * K * 2 <= (4LL << 20);
+}
+
+static int launch_narrow(const SkinnyArgs& a, int units, bool norm, int epi, int out_dtype, hipStream_t stream) {
+    if (a.M <= 4) return cisr_narrow_launch_t1(a, units, norm, epi, out_dtype, stream);
+    if (a.M <= 8) return cisr_narrow_launch_t2(a, units, norm, epi, out_dtype, stream);
+    return cisr_narrow_launch_t4(a, units, norm, epi, out_dtype, stream);
+}
 
 // Plain / residual / SwiGLU forms.  A is bf16 [M, K], or with norm_w != null the float residual
 // [*, K] (rows picked by `rows` if given).  dual_off > 0 selects SwiGLU over two blocks of N rows of W.
@@ -23,8 +42,10 @@ extern "C" int cisr_gemm_skinny_bf16(const void* A, int lda, const void* W, int 
     SkinnyArgs a = {};
     a.A = A; a.lda = lda; a.W = (const bf16_t*)W; a.ldw = ldw; a.C = C; a.ldc = ldc; a.R = R; a.ldr = ldr;
     a.M = M; a.N = N; a.K = K; a.dual_off = dual_off; a.norm_w = norm_w; a.eps = eps; a.rows = rows;
+    const int epi = dual_off > 0 ? EPI_SWIGLU : EPI_STORE;
+    if (narrow_wanted(M, dual_off > 0 ? 2 * N : N, K, norm_w != nullptr)) return launch_narrow(a, (N + 3) / 4, norm_w != nullptr, epi, out_dtype, stream);
     const int blocks = (N + 15) / 16;
-    return launch_rows(a, blocks, norm_w != nullptr, dual_off > 0 ? EPI_SWIGLU : EPI_STORE, out_dtype, stream);
+    return launch_rows(a, blocks, norm_w != nullptr, epi, out_dtype, stream);
 }
 
 // The fused q/k/v projection of a decode step: RMSNorm of the float residual (norm_w may be null: A is
@@ -44,6 +65,7 @@ extern "C" int cisr_qkv_rope_skinny(const void* A, int lda, const void* W, int l
     a.positions = positions; a.slots = slots; a.cos_tab = cos_tab; a.sin_tab = sin_tab;
     a.kcache = (bf16_t*)kcache; a.vcache = (bf16_t*)vcache; a.heads = heads; a.kv_heads = kv_heads;
     a.head_dim = head_dim; a.page_size = page_size; a.max_pos = max_pos;
+    if (narrow_wanted(M, a.N, K, norm_w != nullptr)) return launch_narrow(a, a.N / 4, norm_w != nullptr, EPI_ROPE, DT_BF16, stream);
     const int blocks = (heads + 2 * kv_heads) * (head_dim / 16);
     return launch_rows(a, blocks, norm_w != nullptr, EPI_ROPE, DT_BF16, stream);
 }

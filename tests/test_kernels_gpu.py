@@ -556,11 +556,16 @@ def test_gemm_skinny_and_fused_swiglu(ops):
     gq = torch.from_numpy(f64(a) @ f64(w).T).to(torch.bfloat16).double().numpy()
     two = ops.gemm_swiglu(a, w, torch.empty(70, 90, dtype=torch.bfloat16, device=DEV), scratch=torch.empty(70, 180, dtype=torch.bfloat16, device=DEV))
     np.testing.assert_allclose(f64(two), P.swiglu(gq[:, :90], gq[:, 90:]), rtol=2e-2, atol=2e-2)
-    # a row's result does not depend on how many rows are beside it
+    # a row's result does not depend on how many rows are beside it: bit for bit among the batches that one kernel
+    # takes (up to 16 rows of a narrow output: four columns a block; more: sixteen), to rounding between the two
     a, w = rnd(64, 576, dtype=torch.bfloat16, seed=6), rnd(300, 576, dtype=torch.bfloat16, seed=7)
     full = ops.gemm(a, w, torch.empty(64, 300, device=DEV))
-    for m in (1, 5, 16, 17, 48):
+    few = ops.gemm(a[:16].contiguous(), w, torch.empty(16, 300, device=DEV))
+    for m in (1, 4, 5, 8, 9, 16):
+        assert torch.equal(ops.gemm(a[:m].contiguous(), w, torch.empty(m, 300, device=DEV)), few[:m])
+    for m in (17, 48):
         assert torch.equal(ops.gemm(a[:m].contiguous(), w, torch.empty(m, 300, device=DEV)), full[:m])
+    torch.testing.assert_close(few, full[:16], rtol=1e-5, atol=1e-4)
     # a wide output with more than 32 rows runs with eight waves a block instead of sixteen, which changes the
     # order of the sum over K: bit for bit among such batches, and to rounding against the smaller ones
     a, w = rnd(64, 200, dtype=torch.bfloat16, seed=8), rnd(6400, 200, dtype=torch.bfloat16, seed=9)
@@ -570,6 +575,42 @@ def test_gemm_skinny_and_fused_swiglu(ops):
     assert torch.equal(ops.gemm(a[:40].contiguous(), w, torch.empty(40, 6400, device=DEV)), large[:40])
     torch.testing.assert_close(small, large[:32], rtol=1e-5, atol=1e-4)
     np.testing.assert_allclose(f64(large), f64(a) @ f64(w).T, rtol=1e-4, atol=1e-4 * math.sqrt(200))
+
+
+@pytest.mark.parametrize("M", [1, 3, 4, 5, 8, 9, 13, 16])
+def test_gemm_narrow_outputs_of_few_rows(ops, M):
+    """At most 16 rows against small weights with a narrow output run four output columns a block (four chunks of
+    the inner size side by side in one matrix instruction): every epilogue and the fused norm, widths that are no
+    multiple of 4, inner sizes that are no multiple of the 128-wide step or shorter than one."""
+    for N, K in [(4, 8), (6, 40), (50, 128), (576, 576), (576, 1536), (1003, 136), (37, 4096), (100, 72)]:
+        a, w, r = rnd(M, K, dtype=torch.bfloat16, seed=1), rnd(N, K, dtype=torch.bfloat16, seed=2), rnd(M, N, seed=3)
+        want = f64(a) @ f64(w).T
+        tol_f = dict(rtol=1e-4, atol=1e-4 * math.sqrt(K))
+        np.testing.assert_allclose(f64(ops.gemm(a, w, torch.empty(M, N, device=DEV))), want, **tol_f)
+        np.testing.assert_allclose(f64(ops.gemm(a, w, torch.empty(M, N, dtype=torch.bfloat16, device=DEV))), want, rtol=1e-2, atol=1e-2 * math.sqrt(K))
+        out = r.clone(); ops.gemm(a, w, out, residual=out)
+        np.testing.assert_allclose(f64(out), want + f64(r), **tol_f)
+        # rows of a larger buffer (a stride that is not the width)
+        big = rnd(M, K + 24, dtype=torch.bfloat16, seed=4)
+        np.testing.assert_allclose(f64(ops.gemm(big[:, :K], w, torch.empty(M, N, device=DEV))), f64(big[:, :K]) @ f64(w).T, **tol_f)
+    for I, K, eps in [(6, 40, 1e-5), (172, 64, 1e-6), (1536, 576, 1e-5), (90, 200, 1e-2)]:
+        x, nw = rnd(M + 2, K, seed=5, scale=2.0), 1 + 0.1 * rnd(K, seed=6)
+        w = rnd(2 * I, K, dtype=torch.bfloat16, seed=7, scale=0.2)
+        h = P.rmsnorm(f64(x), f64(nw), eps)
+        gu = h @ f64(w).T
+        want = P.swiglu(gu[:, :I], gu[:, I:])
+        got = ops.gemm_swiglu(x[:M], w, torch.empty(M, I, dtype=torch.bfloat16, device=DEV), norm=(nw, eps, None))
+        assert np.abs(f64(got) - want[:M]).max() < 2e-2 * max(np.abs(want).max(), 1e-3)
+        hb = torch.from_numpy(h[:M]).to(torch.bfloat16).to(DEV)
+        gq = torch.from_numpy(f64(hb) @ f64(w).T).to(torch.bfloat16).double().numpy()
+        got = ops.gemm_swiglu(hb, w, torch.empty(M, I, dtype=torch.bfloat16, device=DEV))
+        np.testing.assert_allclose(f64(got), P.swiglu(gq[:, :I], gq[:, I:]), rtol=2e-2, atol=2e-2)
+        # the fused norm with gathered rows, float output
+        rows = torch.tensor([(M + 1 - i) % (M + 2) for i in range(M)], dtype=torch.int32, device=DEV)
+        wn_ = w[:I].contiguous()
+        got = ops.gemm_normed(x, (nw, eps, rows), wn_, torch.empty(M, I, device=DEV))
+        ref = h[rows.cpu().numpy()] @ f64(wn_).T
+        assert np.abs(f64(got) - ref).max() < 6e-3 * np.abs(ref).max()
 
 
 def test_fused_norm_products(ops):
@@ -600,44 +641,46 @@ def test_fused_norm_products(ops):
     assert np.abs(f64(got) - want).max() < 2e-2 * np.abs(want).max()
 
 
-@pytest.mark.parametrize("heads, kv_heads, dim, theta, normed", [(4, 2, 16, 1e4, True), (9, 3, 64, 1e5, True), (2, 1, 128, 5e5, False), (3, 3, 48, 1e4, True)])
+@pytest.mark.parametrize("heads, kv_heads, dim, theta, normed", [(4, 2, 16, 1e4, True), (9, 3, 64, 1e5, True), (2, 1, 128, 5e5, False), (3, 3, 48, 1e4, True),
+                                                                 (9, 3, 64, 1e5, False), (5, 1, 32, 1e4, True)])
 def test_fused_projection_rotary_scatter(ops, heads, kv_heads, dim, theta, normed):
     from runtime.parts import RotaryEmbedding
     rope = RotaryEmbedding(dim, theta, 700); rope.prepare(DEV, torch.bfloat16)
     cos, sin = rope.tables()
-    M, K, P_, pages = 5, 72, 4, 8
-    pos = [0, 17, 500, 699, 3]
-    slots = [5, 0, 22, -1, 9]
-    x = rnd(M, K, seed=1, scale=1.5)
-    nw = 1 + 0.1 * rnd(K, seed=2)
-    w = rnd((heads + 2 * kv_heads) * dim, K, dtype=torch.bfloat16, seed=3, scale=0.2)
-    h = P.rmsnorm(f64(x), f64(nw), 1e-5) if normed else f64(x.bfloat16())
-    ref = h @ f64(w).T
-    q_ref = P.rope(ref[:, :heads * dim].reshape(M, heads, dim), pos, theta)
-    k_ref = P.rope(ref[:, heads * dim:(heads + kv_heads) * dim].reshape(M, kv_heads, dim), pos, theta)
-    v_ref = ref[:, (heads + kv_heads) * dim:].reshape(M, kv_heads, dim)
-    kc = torch.full((pages, kv_heads, P_, dim), 7.0, dtype=torch.bfloat16, device=DEV)
-    vc = torch.full((pages, kv_heads, dim, P_), 7.0, dtype=torch.bfloat16, device=DEV)
-    q = torch.empty(M, heads * dim, dtype=torch.bfloat16, device=DEV)
-    a = x if normed else x.bfloat16()
-    ops.qkv_rope(a, w, q, torch.tensor(pos, dtype=torch.int32, device=DEV), torch.tensor(slots, dtype=torch.int32, device=DEV),
-                 cos, sin, kc, vc, heads, kv_heads, dim, P_, norm=(nw, 1e-5) if normed else None)
-    tol = dict(rtol=2e-2, atol=2e-2 * np.abs(ref).max())
-    np.testing.assert_allclose(f64(q).reshape(M, heads, dim), q_ref, **tol)
-    kc64, vc64 = f64(kc), f64(vc)
-    for t, s_ in enumerate(slots):
-        if s_ < 0:
-            continue
-        np.testing.assert_allclose(kc64[s_ // P_, :, s_ % P_], k_ref[t], **tol)
-        np.testing.assert_allclose(vc64[s_ // P_, :, :, s_ % P_], v_ref[t], **tol)
-    untouched = [s_ for s_ in range(pages * P_) if s_ not in slots]
-    assert all((kc64[s_ // P_, :, s_ % P_] == 7).all() and (vc64[s_ // P_, :, :, s_ % P_] == 7).all() for s_ in untouched)
-    # q only (a layer that reads another layer's cache)
-    wq = w[:heads * dim].contiguous()
-    q2 = torch.empty_like(q)
-    ops.qkv_rope(a, wq, q2, torch.tensor(pos, dtype=torch.int32, device=DEV), None, cos, sin, None, None, heads, kv_heads, dim, P_,
-                 norm=(nw, 1e-5) if normed else None)
-    assert torch.equal(q, q2)
+    K, P_, pages = 72, 4, 16
+    for M in (1, 5, 12, 40):     # one, two and four tiles of the narrow kernels, and the sixteen-column kernel
+        pos = ([0, 17, 500, 699, 3] + [(53 * i) % 700 for i in range(5, M)])[:M]
+        slots = ([5, 0, 22, -1, 9] + [63 - i for i in range(5, M)])[:M]
+        x = rnd(M, K, seed=1, scale=1.5)
+        nw = 1 + 0.1 * rnd(K, seed=2)
+        w = rnd((heads + 2 * kv_heads) * dim, K, dtype=torch.bfloat16, seed=3, scale=0.2)
+        h = P.rmsnorm(f64(x), f64(nw), 1e-5) if normed else f64(x.bfloat16())
+        ref = h @ f64(w).T
+        q_ref = P.rope(ref[:, :heads * dim].reshape(M, heads, dim), pos, theta)
+        k_ref = P.rope(ref[:, heads * dim:(heads + kv_heads) * dim].reshape(M, kv_heads, dim), pos, theta)
+        v_ref = ref[:, (heads + kv_heads) * dim:].reshape(M, kv_heads, dim)
+        kc = torch.full((pages, kv_heads, P_, dim), 7.0, dtype=torch.bfloat16, device=DEV)
+        vc = torch.full((pages, kv_heads, dim, P_), 7.0, dtype=torch.bfloat16, device=DEV)
+        q = torch.empty(M, heads * dim, dtype=torch.bfloat16, device=DEV)
+        a = x if normed else x.bfloat16()
+        ops.qkv_rope(a, w, q, torch.tensor(pos, dtype=torch.int32, device=DEV), torch.tensor(slots, dtype=torch.int32, device=DEV),
+                     cos, sin, kc, vc, heads, kv_heads, dim, P_, norm=(nw, 1e-5) if normed else None)
+        tol = dict(rtol=2e-2, atol=2e-2 * np.abs(ref).max())
+        np.testing.assert_allclose(f64(q).reshape(M, heads, dim), q_ref, **tol, err_msg=f"M={M}")
+        kc64, vc64 = f64(kc), f64(vc)
+        for t, s_ in enumerate(slots):
+            if s_ < 0:
+                continue
+            np.testing.assert_allclose(kc64[s_ // P_, :, s_ % P_], k_ref[t], **tol, err_msg=f"M={M}")
+            np.testing.assert_allclose(vc64[s_ // P_, :, :, s_ % P_], v_ref[t], **tol, err_msg=f"M={M}")
+        untouched = [s_ for s_ in range(pages * P_) if s_ not in slots]
+        assert all((kc64[s_ // P_, :, s_ % P_] == 7).all() and (vc64[s_ // P_, :, :, s_ % P_] == 7).all() for s_ in untouched)
+        # q only (a layer that reads another layer's cache)
+        wq = w[:heads * dim].contiguous()
+        q2 = torch.empty_like(q)
+        ops.qkv_rope(a, wq, q2, torch.tensor(pos, dtype=torch.int32, device=DEV), None, cos, sin, None, None, heads, kv_heads, dim, P_,
+                     norm=(nw, 1e-5) if normed else None)
+        assert torch.equal(q, q2), f"M={M}"
 
 
 @pytest.mark.parametrize("heads, kv_heads, dim, M, K", [(4, 2, 16, 5, 72), (9, 3, 64, 8, 4104), (2, 1, 128, 20, 2056), (3, 3, 48, 40, 520),

@@ -18,6 +18,10 @@ struct SkinnyArgs {
     // EPI_ROPE
     const int* positions; const int* slots; const float* cos_tab; const float* sin_tab;
     bf16_t* kcache; bf16_t* vcache; int heads, kv_heads, head_dim, page_size, max_pos;
+    // merge prologue of the narrow kernels (A = the split decode attention's partial results, not yet merged):
+    // normalised partial outputs bf16 [M, merge_heads, splits, merge_dim], statistics float [M, merge_heads, splits, 2]
+    // (maximum in log2 units, denominator); K = merge_heads * merge_dim
+    const bf16_t* part_o; const float* part_ml; int merge_heads, merge_dim;
 };
 
 
@@ -32,3 +36,7 @@ int cisr_skinny_launch_m4(const SkinnyArgs& a, int blocks, bool norm, int epi, i
 int cisr_narrow_launch_t1(const SkinnyArgs& a, int units, bool norm, int epi, int out_dtype, hipStream_t stream);
 int cisr_narrow_launch_t2(const SkinnyArgs& a, int units, bool norm, int epi, int out_dtype, hipStream_t stream);
 int cisr_narrow_launch_t4(const SkinnyArgs& a, int units, bool norm, int epi, int out_dtype, hipStream_t stream);
+// the same with the merge prologue (2, 4 or 8 splits): float output with the residual added
+int cisr_narrow_merge_launch_t1(const SkinnyArgs& a, int units, int splits, hipStream_t stream);
+int cisr_narrow_merge_launch_t2(const SkinnyArgs& a, int units, int splits, hipStream_t stream);
+int cisr_narrow_merge_launch_t4(const SkinnyArgs& a, int units, int splits, hipStream_t stream);

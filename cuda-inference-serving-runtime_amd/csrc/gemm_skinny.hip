@@ -69,3 +69,29 @@ extern "C" int cisr_qkv_rope_skinny(const void* A, int lda, const void* W, int l
     const int blocks = (heads + 2 * kv_heads) * (head_dim / 16);
     return launch_rows(a, blocks, norm_w != nullptr, EPI_ROPE, DT_BF16, stream);
 }
+
+// The output projection of a decode step fused with the merge of split attention: A is given as the split blocks'
+// partial results (bf16 [M, heads, splits, head_dim] normalised outputs, float [M, heads, splits, 2] statistics with
+// the maximum in log2 units), C = R + merge(A) . W^T in float.  Takes what cisr_gemm_merged_ok says it takes.
+extern "C" int cisr_gemm_merged_ok(int M, int N, int heads, int head_dim, int splits) {
+    const int K = heads * head_dim, rows = M <= 4 ? 4 : M <= 8 ? 8 : 16;
+    const int batches = rows == 4 ? 2 : rows == 8 ? 3 : 5;
+    return M >= 1 && M <= 16 && head_dim % 8 == 0 && (splits == 2 || splits == 4 || splits == 8) &&
+           narrow_wanted(M, N, K, false) && (size_t)rows * (K + 8) * 2 <= 40 * 1024 && M * (K / 8) <= batches * 256;
+}
+
+extern "C" int cisr_gemm_merged_bf16(const void* part_o, const float* part_ml, int splits, int heads, int head_dim,
+                                     const void* W, int ldw, float* C, int ldc, const float* R, int ldr, int M, int N,
+                                     hipStream_t stream) {
+    if (M <= 0 || N <= 0) return 0;
+    const int K = heads * head_dim;
+    if (!cisr_gemm_merged_ok(M, N, heads, head_dim, splits) || ldw % 8 || !aligned16(W) || !aligned16(part_o) || !aligned16(part_ml))
+        return (int)hipErrorInvalidValue;
+    SkinnyArgs a = {};
+    a.W = (const bf16_t*)W; a.ldw = ldw; a.C = C; a.ldc = ldc; a.R = R; a.ldr = ldr; a.M = M; a.N = N; a.K = K;
+    a.part_o = (const bf16_t*)part_o; a.part_ml = part_ml; a.merge_heads = heads; a.merge_dim = head_dim;
+    const int units = (N + 3) / 4;
+    if (M <= 4) return cisr_narrow_merge_launch_t1(a, units, splits, stream);
+    if (M <= 8) return cisr_narrow_merge_launch_t2(a, units, splits, stream);
+    return cisr_narrow_merge_launch_t4(a, units, splits, stream);
+}

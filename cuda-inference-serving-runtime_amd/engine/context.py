@@ -125,9 +125,12 @@ class StepContext:
         if partials is not None:
             ops.add_partials(rows, partials)
 
-    def attend(self, q, q_row_stride, kcache, vcache, view, out, heads, kv_heads, head_dim, window, scale):
-        """out[r] = attention of row r's queries over its request's cache."""
-        self.runner.attention(self, q, q_row_stride, kcache, vcache, view, out, heads, kv_heads, head_dim, window, scale)
+    def attend(self, q, q_row_stride, kcache, vcache, view, out, heads, kv_heads, head_dim, window, scale, defer_merge=None):
+        """out[r] = attention of row r's queries over its request's cache.  With `defer_merge` (see
+        ModelRunner.attention) the result may come back unmerged instead: (partial outputs, statistics, splits) for
+        ops.gemm_merged, `out` untouched; None means `out` holds the result."""
+        return self.runner.attention(self, q, q_row_stride, kcache, vcache, view, out, heads, kv_heads, head_dim, window, scale,
+                                     defer_merge=defer_merge)
 
 
 class Workspace:

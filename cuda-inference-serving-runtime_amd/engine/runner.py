@@ -435,10 +435,15 @@ class ModelRunner:
         return logits[:wanted]
 
     # -- attention dispatch -------------------------------------------------------
-    def attention(self, ctx, q, q_row_stride, kcache, vcache, view, out, heads, kv_heads, head_dim, window, scale):
+    def attention(self, ctx, q, q_row_stride, kcache, vcache, view, out, heads, kv_heads, head_dim, window, scale,
+                  defer_merge=None):
         """bfloat16 with a head size in steps of 8 and pages of a power of two >= 4 run
         on the matrix cores (one block per row for decode steps, tiles of rows from a
-        task list otherwise); everything else runs the exact row-wise kernel."""
+        task list otherwise); everything else runs the exact row-wise kernel.
+
+        `defer_merge(splits) -> bool`: the caller's next product can merge the partial results of a decode step whose
+        keys are split over `splits` blocks itself (ops.gemm_merged).  Where that is so, no merge kernel runs, `out`
+        is left alone and (partial outputs bf16, statistics float, splits) is returned; otherwise None."""
         rows = out.shape[0]
         span = ctx.span_hint if not window else min(ctx.span_hint, window + 31)
         if ops.mfma_attention_supported(out.dtype, head_dim, view.page_size):
@@ -447,6 +452,17 @@ class ModelRunner:
             if ctx.decode_only:
                 blocks = rows * kv_heads * -(-group // heads_per_chunk)
                 waves, splits = self._rows_launch(blocks, span, heads_per_chunk, head_dim)
+                if splits > 1 and defer_merge is not None:
+                    # the product that follows merges 2, 4 or 8 partial results of a row while it prepares its operand
+                    # (at most 4 with more than 4 rows: it reads them all); one kernel fewer than merging here
+                    fused = next((n for n in (8, 4, 2) if n <= splits and (n <= 4 or rows <= 4) and defer_merge(n)), None)
+                    if fused is not None:
+                        workspace = (ctx.buffer("attn.part_o16", (rows * heads * fused * head_dim,), torch.bfloat16),
+                                     ctx.buffer("attn.part_ml", (rows * heads * fused * 2,), torch.float32))
+                        ops.attention_mfma(q, q_row_stride, kcache, vcache, view.tables, ctx.seg_of_row, ctx.positions, out,
+                                           heads, kv_heads, head_dim, view.page_size, window, scale, None, fused, workspace, waves,
+                                           merge=False)
+                        return workspace[0], workspace[1], fused
                 workspace = None
                 if splits > 1:
                     workspace = (ctx.buffer("attn.part_o", (rows * heads * splits * head_dim,), torch.float32),

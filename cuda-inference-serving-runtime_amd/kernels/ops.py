@@ -62,6 +62,8 @@ def _declare(h):
         "cisr_rmsnorm_partials": [p, p, i, p, p, i, i, f, i, p],
         "cisr_add_rmsnorm_bf16": [p, p, p, p, i, i, f, i, p],
         "cisr_qkv_rope_wide": [p, i, p, i, p, i, i, i, p, p, p, p, p, p, i, i, i, i, i, p, C.c_longlong, p],
+        "cisr_gemm_merged_bf16": [p, p, i, i, i, p, i, p, i, p, i, i, i, p],
+        "cisr_gemm_merged_ok": [i, i, i, i, i],
     }
     for name, args in sig.items():
         fn = getattr(h, name)
@@ -81,7 +83,7 @@ def _attention_entry(dpad):
     if fn is None:
         p, i, f = C.c_void_p, C.c_int, C.c_float
         fn = getattr(library.load_attention(dpad), f"cisr_attn_mfma_d{dpad}")
-        fn.argtypes = [p, i, p, p, p, i, p, i, p, p, p, p, p, i, i, i, i, i, f, i, i, i, p]
+        fn.argtypes = [p, i, p, p, p, i, p, i, p, p, p, p, p, i, i, i, i, i, f, i, i, i, i, p]
         fn.restype = C.c_int
         _attention_entries[dpad] = fn
     return fn
@@ -611,7 +613,7 @@ def qkv_rope(a, w, q_out, positions, slots, cos, sin, kcache, vcache, heads, kv_
 
 def attention_mfma(q, q_row_stride, kcache, vcache, tables, seg_of_row, positions, out, heads, kv_heads, dim,
                    page_size, window, scale, tasks=None, splits=1, workspace=None, waves=4, block_tiles=False,
-                   item_tiles=1, row_ids=None):
+                   item_tiles=1, row_ids=None, merge=True):
     """Matrix-core attention (bf16).  tasks int32 [n, 4] = (segment, first row, rows, 0) runs tiles of
     prompt rows: one tile of 16/GC rows a block whose waves share the keys (with item_tiles=2, head sizes up to
     64: 32/GC rows, two item tiles a wave), or with `block_tiles` (head sizes up to 128) one tile of
@@ -619,7 +621,9 @@ def attention_mfma(q, q_row_stride, kcache, vcache, tables, seg_of_row, position
     (GC = query heads per key head, at most 16); tasks None runs one block
     per row (decode) of `waves` wavefronts (4 or 8) with `splits` blocks along the keys; splits > 1 needs
     workspace = (partials float, statistics float) and a merge.  `row_ids` (int32 [n], with tasks None): only
-    the rows it lists are computed and written (negative entries are skipped): the decode rows of a mixed step."""
+    the rows it lists are computed and written (negative entries are skipped): the decode rows of a mixed step.
+    `merge` False (rows mode with splits > 1): the partial outputs are left unmerged in the workspace, whose first
+    buffer is then bfloat16, for gemm_merged; `out` is not written."""
     rows = out.shape[0]
     if not mfma_attention_supported(out.dtype, dim, page_size):
         raise KernelError(f"attention_mfma: head size {dim} / page size {page_size} / dtype {out.dtype} not supported")
@@ -654,7 +658,7 @@ def attention_mfma(q, q_row_stride, kcache, vcache, tables, seg_of_row, position
             if workspace is None:
                 raise KernelError("attention: split runs need a workspace")
             part_o, part_ml = workspace
-            po, pm = _dev(part_o, "part_o", torch.float32), _dev(part_ml, "part_ml", torch.float32)
+            po, pm = _dev(part_o, "part_o", torch.float32 if merge else torch.bfloat16), _dev(part_ml, "part_ml", torch.float32)
             if part_o.numel() < n_tasks * heads * splits * dim or part_ml.numel() < n_tasks * heads * splits * 2:
                 raise KernelError("attention: split workspace too small")
     _check(fn(q.data_ptr(), q_row_stride, _dev(kcache, "kcache", None, (pages, kv_heads, page_size, dim)),
@@ -662,9 +666,33 @@ def attention_mfma(q, q_row_stride, kcache, vcache, tables, seg_of_row, position
               tables.shape[1], tp, n_tasks, _dev(seg_of_row, "seg_of_row", torch.int32, (rows,)),
               _dev(positions, "positions", torch.int32, (rows,)), _dev(out, "out", None, (rows, heads * dim)), po, pm,
               heads, kv_heads, dim, page_size.bit_length() - 1, int(window or 0), float(scale), int(splits), mode, int(waves),
-              _stream()), "attention_mfma")
-    if mode == 1 and splits > 1:
+              int(mode == 1 and splits > 1 and not merge), _stream()), "attention_mfma")
+    if mode == 1 and splits > 1 and merge:
         _check(lib().cisr_attn_merge(po, pm, out.data_ptr(), n_tasks, heads, dim, int(splits), tp, _stream()), "attention_merge")
+    return out
+
+
+def gemm_merged_ok(m, w, heads, dim, splits):
+    """Whether gemm_merged takes m rows of `splits` partial attention results of heads x dim against the bf16 weights w."""
+    return (w.dtype == torch.bfloat16 and w.dim() == 2 and w.shape[1] == heads * dim and w.stride(1) == 1 and w.stride(0) % 8 == 0
+            and w.data_ptr() % 16 == 0 and bool(lib().cisr_gemm_merged_ok(int(m), int(w.shape[0]), int(heads), int(dim), int(splits))))
+
+
+def gemm_merged(partials, heads, dim, w, out, residual):
+    """out[M, N] = residual + merge(partials) . w^T in float: the output projection of a decode step whose attention
+    was split over `splits` blocks along the keys and left unmerged (attention_mfma with merge=False).
+    partials = (bf16 [M, heads, splits, dim] normalised partial outputs, float [M, heads, splits, 2] statistics, splits)."""
+    part_o, part_ml, splits = partials
+    m, n = out.shape
+    if not gemm_merged_ok(m, w, heads, dim, splits) or w.shape[0] != n:
+        raise KernelError("gemm_merged: shape not supported by the fused kernel")
+    if out.dtype != torch.float32 or out.stride(1) != 1 or tuple(residual.shape) != (m, n) or residual.dtype != torch.float32 or residual.stride(1) != 1:
+        raise KernelError("gemm_merged: float output and residual [M, N]")
+    if part_o.numel() < m * heads * splits * dim or part_ml.numel() < m * heads * splits * 2:
+        raise KernelError("gemm_merged: partial results too small")
+    _check(lib().cisr_gemm_merged_bf16(_dev(part_o, "part_o", torch.bfloat16), _dev(part_ml, "part_ml", torch.float32), int(splits),
+                                       int(heads), int(dim), w.data_ptr(), w.stride(0), out.data_ptr(), out.stride(0),
+                                       residual.data_ptr(), residual.stride(0), m, n, _stream()), "gemm_merged")
     return out
 
 

@@ -85,7 +85,11 @@ class PagedAttention(Mixer):
             ops.rope_scatter(q, ctx.positions, slots, cos, sin, kcache_w, vcache_w, nh, nkv, D, view.page_size,
                              interleaved=self._interleaved)
         out = ctx.buffer("attn.out", (T, nh * D), ctx.dtype)
-        ctx.attend(q, q_stride, kcache, vcache, view, out, nh, nkv, D, self.window, self.scale)
+        # a decode step of few rows may leave the partial results of its split keys to the output projection
+        unmerged = ctx.attend(q, q_stride, kcache, vcache, view, out, nh, nkv, D, self.window, self.scale,
+                              defer_merge=lambda splits: ops.gemm_merged_ok(T, self.w_out, nh, D, splits))
+        if unmerged is not None:
+            return ops.gemm_merged(unmerged, nh, D, self.w_out, residual, residual)
         return ctx.add_product(out, self.w_out, residual)
 
 

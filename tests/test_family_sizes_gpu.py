@@ -83,3 +83,41 @@ def test_a_cut_across_the_library_threshold_changes_rounding_only(family_folders
         assert_close(got, ref, "bfloat16", what=name)
     between = np.linalg.norm(runs[0] - runs[1]) / np.linalg.norm(ref)
     assert between < BF16_RMSE / 4, f"the two cuts differ by {between:.3e}"
+
+
+@pytest.mark.parametrize("execution", ["eager", "graph"])
+def test_decoding_at_a_context_whose_keys_are_split_over_blocks(family_folders, execution):
+    """From a context of about 500 keys on, a decode step of few rows splits every row's keys over blocks; at the
+    135M sizes the output projection then merges the blocks' partial results itself (no merge kernel).  Three requests
+    of very different lengths decode together (the short one's later splits see no key at all), then one alone."""
+    from runtime.engine import load_model, ModelRunner, StepEntry
+    name = "smollm2-135m"
+    folder = family_folders[name]
+    V = FAMILY[name]["vocab_size"]
+    seqs = {"long": random_tokens(11, 506, V), "mid": random_tokens(12, 310, V), "short": random_tokens(13, 20, V)}
+    model = load_model(folder, dtype="bfloat16")
+    runner = ModelRunner(model, n_pages=64, page_size=16, max_requests=4, execution=execution)
+    fed, got = {}, {k: [] for k in seqs}
+    for k, toks in seqs.items():
+        runner.create(k)
+        fed[k] = len(toks) - 12
+        runner.step([StepEntry(k, toks[:fed[k]], [])])
+    seen = []
+    real = runner.attention
+
+    def spy(*args, **kwargs):
+        out = real(*args, **kwargs)
+        seen.append(None if out is None else out[2])
+        return out
+
+    runner.attention = spy
+    for step in range(12):
+        live = [k for k in seqs if step < 8 or k == "long"]          # the last four steps: one row
+        out = runner.step([StepEntry(k, [seqs[k][fed[k]]], [0]) for k in live]).float().cpu().numpy()
+        for row, k in zip(out, live):
+            got[k].append(row); fed[k] += 1
+    assert any(n is not None and n >= 2 for n in seen), "no decode step left its partial results to the output projection"
+    for k, toks in seqs.items():
+        ref = plain_logits(folder, toks)
+        assert_close(np.stack(got[k]), ref[len(toks) - 12:len(toks) - 12 + len(got[k])], "bfloat16", what=f"request {k}")
+    runner.cache.check()

@@ -613,6 +613,59 @@ def test_gemm_narrow_outputs_of_few_rows(ops, M):
         assert np.abs(f64(got) - ref).max() < 6e-3 * np.abs(ref).max()
 
 
+@pytest.mark.parametrize("M, heads, kv_heads, dim, splits", [(1, 9, 3, 64, 8), (3, 4, 2, 16, 2), (8, 9, 3, 64, 4), (5, 6, 6, 24, 4),
+                                                             (16, 4, 1, 32, 2), (4, 9, 3, 64, 8), (13, 2, 2, 128, 4)])
+def test_output_projection_merges_split_attention_itself(ops, M, heads, kv_heads, dim, splits):
+    """Decode attention with its keys split over blocks may leave the partial results unmerged (bf16 normalised
+    outputs, float statistics); the output projection then merges them while it prepares its operand.  Against the
+    merge kernel followed by the plain product, and against a float64 merge of made-up partial results in which
+    one split of a row has no keys and one row has none at all."""
+    K, N = heads * dim, 4 * ((heads * dim // 2) // 4) + 2
+    w = rnd(N, K, dtype=torch.bfloat16, seed=2, scale=0.1)
+    assert ops.gemm_merged_ok(M, w, heads, dim, splits)
+    # made-up partial results
+    rng = np.random.default_rng(M + splits)
+    po = torch.from_numpy(rng.standard_normal((M, heads, splits, dim)).astype(np.float32)).to(torch.bfloat16).to(DEV)
+    ms = rng.standard_normal((M, heads, splits)) * 3
+    ls = rng.uniform(0.5, 40.0, (M, heads, splits))
+    ms[0, :, splits - 1], ls[0, :, splits - 1] = -np.inf, 0.0        # a split that saw no key
+    if M > 2:
+        ms[2], ls[2] = -np.inf, 0.0                                  # a row without keys (padding): zeros
+    pm = torch.from_numpy(np.stack([ms, ls], -1).astype(np.float32)).to(DEV).contiguous()
+    weights = np.where(ls > 0, np.exp2(ms - np.max(ms, -1, keepdims=True, initial=-1e30)) * ls, 0.0)
+    den = weights.sum(-1, keepdims=True)
+    merged = np.where(den > 0, (weights[..., None] * f64(po)).sum(2) / np.where(den > 0, den, 1.0), 0.0).reshape(M, K)
+    r = rnd(M, N, seed=5)
+    out = r.clone()
+    ops.gemm_merged((po, pm, splits), heads, dim, w, out, out)
+    want = f64(r) + merged @ f64(w).T
+    np.testing.assert_allclose(f64(out), want, rtol=2e-2, atol=2e-2 * np.abs(want).max())
+    assert np.isfinite(f64(out)).all()
+    # the real thing: split decode attention left unmerged, against the merge kernel and the plain product
+    lengths = [333, 40, 130, 17, 700][:max(1, min(M, 5))]
+    qt, kt, vt, tables, rows = paged_case(heads, kv_heads, dim, 16, lengths, torch.bfloat16, seed=dim + M)
+    rows = (rows * 4)[:M]
+    qt = qt[[i % qt.shape[0] for i in range(M)]].contiguous()
+    T = len(rows)
+    seg = torch.tensor([x[0] for x in rows], dtype=torch.int32, device=DEV)
+    pos = torch.tensor([x[1] for x in rows], dtype=torch.int32, device=DEV)
+    plain_out = torch.empty(T, K, dtype=torch.bfloat16, device=DEV)
+    ws32 = (torch.empty(T * heads * splits * dim, device=DEV), torch.empty(T * heads * splits * 2, device=DEV))
+    ops.attention_mfma(qt.reshape(T, K), K, kt, vt, tables, seg, pos, plain_out, heads, kv_heads, dim, 16, None, 1 / math.sqrt(dim),
+                       None, splits, ws32, 8)
+    two = r.clone(); ops.gemm(plain_out, w, two, residual=two)
+    ws16 = (torch.empty(T * heads * splits * dim, dtype=torch.bfloat16, device=DEV), torch.empty(T * heads * splits * 2, device=DEV))
+    untouched = torch.full((T, K), 3.0, dtype=torch.bfloat16, device=DEV)
+    ops.attention_mfma(qt.reshape(T, K), K, kt, vt, tables, seg, pos, untouched, heads, kv_heads, dim, 16, None, 1 / math.sqrt(dim),
+                       None, splits, ws16, 8, merge=False)
+    assert (untouched == 3.0).all()
+    one = r.clone(); ops.gemm_merged((ws16[0], ws16[1], splits), heads, dim, w, one, one)
+    scale = np.abs(f64(two) - f64(r)).max()
+    assert np.abs(f64(one) - f64(two)).max() < 2e-2 * scale       # the partial outputs are rounded to bf16 before they are merged
+    # what it refuses: more rows, other split counts
+    assert not ops.gemm_merged_ok(17, w, heads, dim, splits) and not ops.gemm_merged_ok(M, w, heads, dim, 3)
+
+
 def test_fused_norm_products(ops):
     """RMSNorm inside the product's kernel (plain, row-gathered, SwiGLU) against norm then product."""
     for M, N, K, eps in [(1, 48, 64, 1e-5), (8, 1728, 576, 1e-5), (33, 130, 200, 1e-6), (64, 100, 144, 1e-2)]:

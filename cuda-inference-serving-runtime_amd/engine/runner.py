@@ -453,9 +453,11 @@ class ModelRunner:
                 blocks = rows * kv_heads * -(-group // heads_per_chunk)
                 waves, splits = self._rows_launch(blocks, span, heads_per_chunk, head_dim)
                 if splits > 1 and defer_merge is not None:
-                    # the product that follows merges 2, 4 or 8 partial results of a row while it prepares its operand
-                    # (at most 4 with more than 4 rows: it reads them all); one kernel fewer than merging here
-                    fused = next((n for n in (8, 4, 2) if n <= splits and (n <= 4 or rows <= 4) and defer_merge(n)), None)
+                    # the product that follows merges 2, 4 or 8 partial results of a row while it prepares its operand:
+                    # one kernel fewer than merging here.  Every block of that product reads them all, so more than 8
+                    # rows bring at most 4 each.  (135M sizes, 8 rows at 2k: a step of 0.808 ms with the merge kernel,
+                    # 0.808 with 4 splits merged there, whose attention blocks are half as many, 0.784 with 8.)
+                    fused = next((n for n in (8, 4, 2) if n <= splits and (n <= 4 or rows <= 8) and defer_merge(n)), None)
                     if fused is not None:
                         workspace = (ctx.buffer("attn.part_o16", (rows * heads * fused * head_dim,), torch.bfloat16),
                                      ctx.buffer("attn.part_ml", (rows * heads * fused * 2,), torch.float32))

@@ -143,9 +143,10 @@ def main():
     ap.add_argument("--overlap", type=int, default=1, choices=[0, 1],
                     help="1: picked tokens stay on the device and a step is launched before the tokens of the one "
                          "before are read, as the scheduler's overlapped ticks do; 0: every step waits for its tokens")
-    ap.add_argument("--workload", default="decode", choices=["decode", "serving"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "serving", "floor"],
                     help="decode: fixed batch after whole prompts (the default, timed per step); serving: --requests "
-                         "requests with prompts of 128..--prompt tokens and --new-tokens each through the scheduler")
+                         "requests with prompts of 128..--prompt tokens and --new-tokens each through the scheduler; "
+                         "floor: a captured chain of kernels that do nothing (what a launch costs)")
     ap.add_argument("--requests", type=int, default=64)
     ap.add_argument("--new-tokens", type=int, default=256)
     ap.add_argument("--token-budget", type=int, default=2112, help="serving: rows a step (a whole prompt beside 64 decoded tokens)")
@@ -159,6 +160,8 @@ def main():
     from runtime.config import preset
     from runtime.engine import load_model, random_model, write_random_model
 
+    if args.workload == "floor":
+        return launch_floor(args)
     raw = preset(args.model)
     full_layers = raw["num_hidden_layers"]
     if args.layers:
@@ -228,6 +231,42 @@ def main():
     if sizes:
         line["sizes"] = sizes
     print(json.dumps(line))
+    return 0
+
+
+def launch_floor(args):
+    """Microseconds a kernel of a captured chain costs when it computes nothing: 1,000 launches of an empty kernel
+    (one block, and one block a compute unit) in one graph, replayed; the median of 20 replays.  A decode step of
+    L layers is 5 L + 5 kernels, so this times that count is the part of a step that no kernel work can remove."""
+    import statistics
+    import torch
+    from runtime.config import preset
+    from runtime.kernels import ops
+    chain = 1000
+    out = {}
+    for name, blocks in (("one_block", 1), ("block_per_cu", torch.cuda.get_device_properties(0).multi_processor_count)):
+        stream = torch.cuda.Stream()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(stream):
+            ops.idle(blocks)
+            stream.synchronize()
+            with torch.cuda.graph(graph, stream=stream):
+                for _ in range(chain):
+                    ops.idle(blocks)
+        times = []
+        for _ in range(20 + 3):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            graph.replay()
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t0)
+        out[name] = round(statistics.median(times[3:]) / chain * 1e6, 3)
+    layers = preset(args.model)["num_hidden_layers"]
+    kernels = 5 * layers + 5
+    print(json.dumps({"metric": "microseconds a kernel that does nothing costs in a captured chain", "value": out["one_block"],
+                      "unit": "us", "higher_is_better": False, "n_gpus": 1, "chain": chain, "replays": 20, "us_per_kernel": out,
+                      "kernels_of_a_decode_step": kernels, "model": args.model,
+                      "floor_ms_of_a_decode_step": round(kernels * out["one_block"] / 1e3, 4)}))
     return 0
 
 

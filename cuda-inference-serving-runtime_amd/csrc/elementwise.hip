@@ -624,3 +624,13 @@ extern "C" int cisr_f32_to_bf16(const float* x, void* y, long long n, hipStream_
     f32_to_bf16_kernel<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(x, (bf16_t*)y, (size_t)n);
     return CISR_LAUNCH_CHECK();
 }
+
+// A kernel that does nothing: what a launch costs in a chain of kernels when nothing is computed, the floor
+// under every kernel of a decode step (measured by the benchmark's "floor" workload).
+__global__ void idle_kernel() {}
+
+extern "C" int cisr_idle(int blocks, hipStream_t stream) {
+    if (blocks <= 0) return 0;
+    idle_kernel<<<(unsigned)blocks, 256, 0, stream>>>();
+    return CISR_LAUNCH_CHECK();
+}

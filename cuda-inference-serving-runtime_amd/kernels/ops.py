@@ -47,6 +47,7 @@ def _declare(h):
         "cisr_rope_scatter": [p, p, p, p, p, p, p, i, i, i, i, i, i, i, i, i, i, p],
         "cisr_page_copy": [p, p, p, i, i, ll, ll, p],
         "cisr_f32_to_bf16": [p, p, ll, p],
+        "cisr_idle": [i, p],
         "cisr_attn_rowwise": [p, i, p, p, p, p, p, p, p, p, i, i, i, i, i, i, i, f, i, i, p],
         "cisr_gemm_f32": [p, i, p, i, p, i, p, i, i, i, i, p],
         "cisr_gemm_bf16": [p, i, p, i, p, i, p, i, i, i, i, i, p],
@@ -264,6 +265,11 @@ def f32_to_bf16(x, out):
     _check(lib().cisr_f32_to_bf16(_dev(x, "x", torch.float32), _dev(out, "out", torch.bfloat16, x.shape), x.numel(),
                                   _stream()), "f32_to_bf16")
     return out
+
+
+def idle(blocks=1):
+    """Launches a kernel of `blocks` blocks that does nothing (the cost of a launch, for measurement)."""
+    _check(lib().cisr_idle(int(blocks), _stream()), "idle")
 
 
 def attention_rowwise(q, q_row_stride, kcache, vcache, tables, seg_of_row, positions, out, heads, kv_heads, dim,

@@ -23,9 +23,11 @@ class GroupView:
 
 
 def fill_tasks(tasks, counts, rows_per_tile, starts=None, skip_single=False):
-    """Write (segment, first row, rows, 0) for tiles of at most `rows_per_tile` consecutive
+    """Write (segment, first row, rows, p) for tiles of at most `rows_per_tile` consecutive
     rows of one segment into the int32 array tasks[n, 4]; returns how many were written.
-    With `starts` (the position of each segment's first row) the tiles are ordered by the
+    With `starts` (the position of each segment's first row) p is the position of the tile's
+    first row plus one (a segment's rows have consecutive positions, so a kernel that reads p need
+    not wait for the positions array; p = 0 says "not given"), and the tiles are ordered by the
     number of keys they attend to, most first: blocks are handed out in this order, and the
     long ones must not be the last to start.  `skip_single`: segments of one row get no tile
     (they are attended to by a launch of their own)."""
@@ -36,7 +38,7 @@ def fill_tasks(tasks, counts, rows_per_tile, starts=None, skip_single=False):
         tasks[n:n + tiles, 0] = seg
         tasks[n:n + tiles, 1] = row + firsts
         tasks[n:n + tiles, 2] = np.minimum(rows_per_tile, count - firsts)
-        tasks[n:n + tiles, 3] = 0
+        tasks[n:n + tiles, 3] = 0 if starts is None else int(starts[seg]) + firsts + 1
         n += tiles
         row += count
     if starts is not None and n > 1:

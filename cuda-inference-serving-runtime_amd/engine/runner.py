@@ -66,6 +66,8 @@ class ModelRunner:
         self.execution = execution
         self.programs, self.program_capacity = {}, 16
         self.block_tiles = None    # long portions through LDS-shared tiles of 64 x this items: None = by the number of blocks
+        # long portions of long contexts through 32 x 32 tiles, 64 x this items a block (1, 2, 4): None = by size, 0 = never
+        self.square_tiles = int(os.environ["CISR_SQUARE_TILES"]) if os.environ.get("CISR_SQUARE_TILES") else None
         self.tile_waves = int(os.environ.get("CISR_TILE_WAVES", "4"))   # wavefronts that share one tile's keys
         self.item_tiles = int(os.environ.get("CISR_ITEM_TILES", "2"))   # 16-item tiles a wave of long portions (small heads)
         # In a mixed step a decoded token is a tile whose keys one block walks; from this context on the
@@ -488,10 +490,28 @@ class ModelRunner:
                                        heads, kv_heads, head_dim, view.page_size, window, scale, None, splits, workspace, waves,
                                        row_ids=ctx.single_rows[:n])
                 long_portions = rows >= 16 * ctx.n_segments
-                block_tiles = 0
+                block_tiles = square = 0
                 if long_portions and head_dim <= 128:
                     blocks = -(-rows // (64 // heads_per_chunk)) * kv_heads * -(-group // heads_per_chunk)
                     block_tiles = (2 if blocks >= 2048 else 1 if blocks >= 512 else 0) if self.block_tiles is None else self.block_tiles
+                    # Long contexts: blocks of 64, 128 or 256 items on the 32 x 32 matrix instruction, with waves of their
+                    # own for the copies and three steps in flight a wave.  They cost about 3 us more to start than the
+                    # forms below, so they are for tiles that walk a thousand keys and more; larger blocks share the
+                    # copies among more waves but need more blocks to fill the GPU (MI355X, 2,048 rows: 1.7B sizes 61 us
+                    # -> 46, 8B sizes 115 -> 71, 135M sizes 31 -> 30; 4,096 rows at the 1.7B sizes: 147 with 128 items,
+                    # 125 with 256).
+                    if view.page_size >= 8:
+                        if self.square_tiles is not None:
+                            square = self.square_tiles
+                        elif span >= 1024 and blocks >= 512:
+                            square = 4 if blocks >= 2048 and head_dim <= 64 else 2
+                        elif span >= 2048 and blocks >= 256:
+                            square = 1
+                if square:
+                    tasks = ctx.attention_tasks(64 * square // heads_per_chunk)
+                    ops.attention_mfma(q, q_row_stride, kcache, vcache, view.tables, ctx.seg_of_row, ctx.positions, out,
+                                       heads, kv_heads, head_dim, view.page_size, window, scale, tasks, block_tiles=32, item_tiles=square)
+                    return
                 if block_tiles:
                     item_tiles = block_tiles
                     tasks = ctx.attention_tasks(64 * item_tiles // heads_per_chunk)

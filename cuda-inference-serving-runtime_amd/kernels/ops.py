@@ -648,12 +648,19 @@ def attention_mfma(q, q_row_stride, kcache, vcache, tables, seg_of_row, position
     fn = _attention_entry(dpad)
     po = pm = tp = None
     if tasks is not None:
-        if item_tiles not in (1, 2) or (item_tiles == 2 and dim > 64 and not block_tiles):
+        if item_tiles not in ((1, 2, 4) if block_tiles == 32 else (1, 2)) or (item_tiles == 2 and dim > 64 and not block_tiles):
             raise KernelError("attention_mfma: two item tiles a wave need a head size of at most 64")
         if block_tiles and dpad > 128:
             raise KernelError("attention_mfma: block tiles need a head size of at most 128")
         n_tasks, splits = tasks.shape[0], 1
         mode = (2 if item_tiles == 1 else 4) if block_tiles else (3 if item_tiles == 2 else 0)
+        if block_tiles == 32:
+            # the 32 x 32 matrix instruction: 128/GC rows a block and four waves (item_tiles 2), or 64/GC rows and two
+            if out.numel() >= 2 ** 31:
+                raise KernelError("attention_mfma: the output must be fewer than 2^31 elements (32-bit offsets)")
+            if page_size < 8 or dpad > 128:
+                raise KernelError("attention_mfma: 32 x 32 block tiles need pages of at least 8 keys and a head size of at most 128")
+            mode = {1: 6, 2: 5, 4: 7}[item_tiles]
         tp = _dev(tasks, "tasks", torch.int32, (n_tasks, 4))
     else:
         n_tasks, mode = rows, 1

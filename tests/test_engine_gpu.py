@@ -404,6 +404,31 @@ def test_long_portions_through_block_tiles_match_the_plain_model(folders, name, 
     assert_close(got[80:], refs["q"][:97], "bfloat16", "another request in the same step")
 
 
+@pytest.mark.parametrize("name", ["a", "c"])
+@pytest.mark.parametrize("square", [1, 2, 4])
+def test_long_portions_through_square_tiles_match_the_plain_model(folders, name, square):
+    """Long portions of long contexts run on the 32 x 32 matrix instruction with waves of their own for the copies;
+    forced here on small models: a whole prompt, then a second portion beside another request, then graph replays."""
+    from runtime.engine import load_model, ModelRunner, StepEntry
+    from conftest import plain_logits, assert_close
+    V = TINY[name]["vocab_size"]
+    model = load_model(folders[name], dtype="bfloat16")
+    seqs = {k: random_tokens(600 + i, 230, V) for i, k in enumerate("pq")}
+    refs = {k: plain_logits(folders[name], seqs[k]) for k in seqs}
+    for execution in ("eager", "graph"):
+        runner = ModelRunner(model, n_pages=64, page_size=8, max_requests=4, execution=execution)
+        runner.square_tiles = square
+        for k in seqs:
+            runner.create(k)
+        got = runner.step([StepEntry("p", seqs["p"][:150], list(range(150)))]).float().cpu().numpy()
+        assert_close(got, refs["p"][:150], "bfloat16", f"{execution}: first portion")
+        got = runner.step([StepEntry("p", seqs["p"][150:], list(range(80))),
+                           StepEntry("q", seqs["q"][:97], list(range(97)))]).float().cpu().numpy()
+        assert_close(got[:80], refs["p"][150:], "bfloat16", f"{execution}: second portion on a cached prefix")
+        assert_close(got[80:], refs["q"][:97], "bfloat16", f"{execution}: another request in the same step")
+        runner.cache.check()
+
+
 def test_temperature_sampling_is_seeded_and_independent_of_the_batch(folders):
     from runtime.engine.scheduler import Engine, Request
     V = TINY["b"]["vocab_size"]

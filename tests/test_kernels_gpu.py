@@ -365,7 +365,7 @@ def test_attention_equal_large_scores_give_the_mean(ops):
 
 
 def run_mfma(ops, qt, kt, vt, tables, rows, page_size, mode, splits=1, window=None, scale=None, rows_per_tile=None, waves=4,
-             row_ids=None):
+             row_ids=None, positions_given=False):
     """mode "tiles": rows are grouped into tiles of consecutive rows of one segment;
     mode "rows": one block per row with `splits` blocks along the keys."""
     T, heads, dim = qt.shape
@@ -375,19 +375,22 @@ def run_mfma(ops, qt, kt, vt, tables, rows, page_size, mode, splits=1, window=No
     out = torch.full((T, heads * dim), 9.0, dtype=qt.dtype, device=DEV)
     tasks = None
     ws = (torch.empty(T * heads * splits * dim, device=DEV), torch.empty(T * heads * splits * 2, device=DEV))
-    if mode in ("tiles", "tiles2", "block", "block2"):
+    items_of = {"tiles": 16, "tiles2": 32, "block": 64, "block2": 128, "square": 64, "square2": 128, "square4": 256}
+    if mode in items_of:
         group = heads // kv_heads
-        rpt = rows_per_tile or {"tiles": 16, "tiles2": 32, "block": 64, "block2": 128}[mode] // min(group, 16)
+        rpt = rows_per_tile or items_of[mode] // min(group, 16)
         items, i = [], 0
         while i < T:   # consecutive rows of one segment with consecutive positions form a tile
             n = 1
             while i + n < T and n < rpt and rows[i + n][0] == rows[i][0] and rows[i + n][1] == rows[i + n - 1][1] + 1:
                 n += 1
-            items.append((rows[i][0], i, n, 0)); i += n
+            # (the fourth entry: the position of the tile's first row plus one, or 0 for "read the positions array")
+            items.append((rows[i][0], i, n, rows[i][1] + 1 if positions_given else 0)); i += n
         tasks = torch.tensor(items, dtype=torch.int32, device=DEV)
     ops.attention_mfma(qt.reshape(T, heads * dim), heads * dim, kt, vt, tables, seg, pos, out, heads, kv_heads, dim,
                        page_size, window, scale if scale is not None else 1 / math.sqrt(dim), tasks, splits, ws, waves,
-                       block_tiles=mode.startswith("block"), item_tiles=(2 if mode in ("tiles2", "block2") else 1),
+                       block_tiles=32 if mode.startswith("square") else mode.startswith("block"),
+                       item_tiles=(4 if mode == "square4" else 2 if mode in ("tiles2", "block2", "square2") else 1),
                        row_ids=None if row_ids is None else torch.tensor(row_ids, dtype=torch.int32, device=DEV))
     return f64(out).reshape(T, heads, dim)
 
@@ -456,6 +459,41 @@ def test_attention_mfma_tiles(ops, heads, kv_heads, dim, page_size):
         np.testing.assert_allclose(got, want, **MFMA_TOL, err_msg=mode)
         got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, mode, rows_per_tile=3)
         np.testing.assert_allclose(got, want, **MFMA_TOL, err_msg=mode)
+    if page_size < 8:                                                                    # 32 x 32 tiles: pages of at least 8 keys
+        with pytest.raises(ops.KernelError):
+            run_mfma(ops, qt, kt, vt, tables, rows, page_size, "square")
+        return
+    for mode in ("square", "square2", "square4"):                                        # 64 / 128 / 256 items on the 32 x 32 instruction
+        for given in (False, True):
+            got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, mode, positions_given=given)
+            np.testing.assert_allclose(got, want, **MFMA_TOL, err_msg=f"{mode} positions given: {given}")
+        got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, mode, rows_per_tile=3, positions_given=True)
+        np.testing.assert_allclose(got, want, **MFMA_TOL, err_msg=mode)
+
+
+@pytest.mark.parametrize("heads, kv_heads, dim, page_size", [(4, 4, 64, 16), (6, 2, 128, 16), (5, 1, 96, 8), (2, 2, 32, 32)])
+def test_attention_square_tiles_over_long_contexts(ops, heads, kv_heads, dim, page_size):
+    """The 32 x 32 form keeps three steps of a tile in flight and moves the reference point of the exponentials only
+    when the maximum has grown a lot: long prefixes (many plain steps before the diagonal), portions that start in the
+    middle of a 32-key step, one key far above the rest late in the context (the reference point jumps, the outputs
+    are rescaled), and tiles of every height."""
+    plan = [(0, 300), (517, 130), (64, 33), (1000, 40)]
+    qt, kt, vt, tables, rows = portion_case(heads, kv_heads, dim, page_size, plan, seed=dim + 7 * heads)
+    # request 1: key 490 of its 647 carries a score far above the rest for every query of head 0
+    page, off = tables[1, 490 // page_size].item(), 490 % page_size
+    first = sum(b for _, b in plan[:1])
+    direction = torch.nn.functional.normalize(qt[first:first + 130, 0].float().mean(0), dim=0)
+    kt[page, 0, off, :] = (direction * 40).to(kt.dtype)
+    qt[first:first + 130, 0] = (qt[first:first + 130, 0].float() + direction * 6).to(qt.dtype)
+    want = reference_attention(qt, kt, vt, tables, rows, page_size)
+    for mode in ("square", "square2", "square4"):
+        for rpt in (None, 5):
+            got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, mode, rows_per_tile=rpt, positions_given=True)
+            np.testing.assert_allclose(got, want, **MFMA_TOL, err_msg=f"{mode} rows a tile: {rpt}")
+    for window in (40, 257):
+        want_w = reference_attention(qt, kt, vt, tables, rows, page_size, window=window)
+        got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, "square2", window=window, positions_given=True)
+        np.testing.assert_allclose(got, want_w, **MFMA_TOL, err_msg=f"window {window}")
 
 
 def test_attention_mfma_window_and_far_key(ops):
@@ -466,6 +504,8 @@ def test_attention_mfma_window_and_far_key(ops):
         np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables, rows, 8, "block", window=window), want, **MFMA_TOL)
         np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables, rows, 8, "block2", window=window), want, **MFMA_TOL)
         np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables, rows, 8, "tiles2", window=window), want, **MFMA_TOL)
+        for mode in ("square", "square2", "square4"):
+            np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables, rows, 8, mode, window=window), want, **MFMA_TOL, err_msg=mode)
         np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables, rows, 8, "rows", 2, window=window), want, **MFMA_TOL)
     want = reference_attention(qt, kt, vt, tables, rows, 8, scale=0.3)
     np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables, rows, 8, "tiles", scale=0.3), want, **MFMA_TOL)
@@ -475,11 +515,13 @@ def test_attention_mfma_window_and_far_key(ops):
     np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables2, rows, 8, "tiles", window=8), want, **MFMA_TOL)
     np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables2, rows, 8, "block", window=8), want, **MFMA_TOL)
     np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables2, rows, 8, "block2", window=8), want, **MFMA_TOL)
+    np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables2, rows, 8, "square", window=8), want, **MFMA_TOL)
+    np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables2, rows, 8, "square2", window=8, positions_given=True), want, **MFMA_TOL)
     np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables2, rows, 8, "rows", 3, window=8), want, **MFMA_TOL)
     # one far key among hundreds stands out
     qt, kt, vt, tables, rows = paged_case(4, 2, 64, 16, [700, 40], torch.bfloat16, seed=5, sharpen=(0, 3))
     want = reference_attention(qt, kt, vt, tables, rows, 16)
-    for mode, splits in (("rows", 1), ("rows", 8), ("tiles", 1), ("block", 1), ("block2", 1)):
+    for mode, splits in (("rows", 1), ("rows", 8), ("tiles", 1), ("block", 1), ("block2", 1), ("square", 1), ("square2", 1)):
         np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables, rows, 16, mode, splits), want, **MFMA_TOL)
 
 
@@ -508,7 +550,8 @@ def test_attention_mfma_ignores_what_unseen_slots_hold(ops):
         t2 = tables.clone()
         if window:                                           # request 2 (position 70, window 16 from 55): pages 0..2 passed
             t2[2, :3] = -1
-        for mode, splits in (("tiles", 1), ("tiles2", 1), ("block", 1), ("block2", 1), ("rows", 1), ("rows", 3)):
+        for mode, splits in (("tiles", 1), ("tiles2", 1), ("block", 1), ("block2", 1), ("square", 1), ("square2", 1), ("square4", 1),
+                             ("rows", 1), ("rows", 3)):
             got = run_mfma(ops, qt, kt, vt, t2, rows, P_, mode, splits, window=window)
             assert np.isfinite(got).all(), f"{mode} window={window}: poison reached the output"
             np.testing.assert_allclose(got, want[window], **MFMA_TOL, err_msg=f"{mode} window={window}")

@@ -26,9 +26,11 @@ def test_task_lists_cover_every_row_once_and_never_cross_a_segment():
         seg_starts = rng.integers(0, 100, size=len(counts)).tolist()
         ordered = np.full((most, 4), -7, dtype=np.int32)
         assert fill_tasks(ordered, counts, rows_per_tile, seg_starts) == n
-        assert sorted(map(tuple, ordered[:n])) == sorted(map(tuple, tasks[:n]))
+        assert sorted(map(tuple, ordered[:n, :3])) == sorted(map(tuple, tasks[:n, :3]))
         keys = [seg_starts[seg] + first - starts[seg] + rows for seg, first, rows, _ in ordered[:n]]
         assert keys == sorted(keys, reverse=True)
+        # and the fourth entry is the position of the tile's first row, plus one (0 stands for "not given")
+        assert [p for *_, p in ordered[:n]] == [seg_starts[seg] + first - starts[seg] + 1 for seg, first, _, _ in ordered[:n]]
 
 
 def test_program_sizes_are_powers_of_two_then_multiples_of_64():

@@ -143,10 +143,12 @@ def main():
     ap.add_argument("--overlap", type=int, default=1, choices=[0, 1],
                     help="1: picked tokens stay on the device and a step is launched before the tokens of the one "
                          "before are read, as the scheduler's overlapped ticks do; 0: every step waits for its tokens")
-    ap.add_argument("--workload", default="decode", choices=["decode", "serving", "floor"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "serving", "floor", "attention"],
                     help="decode: fixed batch after whole prompts (the default, timed per step); serving: --requests "
                          "requests with prompts of 128..--prompt tokens and --new-tokens each through the scheduler; "
-                         "floor: a captured chain of kernels that do nothing (what a launch costs)")
+                         "floor: a captured chain of kernels that do nothing (what a launch costs); attention: the attention kernel "
+                         "alone over whole prompts of --attention-rows rows at the family's head shapes")
+    ap.add_argument("--attention-rows", default="2048,7936", help="attention workload: prompt lengths (comma separated)")
     ap.add_argument("--requests", type=int, default=64)
     ap.add_argument("--new-tokens", type=int, default=256)
     ap.add_argument("--token-budget", type=int, default=2112, help="serving: rows a step (a whole prompt beside 64 decoded tokens)")
@@ -162,6 +164,8 @@ def main():
 
     if args.workload == "floor":
         return launch_floor(args)
+    if args.workload == "attention":
+        return prompt_attention(args)
     raw = preset(args.model)
     full_layers = raw["num_hidden_layers"]
     if args.layers:
@@ -267,6 +271,68 @@ def launch_floor(args):
                       "unit": "us", "higher_is_better": False, "n_gpus": 1, "chain": chain, "replays": 20, "us_per_kernel": out,
                       "kernels_of_a_decode_step": kernels, "model": args.model,
                       "floor_ms_of_a_decode_step": round(kernels * out["one_block"] / 1e3, 4)}))
+    return 0
+
+
+def prompt_attention(args):
+    """The attention kernel alone on whole prompts: causal attention of T rows over their own T keys in a paged cache, at
+    the head shapes of the three family members, in the form the engine chooses for that size.  Twenty calls in one
+    captured graph, the median of five replays; flops are those of the causal half, 4 T (T + 1) / 2 x head size x heads."""
+    import statistics
+    import numpy as np
+    import torch
+    from runtime.config import preset
+    from runtime.engine import ModelRunner
+    from runtime.engine.context import fill_tasks
+    from runtime.kernels import ops
+    dev = torch.device("cuda:0")
+    P = args.page_size
+    out = {}
+    chooser = ModelRunner.__new__(ModelRunner)          # only its tiling rule is used
+    chooser.square_tiles = chooser.block_tiles = None
+    chooser.item_tiles = 2
+    for name in ("smollm2-135m", "smollm2-1.7b", "llama-3-8b"):
+        raw = preset(name)
+        heads, kv_heads = raw["num_attention_heads"], raw["num_key_value_heads"]
+        D = raw.get("head_dim") or raw["hidden_size"] // heads
+        for T in [int(t) for t in args.attention_rows.split(",") if t]:
+            pages = -(-T // P)
+            q = torch.randn(T, heads * D, device=dev).bfloat16()
+            K = torch.randn(pages, kv_heads, P, D, device=dev).bfloat16()
+            V = torch.randn(pages, kv_heads, D, P, device=dev).bfloat16()
+            tables = torch.arange(pages, dtype=torch.int32, device=dev).reshape(1, pages)
+            seg = torch.zeros(T, dtype=torch.int32, device=dev)
+            pos = torch.arange(T, dtype=torch.int32, device=dev)
+            o = torch.empty(T, heads * D, device=dev, dtype=torch.bfloat16)
+            kind, n = chooser.prompt_attention_form(T, 1, T, heads, kv_heads, D, P)
+            rows_per_tile = (16 if kind == "tiles" else 64) * n // min(heads // kv_heads, 16)
+            host = np.full((-(-T // rows_per_tile), 4), -1, dtype=np.int32)
+            fill_tasks(host, [T], rows_per_tile, [0])
+            tasks = torch.from_numpy(host).to(dev)
+
+            def run():
+                ops.attention_mfma(q, heads * D, K, V, tables, seg, pos, o, heads, kv_heads, D, P, None, D ** -0.5, tasks,
+                                   block_tiles={"tiles": False, "block": True, "square": 32}[kind], item_tiles=n)
+            calls = 20
+            stream, graph = torch.cuda.Stream(), torch.cuda.CUDAGraph()
+            with torch.cuda.stream(stream):
+                run(); stream.synchronize()
+                with torch.cuda.graph(graph, stream=stream):
+                    for _ in range(calls):
+                        run()
+            times = []
+            for _ in range(6):
+                torch.cuda.synchronize(); t0 = time.perf_counter()
+                graph.replay()
+                torch.cuda.synchronize(); times.append((time.perf_counter() - t0) / calls)
+            us = statistics.median(times[1:]) * 1e6
+            flops = 4 * T * (T + 1) / 2 * D * heads
+            out[f"{name}_{T}"] = {"heads": heads, "kv_heads": kv_heads, "head_dim": D, "rows": T, "form": f"{kind} x{n}",
+                                  "us": round(us, 1), "pflops": round(flops / us / 1e9, 3),
+                                  "frac_of_bf16_peak": round(flops / us / 1e6 / PEAK_TFLOPS["bf16"], 4)}
+    print(json.dumps({"metric": "prompt attention alone, PFLOP/s of the causal half (bf16, paged cache, page size %d)" % P,
+                      "unit": "PFLOP/s", "n_gpus": 1, "value": out["smollm2-1.7b_%s" % args.attention_rows.split(",")[0]]["pflops"],
+                      "higher_is_better": True, "shapes": out}))
     return 0
 
 

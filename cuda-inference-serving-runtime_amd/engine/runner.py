@@ -474,10 +474,6 @@ class ModelRunner:
                 ops.attention_mfma(q, q_row_stride, kcache, vcache, view.tables, ctx.seg_of_row, ctx.positions, out,
                                    heads, kv_heads, head_dim, view.page_size, window, scale, None, splits, workspace, waves)
             else:
-                # long portions, enough of them to fill the GPU with blocks of 64 items (or 128): the four waves of
-                # a block own different rows and share each step's keys and values through LDS.  Otherwise (few
-                # heads, short portions) the waves of a block share one tile of 16 items (32 with small heads)
-                # and split its keys, which is what hides the latency of a step when blocks are scarce.
                 if ctx.n_single:
                     # the decoded tokens of this mixed step: a launch of their own that splits their keys
                     n = ctx.n_single
@@ -489,38 +485,11 @@ class ModelRunner:
                     ops.attention_mfma(q, q_row_stride, kcache, vcache, view.tables, ctx.seg_of_row, ctx.positions, out,
                                        heads, kv_heads, head_dim, view.page_size, window, scale, None, splits, workspace, waves,
                                        row_ids=ctx.single_rows[:n])
-                long_portions = rows >= 16 * ctx.n_segments
-                block_tiles = square = 0
-                if long_portions and head_dim <= 128:
-                    blocks = -(-rows // (64 // heads_per_chunk)) * kv_heads * -(-group // heads_per_chunk)
-                    block_tiles = (2 if blocks >= 2048 else 1 if blocks >= 512 else 0) if self.block_tiles is None else self.block_tiles
-                    # Long contexts: blocks of 64, 128 or 256 items on the 32 x 32 matrix instruction, with waves of their
-                    # own for the copies and three steps in flight a wave.  They cost about 3 us more to start than the
-                    # forms below, so they are for tiles that walk a thousand keys and more; larger blocks share the
-                    # copies among more waves but need more blocks to fill the GPU (MI355X, 2,048 rows: 1.7B sizes 61 us
-                    # -> 46, 8B sizes 115 -> 71, 135M sizes 31 -> 30; 4,096 rows at the 1.7B sizes: 147 with 128 items,
-                    # 125 with 256).
-                    if view.page_size >= 8:
-                        if self.square_tiles is not None:
-                            square = self.square_tiles
-                        elif span >= 1024 and blocks >= 512:
-                            square = 4 if blocks >= 2048 and head_dim <= 64 else 2
-                        elif span >= 2048 and blocks >= 256:
-                            square = 1
-                if square:
-                    tasks = ctx.attention_tasks(64 * square // heads_per_chunk)
-                    ops.attention_mfma(q, q_row_stride, kcache, vcache, view.tables, ctx.seg_of_row, ctx.positions, out,
-                                       heads, kv_heads, head_dim, view.page_size, window, scale, tasks, block_tiles=32, item_tiles=square)
-                    return
-                if block_tiles:
-                    item_tiles = block_tiles
-                    tasks = ctx.attention_tasks(64 * item_tiles // heads_per_chunk)
-                else:
-                    item_tiles = 2 if self.item_tiles == 2 and long_portions and head_dim <= 64 else 1
-                    tasks = ctx.attention_tasks(16 * item_tiles // heads_per_chunk)
+                kind, item_tiles = self.prompt_attention_form(rows, ctx.n_segments, span, heads, kv_heads, head_dim, view.page_size)
+                tasks = ctx.attention_tasks((16 if kind == "tiles" else 64) * item_tiles // heads_per_chunk)
                 ops.attention_mfma(q, q_row_stride, kcache, vcache, view.tables, ctx.seg_of_row, ctx.positions, out,
                                    heads, kv_heads, head_dim, view.page_size, window, scale, tasks, waves=self.tile_waves,
-                                   block_tiles=bool(block_tiles), item_tiles=item_tiles)
+                                   block_tiles={"tiles": False, "block": True, "square": 32}[kind], item_tiles=item_tiles)
             return
         splits = self._splits(rows * heads, span)
         workspace = None
@@ -529,6 +498,36 @@ class ModelRunner:
                          ctx.buffer("attn.part_ml", (rows * heads * splits * 2,), torch.float32))
         ops.attention_rowwise(q, q_row_stride, kcache, vcache, view.tables, ctx.seg_of_row, ctx.positions, out,
                               heads, kv_heads, head_dim, view.page_size, window, scale, splits, workspace)
+
+    def prompt_attention_form(self, rows, n_segments, span, heads, kv_heads, head_dim, page_size):
+        """Which form of the matrix-core kernel the prompt rows of a step take: ("tiles", n): a block is one tile of 16 n
+        items (a token row and a query head) whose waves split its keys; ("block", n): 64 n items, four waves that own
+        different rows and share keys and values through LDS; ("square", n): 64 n items on the 32 x 32 instruction with
+        waves of their own for the copies.  `span`: the longest context of the step."""
+        group = heads // kv_heads
+        heads_per_chunk = min(group, 16)
+        long_portions = rows >= 16 * n_segments
+        if long_portions and head_dim <= 128:
+            # enough long portions to fill the GPU with blocks of 64 items (or more): the waves of a block own different
+            # rows and share each step's keys and values through LDS.  Otherwise (few heads, short portions) the waves
+            # of a block share one tile of 16 items (32 with small heads) and split its keys, which is what hides
+            # the latency of a step when blocks are scarce.
+            blocks = -(-rows // (64 // heads_per_chunk)) * kv_heads * -(-group // heads_per_chunk)
+            # Long contexts: the 32 x 32 form, with three steps in flight a wave.  It costs about 3 us more to start
+            # than the others, so it is for tiles that walk a thousand keys and more; larger blocks share the copies
+            # among more waves but need more blocks to fill the GPU (MI355X, 2,048 rows: 1.7B sizes 61 us -> 46,
+            # 8B sizes 115 -> 71, 135M sizes 32 -> 30; 4,096 rows at the 1.7B sizes: 147 with 128 items, 125 with 256).
+            if page_size >= 8 and self.square_tiles != 0:
+                if self.square_tiles is not None:
+                    return "square", self.square_tiles
+                if span >= 1024 and blocks >= 512:
+                    return "square", 4 if blocks >= 2048 and head_dim <= 64 else 2
+                if span >= 2048 and blocks >= 256:
+                    return "square", 1
+            block_tiles = (2 if blocks >= 2048 else 1 if blocks >= 512 else 0) if self.block_tiles is None else self.block_tiles
+            if block_tiles:
+                return "block", block_tiles
+        return "tiles", 2 if self.item_tiles == 2 and long_portions and head_dim <= 64 else 1
 
     @staticmethod
     def _splits(waves, span):

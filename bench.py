@@ -81,15 +81,19 @@ def measure(model, args, batches, prompt, context, steps, warmup, repeats):
 
         for _ in range(warmup):
             one()
-        timings = []
+        timings, event_ms = [], []
         for _ in range(repeats):
             torch.cuda.synchronize()
             ctx0 = runner.length(keys[0])
+            begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             t0 = time.perf_counter()
+            begin.record()
             for _ in range(steps):
                 one()
+            end.record()
             torch.cuda.synchronize()      # (overlapped: the tokens of the last step are read by the next repeat's first)
             timings.append((time.perf_counter() - t0, ctx0 + steps / 2))
+            event_ms.append(begin.elapsed_time(end) / steps)   # the same steps by the GPU's own events
         if unread is not None:
             last, unread = unread.tokens(), None
         for key in keys:
@@ -97,11 +101,32 @@ def measure(model, args, batches, prompt, context, steps, warmup, repeats):
         elapsed, ctx_mid = sorted(timings)[len(timings) // 2]
         step_bytes = weight_bytes + batch * ctx_mid * kv_bytes_per_token
         out[batch] = {"ms_per_step": elapsed / steps * 1e3, "tokens_per_s": batch * steps / elapsed,
-                      "gbps": step_bytes / (elapsed / steps) / 1e9, "ms_all": [round(t / steps * 1e3, 4) for t, _ in timings]}
+                      "gbps": step_bytes / (elapsed / steps) / 1e9, "ms_all": [round(t / steps * 1e3, 4) for t, _ in timings],
+                      "event_ms": round(statistics.median(event_ms), 4)}
     # the prompt step: the median of all timed ones but the very first (which pays one-time set-up)
     pf = statistics.median(prefill_times[1:] if len(prefill_times) > 1 else prefill_times)
     del runner
     return out, pf, prefill_flops
+
+
+def library_matmul_tflops():
+    """TFLOP/s of the vendor library's bf16 product of two 8192 x 8192 matrices, the median of five: what the matrix
+    cores give a large product on this GPU, beside the published peak."""
+    import statistics
+    import torch
+    n = 8192
+    a = torch.randn(n, n, device="cuda", dtype=torch.bfloat16)
+    b = torch.randn(n, n, device="cuda", dtype=torch.bfloat16)
+    c = torch.empty(n, n, device="cuda", dtype=torch.bfloat16)
+    torch.mm(a, b, out=c)
+    times = []
+    for _ in range(5):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        torch.mm(a, b, out=c)
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t0)
+    return 2 * n ** 3 / statistics.median(times) / 1e12
 
 
 def copy_bandwidth():
@@ -189,6 +214,7 @@ def main():
     main_r = results[args.batch]
     peak = PEAK_TFLOPS["bf16" if args.dtype == "bfloat16" else "fp32"] * 1e12
     copy_gbps = copy_bandwidth()
+    matmul_tflops = library_matmul_tflops()
     points = {f"decode_b{b}": round(results[b]["tokens_per_s"], 1) for b in batches if b != args.batch}
     line = {
         "metric": f"decode tokens/s, {args.model} layer sizes, batch {args.batch}, {args.prompt}-token prompts in a {args.context} context",
@@ -201,12 +227,14 @@ def main():
                    "rope_theta": c.rope_theta, "rms_norm_eps": c.rms_norm_eps, "tied_head": c.tie_word_embeddings,
                    "page_size": args.page_size, "execution": args.execution + (", steps overlapped" if args.overlap else "")},
         "prefill": {"value": round(args.prompt / pf, 1), "tokens": args.prompt, "ms": round(pf * 1e3, 3),
-                    "frac": round(pf_flops / pf / peak, 5)},
+                    "frac": round(pf_flops / pf / peak, 5), "peak_tflops": peak / 1e12,
+                    "measured_library_matmul_tflops": round(matmul_tflops, 1)},
         "roofline": {"bound": "hbm", "achieved": round(main_r["gbps"], 1), "peak": HBM_GBPS, "unit": "GB/s",
                      "frac": round(main_r["gbps"] / HBM_GBPS, 5), "measured_copy": round(copy_gbps, 1)},
         "points": points,
         "points_roofline_frac": {f"decode_b{b}": round(results[b]["gbps"] / HBM_GBPS, 5) for b in batches if b != args.batch},
-        "method": {"repeats": repeats, "statistic": "median", "ms_per_step_of_repeats": main_r["ms_all"], "clock": "host, synchronised"},
+        "method": {"repeats": repeats, "statistic": "median", "ms_per_step_of_repeats": main_r["ms_all"], "clock": "host, synchronised",
+                   "ms_per_step_by_gpu_events": main_r["event_ms"]},
         "reference_b1_tokens_per_s": REFERENCE_B1_TOKS,
     }
     # further layer sizes, with fewer layers than their configurations have (both numbers named): random weights drawn

@@ -317,7 +317,7 @@ def prompt_attention(args):
     P = args.page_size
     out = {}
     chooser = ModelRunner.__new__(ModelRunner)          # only its tiling rule is used
-    chooser.square_tiles = chooser.block_tiles = None
+    chooser.square_tiles = chooser.block_tiles = chooser.square_halves = None
     chooser.item_tiles = 2
     for name in ("smollm2-135m", "smollm2-1.7b", "llama-3-8b"):
         raw = preset(name)
@@ -332,7 +332,7 @@ def prompt_attention(args):
             seg = torch.zeros(T, dtype=torch.int32, device=dev)
             pos = torch.arange(T, dtype=torch.int32, device=dev)
             o = torch.empty(T, heads * D, device=dev, dtype=torch.bfloat16)
-            kind, n = chooser.prompt_attention_form(T, 1, T, heads, kv_heads, D, P)
+            kind, n, halves = chooser.prompt_attention_form(T, 1, T, heads, kv_heads, D, P)
             rows_per_tile = (16 if kind == "tiles" else 64) * n // min(heads // kv_heads, 16)
             host = np.full((-(-T // rows_per_tile), 4), -1, dtype=np.int32)
             fill_tasks(host, [T], rows_per_tile, [0])
@@ -340,7 +340,7 @@ def prompt_attention(args):
 
             def run():
                 ops.attention_mfma(q, heads * D, K, V, tables, seg, pos, o, heads, kv_heads, D, P, None, D ** -0.5, tasks,
-                                   block_tiles={"tiles": False, "block": True, "square": 32}[kind], item_tiles=n)
+                                   block_tiles={"tiles": False, "block": True, "square": 32}[kind], item_tiles=n, key_groups=halves)
             calls = 20
             stream, graph = torch.cuda.Stream(), torch.cuda.CUDAGraph()
             with torch.cuda.stream(stream):
@@ -355,7 +355,7 @@ def prompt_attention(args):
                 torch.cuda.synchronize(); times.append((time.perf_counter() - t0) / calls)
             us = statistics.median(times[1:]) * 1e6
             flops = 4 * T * (T + 1) / 2 * D * heads
-            out[f"{name}_{T}"] = {"heads": heads, "kv_heads": kv_heads, "head_dim": D, "rows": T, "form": f"{kind} x{n}",
+            out[f"{name}_{T}"] = {"heads": heads, "kv_heads": kv_heads, "head_dim": D, "rows": T, "form": f"{kind} x{n}" + (", two halves" if halves == 2 else ""),
                                   "us": round(us, 1), "pflops": round(flops / us / 1e9, 3),
                                   "frac_of_bf16_peak": round(flops / us / 1e6 / PEAK_TFLOPS["bf16"], 4)}
     print(json.dumps({"metric": "prompt attention alone, PFLOP/s of the causal half (bf16, paged cache, page size %d)" % P,

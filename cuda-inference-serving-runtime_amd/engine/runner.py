@@ -68,6 +68,7 @@ class ModelRunner:
         self.block_tiles = None    # long portions through LDS-shared tiles of 64 x this items: None = by the number of blocks
         # long portions of long contexts through 32 x 32 tiles, 64 x this items a block (1, 2, 4): None = by size, 0 = never
         self.square_tiles = int(os.environ["CISR_SQUARE_TILES"]) if os.environ.get("CISR_SQUARE_TILES") else None
+        self.square_halves = None  # two halves a block in that form (even and odd steps): None = by the number of blocks, 1, 2
         self.tile_waves = int(os.environ.get("CISR_TILE_WAVES", "4"))   # wavefronts that share one tile's keys
         self.item_tiles = int(os.environ.get("CISR_ITEM_TILES", "2"))   # 16-item tiles a wave of long portions (small heads)
         # In a mixed step a decoded token is a tile whose keys one block walks; from this context on the
@@ -485,11 +486,12 @@ class ModelRunner:
                     ops.attention_mfma(q, q_row_stride, kcache, vcache, view.tables, ctx.seg_of_row, ctx.positions, out,
                                        heads, kv_heads, head_dim, view.page_size, window, scale, None, splits, workspace, waves,
                                        row_ids=ctx.single_rows[:n])
-                kind, item_tiles = self.prompt_attention_form(rows, ctx.n_segments, span, heads, kv_heads, head_dim, view.page_size)
+                kind, item_tiles, halves = self.prompt_attention_form(rows, ctx.n_segments, span, heads, kv_heads, head_dim, view.page_size)
                 tasks = ctx.attention_tasks((16 if kind == "tiles" else 64) * item_tiles // heads_per_chunk)
                 ops.attention_mfma(q, q_row_stride, kcache, vcache, view.tables, ctx.seg_of_row, ctx.positions, out,
                                    heads, kv_heads, head_dim, view.page_size, window, scale, tasks, waves=self.tile_waves,
-                                   block_tiles={"tiles": False, "block": True, "square": 32}[kind], item_tiles=item_tiles)
+                                   block_tiles={"tiles": False, "block": True, "square": 32}[kind], item_tiles=item_tiles,
+                                   key_groups=halves)
             return
         splits = self._splits(rows * heads, span)
         workspace = None
@@ -500,10 +502,11 @@ class ModelRunner:
                               heads, kv_heads, head_dim, view.page_size, window, scale, splits, workspace)
 
     def prompt_attention_form(self, rows, n_segments, span, heads, kv_heads, head_dim, page_size):
-        """Which form of the matrix-core kernel the prompt rows of a step take: ("tiles", n): a block is one tile of 16 n
-        items (a token row and a query head) whose waves split its keys; ("block", n): 64 n items, four waves that own
-        different rows and share keys and values through LDS; ("square", n): 64 n items on the 32 x 32 instruction with
-        waves of their own for the copies.  `span`: the longest context of the step."""
+        """Which form of the matrix-core kernel the prompt rows of a step take, (kind, n, halves): ("tiles", n, 1): a block
+        is one tile of 16 n items (a token row and a query head) whose waves split its keys; ("block", n, 1): 64 n items,
+        four waves that own different rows and share keys and values through LDS; ("square", n, halves): 64 n items on
+        the 32 x 32 instruction with waves of their own for the copies, as one half or as two that take the even and the
+        odd steps.  `span`: the longest context of the step."""
         group = heads // kv_heads
         heads_per_chunk = min(group, 16)
         long_portions = rows >= 16 * n_segments
@@ -518,16 +521,25 @@ class ModelRunner:
             # among more waves but need more blocks to fill the GPU (MI355X, 2,048 rows: 1.7B sizes 61 us -> 46,
             # 8B sizes 115 -> 71, 135M sizes 32 -> 30; 4,096 rows at the 1.7B sizes: 147 with 128 items, 125 with 256).
             if page_size >= 8 and self.square_tiles != 0:
+                n = 0
                 if self.square_tiles is not None:
-                    return "square", self.square_tiles
-                if span >= 1024 and blocks >= 512:
-                    return "square", 4 if blocks >= 2048 and head_dim <= 64 else 2
-                if span >= 2048 and blocks >= 256:
-                    return "square", 1
+                    n = self.square_tiles
+                elif span >= 1024 and blocks >= 512:
+                    n = 4 if blocks >= 2048 and head_dim <= 64 else 2
+                elif span >= 2048 and blocks >= 256:
+                    n = 1
+                if n:
+                    # about one block a compute unit: the time is the longest tile's chain of steps, which two halves a
+                    # block cut in two (2,048 rows at the 135M sizes 31.6 -> 28.4 us, 4,096 rows 64 -> 55; with more
+                    # blocks than that the halves only crowd the compute units: 46 -> 68 us at the 1.7B sizes)
+                    few = -(-blocks // n) <= 320
+                    fits = n == 1 or (n == 2 and head_dim <= 64)
+                    halves = 2 if (few and fits if self.square_halves is None else self.square_halves == 2 and fits) else 1
+                    return "square", n, halves
             block_tiles = (2 if blocks >= 2048 else 1 if blocks >= 512 else 0) if self.block_tiles is None else self.block_tiles
             if block_tiles:
-                return "block", block_tiles
-        return "tiles", 2 if self.item_tiles == 2 and long_portions and head_dim <= 64 else 1
+                return "block", block_tiles, 1
+        return "tiles", 2 if self.item_tiles == 2 and long_portions and head_dim <= 64 else 1, 1
 
     @staticmethod
     def _splits(waves, span):

@@ -619,7 +619,7 @@ def qkv_rope(a, w, q_out, positions, slots, cos, sin, kcache, vcache, heads, kv_
 
 def attention_mfma(q, q_row_stride, kcache, vcache, tables, seg_of_row, positions, out, heads, kv_heads, dim,
                    page_size, window, scale, tasks=None, splits=1, workspace=None, waves=4, block_tiles=False,
-                   item_tiles=1, row_ids=None, merge=True):
+                   item_tiles=1, row_ids=None, merge=True, key_groups=1):
     """Matrix-core attention (bf16).  tasks int32 [n, 4] = (segment, first row, rows, 0) runs tiles of
     prompt rows: one tile of 16/GC rows a block whose waves share the keys (with item_tiles=2, head sizes up to
     64: 32/GC rows, two item tiles a wave), or with `block_tiles` (head sizes up to 128) one tile of
@@ -629,7 +629,8 @@ def attention_mfma(q, q_row_stride, kcache, vcache, tables, seg_of_row, position
     workspace = (partials float, statistics float) and a merge.  `row_ids` (int32 [n], with tasks None): only
     the rows it lists are computed and written (negative entries are skipped): the decode rows of a mixed step.
     `merge` False (rows mode with splits > 1): the partial outputs are left unmerged in the workspace, whose first
-    buffer is then bfloat16, for gemm_merged; `out` is not written."""
+    buffer is then bfloat16, for gemm_merged; `out` is not written.  `key_groups` 2 (block_tiles 32): a block is two
+    halves that take the even and the odd 32-key steps of its items and merge at the end."""
     rows = out.shape[0]
     if not mfma_attention_supported(out.dtype, dim, page_size):
         raise KernelError(f"attention_mfma: head size {dim} / page size {page_size} / dtype {out.dtype} not supported")
@@ -660,7 +661,11 @@ def attention_mfma(q, q_row_stride, kcache, vcache, tables, seg_of_row, position
                 raise KernelError("attention_mfma: the output must be fewer than 2^31 elements (32-bit offsets)")
             if page_size < 8 or dpad > 128:
                 raise KernelError("attention_mfma: 32 x 32 block tiles need pages of at least 8 keys and a head size of at most 128")
-            mode = {1: 6, 2: 5, 4: 7}[item_tiles]
+            if key_groups not in (1, 2) or (key_groups == 2 and item_tiles == 4):
+                raise KernelError("attention_mfma: one or two key groups, two with 64 or 128 items a block")
+            if dpad > 64 and (item_tiles == 4 or (item_tiles == 2 and key_groups == 2)):
+                raise KernelError("attention_mfma: blocks of more than eight waves need a head size of at most 64")
+            mode = {(1, 1): 6, (2, 1): 5, (4, 1): 7, (1, 2): 8, (2, 2): 9}[(item_tiles, key_groups)]
         tp = _dev(tasks, "tasks", torch.int32, (n_tasks, 4))
     else:
         n_tasks, mode = rows, 1

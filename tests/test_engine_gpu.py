@@ -405,8 +405,8 @@ def test_long_portions_through_block_tiles_match_the_plain_model(folders, name, 
 
 
 @pytest.mark.parametrize("name", ["a", "c"])
-@pytest.mark.parametrize("square", [1, 2, 4])
-def test_long_portions_through_square_tiles_match_the_plain_model(folders, name, square):
+@pytest.mark.parametrize("square, halves", [(1, 1), (2, 1), (4, 1), (1, 2), (2, 2)])
+def test_long_portions_through_square_tiles_match_the_plain_model(folders, name, square, halves):
     """Long portions of long contexts run on the 32 x 32 matrix instruction with waves of their own for the copies;
     forced here on small models: a whole prompt, then a second portion beside another request, then graph replays."""
     from runtime.engine import load_model, ModelRunner, StepEntry
@@ -417,7 +417,7 @@ def test_long_portions_through_square_tiles_match_the_plain_model(folders, name,
     refs = {k: plain_logits(folders[name], seqs[k]) for k in seqs}
     for execution in ("eager", "graph"):
         runner = ModelRunner(model, n_pages=64, page_size=8, max_requests=4, execution=execution)
-        runner.square_tiles = square
+        runner.square_tiles, runner.square_halves = square, halves
         for k in seqs:
             runner.create(k)
         got = runner.step([StepEntry("p", seqs["p"][:150], list(range(150)))]).float().cpu().numpy()

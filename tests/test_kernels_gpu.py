@@ -375,7 +375,9 @@ def run_mfma(ops, qt, kt, vt, tables, rows, page_size, mode, splits=1, window=No
     out = torch.full((T, heads * dim), 9.0, dtype=qt.dtype, device=DEV)
     tasks = None
     ws = (torch.empty(T * heads * splits * dim, device=DEV), torch.empty(T * heads * splits * 2, device=DEV))
-    items_of = {"tiles": 16, "tiles2": 32, "block": 64, "block2": 128, "square": 64, "square2": 128, "square4": 256}
+    # ("square...": blocks on the 32 x 32 instruction; "...halves": two halves a block for the even and the odd steps)
+    items_of = {"tiles": 16, "tiles2": 32, "block": 64, "block2": 128, "square": 64, "square2": 128, "square4": 256,
+                "square_halves": 64, "square2_halves": 128}
     if mode in items_of:
         group = heads // kv_heads
         rpt = rows_per_tile or items_of[mode] // min(group, 16)
@@ -390,12 +392,18 @@ def run_mfma(ops, qt, kt, vt, tables, rows, page_size, mode, splits=1, window=No
     ops.attention_mfma(qt.reshape(T, heads * dim), heads * dim, kt, vt, tables, seg, pos, out, heads, kv_heads, dim,
                        page_size, window, scale if scale is not None else 1 / math.sqrt(dim), tasks, splits, ws, waves,
                        block_tiles=32 if mode.startswith("square") else mode.startswith("block"),
-                       item_tiles=(4 if mode == "square4" else 2 if mode in ("tiles2", "block2", "square2") else 1),
+                       item_tiles=(4 if mode == "square4" else 2 if mode in ("tiles2", "block2", "square2", "square2_halves") else 1),
+                       key_groups=2 if mode.endswith("_halves") else 1,
                        row_ids=None if row_ids is None else torch.tensor(row_ids, dtype=torch.int32, device=DEV))
     return f64(out).reshape(T, heads, dim)
 
 
 MFMA_TOL = dict(rtol=2e-2, atol=2e-2)
+
+
+def square_modes(dim):
+    """The forms of the 32 x 32 kernel that take this head size (blocks of more than eight waves: up to 64)."""
+    return ("square", "square2", "square_halves") + (("square4", "square2_halves") if dim <= 64 else ())
 
 
 @pytest.mark.parametrize("heads, kv_heads, dim, page_size", [
@@ -463,7 +471,10 @@ def test_attention_mfma_tiles(ops, heads, kv_heads, dim, page_size):
         with pytest.raises(ops.KernelError):
             run_mfma(ops, qt, kt, vt, tables, rows, page_size, "square")
         return
-    for mode in ("square", "square2", "square4"):                                        # 64 / 128 / 256 items on the 32 x 32 instruction
+    if dim > 64:
+        with pytest.raises(ops.KernelError):
+            run_mfma(ops, qt, kt, vt, tables, rows, page_size, "square4")
+    for mode in square_modes(dim):                                                       # 64 / 128 / 256 items on the 32 x 32 instruction
         for given in (False, True):
             got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, mode, positions_given=given)
             np.testing.assert_allclose(got, want, **MFMA_TOL, err_msg=f"{mode} positions given: {given}")
@@ -486,7 +497,7 @@ def test_attention_square_tiles_over_long_contexts(ops, heads, kv_heads, dim, pa
     kt[page, 0, off, :] = (direction * 40).to(kt.dtype)
     qt[first:first + 130, 0] = (qt[first:first + 130, 0].float() + direction * 6).to(qt.dtype)
     want = reference_attention(qt, kt, vt, tables, rows, page_size)
-    for mode in ("square", "square2", "square4"):
+    for mode in square_modes(dim):
         for rpt in (None, 5):
             got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, mode, rows_per_tile=rpt, positions_given=True)
             np.testing.assert_allclose(got, want, **MFMA_TOL, err_msg=f"{mode} rows a tile: {rpt}")
@@ -504,7 +515,7 @@ def test_attention_mfma_window_and_far_key(ops):
         np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables, rows, 8, "block", window=window), want, **MFMA_TOL)
         np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables, rows, 8, "block2", window=window), want, **MFMA_TOL)
         np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables, rows, 8, "tiles2", window=window), want, **MFMA_TOL)
-        for mode in ("square", "square2", "square4"):
+        for mode in square_modes(32):
             np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables, rows, 8, mode, window=window), want, **MFMA_TOL, err_msg=mode)
         np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables, rows, 8, "rows", 2, window=window), want, **MFMA_TOL)
     want = reference_attention(qt, kt, vt, tables, rows, 8, scale=0.3)
@@ -551,7 +562,7 @@ def test_attention_mfma_ignores_what_unseen_slots_hold(ops):
         if window:                                           # request 2 (position 70, window 16 from 55): pages 0..2 passed
             t2[2, :3] = -1
         for mode, splits in (("tiles", 1), ("tiles2", 1), ("block", 1), ("block2", 1), ("square", 1), ("square2", 1), ("square4", 1),
-                             ("rows", 1), ("rows", 3)):
+                             ("square_halves", 1), ("square2_halves", 1), ("rows", 1), ("rows", 3)):
             got = run_mfma(ops, qt, kt, vt, t2, rows, P_, mode, splits, window=window)
             assert np.isfinite(got).all(), f"{mode} window={window}: poison reached the output"
             np.testing.assert_allclose(got, want[window], **MFMA_TOL, err_msg=f"{mode} window={window}")

@@ -429,6 +429,29 @@ def test_attention_mfma_rows(ops, heads, kv_heads, dim, page_size):
         assert (got[[1, 2, 4]] == 9.0).all()
 
 
+@pytest.mark.parametrize("heads, kv_heads, dim, page_size", [(9, 3, 64, 16), (4, 2, 32, 4), (8, 2, 128, 32), (6, 6, 24, 8)])
+def test_attention_mfma_rows_over_many_steps(ops, heads, kv_heads, dim, page_size):
+    """Decode form with many 32-key steps a wave (long contexts, few or no splits): the loop that keeps several steps'
+    loads in flight, with wave counts and splits that give a wave 1 to 35 steps, a far key that stands out, and a
+    window whose passed pages are gone from the table."""
+    lengths = [1100, 97, 705, 2]
+    qt, kt, vt, tables, rows = paged_case(heads, kv_heads, dim, page_size, lengths, torch.bfloat16, seed=3 * dim + heads, sharpen=(0, 5))
+    want = reference_attention(qt, kt, vt, tables, rows, page_size)
+    for splits in (1, 2, 5):
+        for waves in (4, 8):
+            got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, "rows", splits, waves=waves)
+            np.testing.assert_allclose(got, want, **MFMA_TOL, err_msg=f"splits={splits} waves={waves}")
+    window = 300
+    want_w = reference_attention(qt, kt, vt, tables, rows, page_size, window=window)
+    t2 = tables.clone()
+    first_needed = min(p + 1 - window for s, p in rows if s == 0 and p + 1 > window)      # request 0: rows at 1099 and 550
+    t2[0, :first_needed // page_size] = -1
+    only = [i for i, (s, p) in enumerate(rows) if not (s == 0 and p + 1 <= window)]       # (its row at 0 needs page 0)
+    for splits, waves in ((1, 8), (1, 4), (3, 8)):
+        got = run_mfma(ops, qt[only].contiguous(), kt, vt, t2, [rows[i] for i in only], page_size, "rows", splits, waves=waves, window=window)
+        np.testing.assert_allclose(got, want_w[only], **MFMA_TOL, err_msg=f"window, splits={splits} waves={waves}")
+
+
 def portion_case(heads, kv_heads, dim, page_size, plan, seed):
     """plan: [(cached keys before the portion, portion length)] per request: every row of every portion is a query."""
     rng = np.random.default_rng(seed)

@@ -530,6 +530,40 @@ def test_attention_square_tiles_over_long_contexts(ops, heads, kv_heads, dim, pa
         np.testing.assert_allclose(got, want_w, **MFMA_TOL, err_msg=f"window {window}")
 
 
+@pytest.mark.parametrize("dim, page_size", [(64, 16), (128, 16), (32, 8)])
+def test_attention_survives_scores_beyond_the_exponent_range(ops, dim, page_size):
+    """One key whose score lies a thousand powers of two above every score before it (the weights computed with the
+    old reference point overflow to infinity, which must be noticed and redone), and a prefix whose scores all lie far
+    below the first key's (weights that underflow to zero must stay harmless): every form of the kernel against the
+    plain softmax in float64."""
+    heads, kv_heads = 4, 2
+    plan = [(0, 200), (300, 70)]
+    qt, kt, vt, tables, rows = portion_case(heads, kv_heads, dim, page_size, plan, seed=5 * dim)
+    first = plan[0][1]
+    direction = torch.nn.functional.normalize(qt[first:, 0].float().mean(0), dim=0)
+    # request 1: key 330 (inside its portion) answers head 0 and 1 of every later row with a huge score
+    page, off = tables[1, 330 // page_size].item(), 330 % page_size
+    kt[page, 0, off, :] = (direction * 200).to(kt.dtype)
+    qt[first:, 0] = (qt[first:, 0].float() + direction * 30).to(qt.dtype)
+    qt[first:, 1] = qt[first:, 0]
+    # request 0: key 0 towers over all that follow for head 2 (kv head 1): their weights underflow
+    d0 = torch.nn.functional.normalize(qt[:first, 2].float().mean(0), dim=0)
+    page0 = tables[0, 0].item()
+    kt[page0, 1, 0, :] = (d0 * 200).to(kt.dtype)
+    qt[:first, 2] = (qt[:first, 2].float() + d0 * 30).to(qt.dtype)
+    want = reference_attention(qt, kt, vt, tables, rows, page_size)
+    assert np.isfinite(want).all()
+    modes = ["tiles", "block", "block2"] + list(square_modes(dim)) + (["tiles2"] if dim <= 64 else [])
+    for mode in modes:
+        got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, mode, positions_given=mode.startswith("square"))
+        assert np.isfinite(got).all(), mode
+        np.testing.assert_allclose(got, want, **MFMA_TOL, err_msg=mode)
+    for splits in (1, 3):
+        got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, "rows", splits)
+        assert np.isfinite(got).all()
+        np.testing.assert_allclose(got, want, **MFMA_TOL, err_msg=f"rows, splits={splits}")
+
+
 def test_attention_mfma_window_and_far_key(ops):
     qt, kt, vt, tables, rows = portion_case(4, 2, 32, 8, [(40, 30), (0, 9)], seed=21)
     for window in (1, 8, 9, 33, 64):

@@ -526,7 +526,9 @@ class ModelRunner:
                     n = self.square_tiles
                 elif span >= 1024 and blocks >= 512:
                     n = 4 if blocks >= 2048 and head_dim <= 64 else 2
-                elif span >= 2048 and blocks >= 256:
+                elif span >= 1024 and blocks >= 128:
+                    # (fewer blocks than compute units and a thousand keys: 64-item blocks, in two halves; 1,024 rows of
+                    # 12 heads of 128 take 25 us against 35 as LDS block tiles, of 16 heads of 64 over 4: 17 against 18)
                     n = 1
                 if n:
                     # about one block a compute unit: the time is the longest tile's chain of steps, which two halves a

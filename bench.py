@@ -164,6 +164,9 @@ def main():
     ap.add_argument("--sizes", default="smollm2-1.7b:8:4096,llama-3-8b:8:8192",
                     help="further layer sizes, measured with fewer layers than their configurations have: "
                          "preset:layers:context, comma separated (empty for none); batches 1, 8 and 64 and a prompt step each")
+    ap.add_argument("--contexts", default="7936:8192,32000:32768",
+                    help="longer contexts of the main model: prompt:context, comma separated (empty for none); batches 8 and "
+                         "64 and a prompt step each")
     ap.add_argument("--execution", default="graph", choices=["graph", "eager"])
     ap.add_argument("--overlap", type=int, default=1, choices=[0, 1],
                     help="1: picked tokens stay on the device and a step is launched before the tokens of the one "
@@ -195,7 +198,8 @@ def main():
     full_layers = raw["num_hidden_layers"]
     if args.layers:
         raw["num_hidden_layers"] = args.layers
-    raw["max_position_embeddings"] = max(raw["max_position_embeddings"], args.context)
+    longer = [tuple(int(x) for x in item.split(":")) for item in args.contexts.split(",") if item] if args.workload == "decode" else []
+    raw["max_position_embeddings"] = max([raw["max_position_embeddings"], args.context] + [context for _, context in longer])
     folder = tempfile.mkdtemp(prefix="bench-model-")
     write_random_model(folder, raw, seed=0, dtype="bfloat16")
     model = load_model(folder, dtype=args.dtype)
@@ -237,6 +241,20 @@ def main():
                    "ms_per_step_by_gpu_events": main_r["event_ms"]},
         "reference_b1_tokens_per_s": REFERENCE_B1_TOKS,
     }
+    # the same model at longer contexts: 8 and 64 requests after whole prompts, and the prompt step
+    contexts = {}
+    for prompt, context in longer:
+        torch.cuda.empty_cache()
+        n = steps_for(context, prompt)
+        r, pf2, flops2 = measure(model, args, [8, 64], prompt, context, n, args.warmup, repeats)
+        contexts[str(context)] = {"prompt_len": prompt, "steps": n,
+                                  **{f"decode_b{b}": round(r[b]["tokens_per_s"], 1) for b in r},
+                                  **{f"decode_b{b}_ms": round(r[b]["ms_per_step"], 4) for b in r},
+                                  **{f"decode_b{b}_hbm_frac": round(r[b]["gbps"] / HBM_GBPS, 5) for b in r},
+                                  "prefill_tokens_per_s": round(prompt / pf2, 1), "prefill_ms": round(pf2 * 1e3, 3),
+                                  "prefill_frac": round(flops2 / pf2 / peak, 5)}
+    if contexts:
+        line["contexts"] = contexts
     # further layer sizes, with fewer layers than their configurations have (both numbers named): random weights drawn
     # on the device, batches 1, 8 and 64 after 2,048-token prompts, and the prompt step
     del model

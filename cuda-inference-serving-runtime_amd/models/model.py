@@ -37,6 +37,18 @@ class Model:
                     raise ValueError(f"schedule entry {index} must read an earlier entry that keeps a cache")
                 if self.layers[entry.layer].mixer.cache_need() is not None:
                     raise ValueError(f"schedule entry {index} reads another cache but its mixer keeps one")
+                kept = self.layers[self.schedule[entry.reads].layer].mixer.cache_need()
+                reader = self.layers[entry.layer].mixer
+                wanted = reader.cache_read() if hasattr(reader, "cache_read") else None
+                if kept is None:
+                    raise ValueError(f"schedule entry {index} reads entry {entry.reads}, which keeps no cache")
+                if wanted is not None:
+                    if (wanted.kv_heads, wanted.head_dim) != (kept.kv_heads, kept.head_dim):
+                        raise ValueError(f"schedule entry {index} expects keys of {wanted.kv_heads} heads x {wanted.head_dim}, "
+                                         f"entry {entry.reads} keeps {kept.kv_heads} x {kept.head_dim}")
+                    if kept.window is not None and (wanted.window is None or wanted.window > kept.window):
+                        raise ValueError(f"schedule entry {index} looks back over {wanted.window or 'all'} keys, "
+                                         f"entry {entry.reads} keeps the last {kept.window}")
         self.dtype = None
         self.device = None
 

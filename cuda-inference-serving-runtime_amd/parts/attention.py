@@ -33,6 +33,9 @@ class PagedAttention(Mixer):
     def cache_need(self):
         return KVNeed(self.kv_heads, self.head_dim, self.window) if self.own_kv else None
 
+    def cache_read(self):
+        return None if self.own_kv else KVNeed(self.kv_heads, self.head_dim, self.window)
+
     def tensor_specs(self):
         n, H, D = self.name, self.hidden, self.head_dim
         specs = [TensorSpec(f"{n}.q_proj.weight", (self.heads * D, H))]

@@ -67,6 +67,12 @@ class Mixer(Part):
     def cache_need(self):
         return None
 
+    def cache_read(self):
+        """What a mixer that keeps no cache expects of the cache the order of layers lets it read (a KVNeed: heads,
+        head size, and the window it looks back over; None: it reads none, or cannot say).  The model checks it
+        against what the layer it reads keeps."""
+        return None
+
     def state_need(self):
         return None
 

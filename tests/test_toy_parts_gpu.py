@@ -433,3 +433,154 @@ def test_toy_position_encoding_with_interleaved_pairs(tmp_path, dtype):
     finally:
         unregister_part("position", "toy-neighbour-pairs")
         unregister_architecture("toy-pairs-lm")
+
+
+def build_shared_cache_toy():
+    """A norm of another law (centred, with a bias: nothing the product kernels can take over) and a layer whose
+    attention keeps no keys of its own and reads the cache of the layer before, both in one model beside the
+    framework's norm, attention and feed-forward."""
+    from runtime import register_part, make_part, register_architecture, TensorSpec
+    from runtime.config import unregister_architecture
+    from runtime.parts import Part, TokenEmbedding, LMHead, unregister_part
+    from runtime.models import Model, ScheduleEntry
+
+    class CentredNorm(Part):
+        """y = (x - mean) / sqrt(var + eps) * weight + bias over the row, in float."""
+
+        def __init__(self, name, dim, eps):
+            self.name, self.dim, self.eps = name, dim, eps
+
+        def tensor_specs(self):
+            return [TensorSpec(self.name + ".weight", (self.dim,), init="one_plus_normal"), TensorSpec(self.name + ".bias", (self.dim,))]
+
+        def bind(self, tensors, dtype):
+            self.weight, self.bias = tensors[self.name + ".weight"].float(), tensors[self.name + ".bias"].float()
+
+        def forward(self, x, ctx, rows=None, tag="norm"):
+            if rows is not None:
+                x = x[rows.long()]
+            centred = x - x.mean(-1, keepdim=True)
+            y = centred * torch.rsqrt(centred.square().mean(-1, keepdim=True) + self.eps) * self.weight + self.bias
+            out = ctx.buffer(tag, tuple(y.shape), ctx.dtype)
+            out.copy_(y)
+            return out
+
+    @dataclass(frozen=True)
+    class SharedConfig:
+        vocab_size: int
+        hidden_size: int
+        heads: int
+        kv_heads: int
+        head_dim: int
+        intermediate_size: int
+        rope_theta: float
+        max_position_embeddings: int
+        rms_norm_eps: float
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(*(raw[k] for k in ("vocab_size", "hidden_size", "heads", "kv_heads", "head_dim", "intermediate_size",
+                                          "rope_theta", "max_position_embeddings", "rms_norm_eps")))
+
+    def build(c):
+        def rms(n): return make_part("norm", "rmsnorm", name=n, dim=c.hidden_size, eps=c.rms_norm_eps)
+        def centred(n): return make_part("norm", "toy-centred", name=n, dim=c.hidden_size, eps=c.rms_norm_eps)
+        position = make_part("position", "rotary", head_dim=c.head_dim, theta=c.rope_theta, max_positions=c.max_position_embeddings)
+        def attention(n, own_kv):
+            return make_part("mixer", "attention", name=n, hidden=c.hidden_size, heads=c.heads, kv_heads=c.kv_heads,
+                             head_dim=c.head_dim, position=position, own_kv=own_kv)
+        def mlp(n): return make_part("ffn", "gated_mlp", name=n, hidden=c.hidden_size, intermediate=c.intermediate_size)
+        layers = [
+            make_part("block", "prenorm", mixer_norm=rms("l0.n1"), mixer=attention("l0.attn", True), ffn_norm=rms("l0.n2"), ffn=mlp("l0.mlp")),
+            make_part("block", "prenorm", mixer_norm=centred("l1.n1"), mixer=attention("l1.attn", False), ffn_norm=centred("l1.n2"), ffn=mlp("l1.mlp")),
+            make_part("block", "prenorm", mixer_norm=rms("l2.n1"), mixer=attention("l2.attn", True), ffn_norm=centred("l2.n2"), ffn=mlp("l2.mlp")),
+        ]
+        # the second layer reads the keys and values that the first one wrote
+        return Model(c, TokenEmbedding("embed", c.vocab_size, c.hidden_size), layers, centred("final"),
+                     LMHead("head", c.vocab_size, c.hidden_size),
+                     schedule=[ScheduleEntry(0), ScheduleEntry(1, reads=0), ScheduleEntry(2)])
+
+    register_part("norm", "toy-centred", CentredNorm)
+    register_architecture("toy-shared-cache-lm", SharedConfig, build)
+
+    def cleanup():
+        unregister_part("norm", "toy-centred")
+        unregister_architecture("toy-shared-cache-lm")
+    return cleanup
+
+
+def plain_shared_cache_toy(raw, w, tokens):
+    import plain_llama as P
+    eps, theta = raw["rms_norm_eps"], raw["rope_theta"]
+    nh, nkv, D = raw["heads"], raw["kv_heads"], raw["head_dim"]
+    T = len(tokens)
+    pos = np.arange(T)
+
+    def centred(x, p):
+        x = np.asarray(x, np.float64)
+        c = x - x.mean(-1, keepdims=True)
+        return c / np.sqrt((c * c).mean(-1, keepdims=True) + eps) * w[p + ".weight"] + w[p + ".bias"]
+
+    def mlp(h, p):
+        return P.linear(P.swiglu(P.linear(h, w[p + ".gate_proj.weight"]), P.linear(h, w[p + ".up_proj.weight"])), w[p + ".down_proj.weight"])
+
+    def keys_values(h, p):
+        k = P.rope(P.linear(h, w[p + ".k_proj.weight"]).reshape(T, nkv, D), pos, theta)
+        return k, P.linear(h, w[p + ".v_proj.weight"]).reshape(T, nkv, D)
+
+    def attend(h, p, k, v):
+        q = P.rope(P.linear(h, w[p + ".q_proj.weight"]).reshape(T, nh, D), pos, theta)
+        return P.linear(P.causal_attention(q, k, v).reshape(T, nh * D), w[p + ".o_proj.weight"])
+
+    x = np.asarray(w["embed.weight"], np.float64)[tokens]
+    h = P.rmsnorm(x, w["l0.n1.weight"], eps)
+    k0, v0 = keys_values(h, "l0.attn")
+    x = x + attend(h, "l0.attn", k0, v0)
+    x = x + mlp(P.rmsnorm(x, w["l0.n2.weight"], eps), "l0.mlp")
+    x = x + attend(centred(x, "l1.n1"), "l1.attn", k0, v0)          # its own queries over the first layer's keys and values
+    x = x + mlp(centred(x, "l1.n2"), "l1.mlp")
+    h = P.rmsnorm(x, w["l2.n1.weight"], eps)
+    k2, v2 = keys_values(h, "l2.attn")
+    x = x + attend(h, "l2.attn", k2, v2)
+    x = x + mlp(centred(x, "l2.n2"), "l2.mlp")
+    return P.linear(centred(x, "final"), w["head.weight"])
+
+
+@pytest.mark.parametrize("dtype, execution", [("float32", "eager"), ("bfloat16", "eager"), ("bfloat16", "graph")])
+def test_toy_norm_and_a_layer_that_reads_another_layers_cache(tmp_path, dtype, execution):
+    """A norm defined in this file (not one the product kernels can fuse) and an order of layers in which the second
+    keeps no cache and reads the first one's: registered, given random weights, loaded and stepped in portions beside
+    decoded tokens, against a plain implementation; only two of the three layers have pages."""
+    import plain_llama as P
+    from runtime.engine import load_model, ModelRunner, StepEntry
+    from runtime.engine.loading import build_from_config_dict
+    from runtime.weights import write_model_folder
+    cleanup = build_shared_cache_toy()
+    try:
+        raw = {"model_type": "toy-shared-cache-lm", "vocab_size": 67, "hidden_size": 40, "heads": 4, "kv_heads": 2, "head_dim": 16,
+               "intermediate_size": 56, "rope_theta": 5000.0, "max_position_embeddings": 128, "rms_norm_eps": 1e-5}
+        tmp_path.mkdir(exist_ok=True)
+        _, _, blueprint = build_from_config_dict(raw)
+        write_model_folder(tmp_path, raw, blueprint.tensor_specs(), seed=11, dtype=torch.float32 if dtype == "float32" else torch.bfloat16, std=0.15)
+        cfg, w = P.read_folder(tmp_path)
+        assert "l1.attn.k_proj.weight" not in w and "l1.attn.q_proj.weight" in w and "l1.n1.bias" in w
+        model = load_model(tmp_path, dtype=dtype)
+        assert set(model.cache_needs()) == {0, 2} and model.site_of(1) == 0
+        runner = ModelRunner(model, n_pages=14, page_size=8, max_requests=2, execution=execution)
+        tokens = {"x": np.random.default_rng(4).integers(0, 67, 41).tolist(), "y": np.random.default_rng(5).integers(0, 67, 19).tolist()}
+        want = {k: plain_shared_cache_toy(raw, w, v) for k, v in tokens.items()}
+        runner.create("x"); runner.create("y")
+        got, fed = {"x": [], "y": []}, {"x": 0, "y": 0}
+        plan = [[("x", 17), ("y", 3)], [("x", 1), ("y", 9)], [("x", 1), ("y", 1)], [("x", 1), ("y", 1)], [("x", 21), ("y", 5)]]
+        for step in plan:
+            entries = [StepEntry(k, tokens[k][fed[k]:fed[k] + n], list(range(n))) for k, n in step]
+            out = runner.step(entries).float().cpu().numpy()
+            row = 0
+            for k, n in step:
+                got[k].append(out[row:row + n]); row += n; fed[k] += n
+        from conftest import assert_close
+        for k in tokens:
+            assert_close(np.concatenate(got[k]), want[k], dtype, f"request {k}")
+        runner.cache.check()
+    finally:
+        cleanup()

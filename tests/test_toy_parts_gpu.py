@@ -584,3 +584,117 @@ def test_toy_norm_and_a_layer_that_reads_another_layers_cache(tmp_path, dtype, e
         runner.cache.check()
     finally:
         cleanup()
+
+
+def build_window_toy():
+    """Layers with different needs in one model: two whose attention looks back over a window of keys (they share a
+    group of pages, which are given back as the window passes them) around one that sees all keys (a group of its
+    own).  Only the framework's parts, put together here."""
+    from runtime import make_part, register_architecture
+    from runtime.config import unregister_architecture
+    from runtime.parts import TokenEmbedding, LMHead
+    from runtime.models import Model
+
+    @dataclass(frozen=True)
+    class WindowConfig:
+        vocab_size: int
+        hidden_size: int
+        heads: int
+        kv_heads: int
+        head_dim: int
+        window: int
+        intermediate_size: int
+        rope_theta: float
+        max_position_embeddings: int
+        rms_norm_eps: float
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(*(raw[k] for k in ("vocab_size", "hidden_size", "heads", "kv_heads", "head_dim", "window", "intermediate_size",
+                                          "rope_theta", "max_position_embeddings", "rms_norm_eps")))
+
+    def build(c):
+        def rms(n): return make_part("norm", "rmsnorm", name=n, dim=c.hidden_size, eps=c.rms_norm_eps)
+        position = make_part("position", "rotary", head_dim=c.head_dim, theta=c.rope_theta, max_positions=c.max_position_embeddings)
+        def layer(n, window):
+            return make_part("block", "prenorm", mixer_norm=rms(n + ".n1"),
+                             mixer=make_part("mixer", "attention", name=n + ".attn", hidden=c.hidden_size, heads=c.heads,
+                                             kv_heads=c.kv_heads, head_dim=c.head_dim, position=position, window=window),
+                             ffn_norm=rms(n + ".n2"),
+                             ffn=make_part("ffn", "gated_mlp", name=n + ".mlp", hidden=c.hidden_size, intermediate=c.intermediate_size))
+        return Model(c, TokenEmbedding("embed", c.vocab_size, c.hidden_size), [layer("l0", c.window), layer("l1", None), layer("l2", c.window)],
+                     rms("final"), LMHead("head", c.vocab_size, c.hidden_size))
+
+    register_architecture("toy-window-lm", WindowConfig, build)
+    return lambda: unregister_architecture("toy-window-lm")
+
+
+def plain_window_toy(raw, w, tokens):
+    import plain_llama as P
+    eps, theta, nh, nkv, D = raw["rms_norm_eps"], raw["rope_theta"], raw["heads"], raw["kv_heads"], raw["head_dim"]
+    T = len(tokens)
+    pos = np.arange(T)
+    x = np.asarray(w["embed.weight"], np.float64)[tokens]
+    for name, window in (("l0", raw["window"]), ("l1", None), ("l2", raw["window"])):
+        h = P.rmsnorm(x, w[name + ".n1.weight"], eps)
+        q = P.rope(P.linear(h, w[name + ".attn.q_proj.weight"]).reshape(T, nh, D), pos, theta)
+        k = P.rope(P.linear(h, w[name + ".attn.k_proj.weight"]).reshape(T, nkv, D), pos, theta)
+        v = P.linear(h, w[name + ".attn.v_proj.weight"]).reshape(T, nkv, D)
+        x = x + P.linear(P.causal_attention(q, k, v, window=window).reshape(T, nh * D), w[name + ".attn.o_proj.weight"])
+        h = P.rmsnorm(x, w[name + ".n2.weight"], eps)
+        x = x + P.linear(P.swiglu(P.linear(h, w[name + ".mlp.gate_proj.weight"]), P.linear(h, w[name + ".mlp.up_proj.weight"])),
+                         w[name + ".mlp.down_proj.weight"])
+    return P.linear(P.rmsnorm(x, w["final.weight"], eps), w["head.weight"])
+
+
+@pytest.mark.parametrize("dtype, execution", [("float32", "eager"), ("bfloat16", "eager"), ("bfloat16", "graph"), ("float32", "graph")])
+def test_layers_with_a_window_beside_layers_without_share_no_pages_and_give_theirs_back(tmp_path, dtype, execution):
+    """Two groups of pages in one model (a window of 20 keys; all keys).  Requests run in portions longer and
+    shorter than the window beside decoded tokens; the window group has far fewer pages than a request has keys,
+    so the pages that the window has passed are taken again, by the same request and by the other."""
+    import plain_llama as P
+    from conftest import assert_close
+    from runtime.engine import load_model, ModelRunner, StepEntry
+    from runtime.engine.loading import build_from_config_dict
+    from runtime.weights import write_model_folder
+    cleanup = build_window_toy()
+    try:
+        raw = {"model_type": "toy-window-lm", "vocab_size": 71, "hidden_size": 40, "heads": 6, "kv_heads": 2, "head_dim": 16,
+               "window": 20, "intermediate_size": 48, "rope_theta": 3000.0, "max_position_embeddings": 256, "rms_norm_eps": 1e-5}
+        tmp_path.mkdir(exist_ok=True)
+        _, _, blueprint = build_from_config_dict(raw)
+        write_model_folder(tmp_path, raw, blueprint.tensor_specs(), seed=13, dtype=torch.float32 if dtype == "float32" else torch.bfloat16, std=0.15)
+        cfg, w = P.read_folder(tmp_path)
+        model = load_model(tmp_path, dtype=dtype)
+        needs = model.cache_needs()
+        assert needs[0] == needs[2] and needs[0].window == 20 and needs[1].window is None
+        # 8 keys a page; the requests hold 150 + 61 keys: 27 pages where all keys stay
+        runner = ModelRunner(model, n_pages=28, page_size=8, max_requests=2, execution=execution)
+        groups = {g.need.window: g for g in runner.cache.groups}
+        assert set(groups) == {20, None} and len(groups[20].sites) == 2 and len(groups[None].sites) == 1
+        tokens = {"x": np.random.default_rng(6).integers(0, 71, 150).tolist(), "y": np.random.default_rng(7).integers(0, 71, 61).tolist()}
+        want = {k: plain_window_toy(raw, w, v) for k, v in tokens.items()}
+        runner.create("x"); runner.create("y")
+        got, fed = {"x": [], "y": []}, {"x": 0, "y": 0}
+        plan = [[("x", 45), ("y", 2)], [("x", 1), ("y", 7)], [("x", 1), ("y", 1)], [("x", 33), ("y", 1)], [("x", 2), ("y", 30)],
+                [("x", 1), ("y", 1)], [("x", 50), ("y", 1)], [("x", 1), ("y", 17)], [("x", 16), ("y", 1)]]
+        most_window_pages = 0
+        for step in plan:
+            entries = [StepEntry(k, tokens[k][fed[k]:fed[k] + n], list(range(n))) for k, n in step]
+            out = runner.step(entries).float().cpu().numpy()
+            row = 0
+            for k, n in step:
+                got[k].append(out[row:row + n]); row += n; fed[k] += n
+            runner.cache.check()
+            most_window_pages = max(most_window_pages, groups[20].pool.used)
+        assert fed == {k: len(v) for k, v in tokens.items()}
+        for k in tokens:
+            assert_close(np.concatenate(got[k]), want[k], dtype, f"request {k}")
+        # the window group never held more than a window and a portion a request (here: 20 + 50 and 20 + 30 keys, 8 a page)
+        assert most_window_pages <= 9 + 7 + 2, most_window_pages
+        assert groups[None].pool.used == 19 + 8
+        runner.release("x"); runner.release("y")
+        runner.cache.check()
+        assert all(g.pool.used == 0 for g in runner.cache.groups)
+    finally:
+        cleanup()

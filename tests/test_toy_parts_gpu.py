@@ -698,3 +698,104 @@ def test_layers_with_a_window_beside_layers_without_share_no_pages_and_give_thei
         assert all(g.pool.used == 0 for g in runner.cache.groups)
     finally:
         cleanup()
+
+
+def build_partial_rotary_toy():
+    """The framework's attention with other constants than the architecture's: a rotary embedding that turns only the
+    first 8 of a head's 24 coordinates, and a score scale that is not 1/sqrt(head size); the second layer is plain."""
+    from runtime import make_part, register_architecture
+    from runtime.config import unregister_architecture
+    from runtime.parts import TokenEmbedding, LMHead
+    from runtime.models import Model
+
+    @dataclass(frozen=True)
+    class PartialConfig:
+        vocab_size: int
+        hidden_size: int
+        rotary_dim: int
+        score_scale: float
+        rope_theta: float
+        max_position_embeddings: int
+        rms_norm_eps: float
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(*(raw[k] for k in ("vocab_size", "hidden_size", "rotary_dim", "score_scale", "rope_theta",
+                                          "max_position_embeddings", "rms_norm_eps")))
+
+    def build(c):
+        def rms(n): return make_part("norm", "rmsnorm", name=n, dim=c.hidden_size, eps=c.rms_norm_eps)
+        partial = make_part("position", "rotary", head_dim=24, theta=c.rope_theta, max_positions=c.max_position_embeddings, rotary_dim=c.rotary_dim)
+        whole = make_part("position", "rotary", head_dim=24, theta=c.rope_theta, max_positions=c.max_position_embeddings)
+        def layer(n, position, scale):
+            return make_part("block", "prenorm", mixer_norm=rms(n + ".n1"),
+                             mixer=make_part("mixer", "attention", name=n + ".attn", hidden=c.hidden_size, heads=3, kv_heads=3,
+                                             head_dim=24, position=position, scale=scale),
+                             ffn_norm=rms(n + ".n2"),
+                             ffn=make_part("ffn", "gated_mlp", name=n + ".mlp", hidden=c.hidden_size, intermediate=40))
+        return Model(c, TokenEmbedding("embed", c.vocab_size, c.hidden_size), [layer("l0", partial, c.score_scale), layer("l1", whole, None)],
+                     rms("final"), LMHead("head", c.vocab_size, c.hidden_size))
+
+    register_architecture("toy-partial-rotary-lm", PartialConfig, build)
+    return lambda: unregister_architecture("toy-partial-rotary-lm")
+
+
+def plain_partial_rotary_toy(raw, w, tokens):
+    import plain_llama as P
+    eps, theta, rot, scale = raw["rms_norm_eps"], raw["rope_theta"], raw["rotary_dim"], raw["score_scale"]
+    T, nh, D = len(tokens), 3, 24
+    pos = np.arange(T)
+    x = np.asarray(w["embed.weight"], np.float64)[tokens]
+    for name, turned, s in (("l0", rot, scale), ("l1", D, 1 / np.sqrt(D))):
+        h = P.rmsnorm(x, w[name + ".n1.weight"], eps)
+        q = P.linear(h, w[name + ".attn.q_proj.weight"]).reshape(T, nh, D)
+        k = P.linear(h, w[name + ".attn.k_proj.weight"]).reshape(T, nh, D)
+        v = P.linear(h, w[name + ".attn.v_proj.weight"]).reshape(T, nh, D)
+        # the first `turned` coordinates turn (pairs (i, i + turned/2) by pos * theta^(-2i/turned)), the rest pass
+        q = np.concatenate([P.rope(q[..., :turned], pos, theta), q[..., turned:]], axis=-1)
+        k = np.concatenate([P.rope(k[..., :turned], pos, theta), k[..., turned:]], axis=-1)
+        q = q * (s * np.sqrt(D))                                   # the plain attention divides by sqrt(D)
+        x = x + P.linear(P.causal_attention(q, k, v).reshape(T, nh * D), w[name + ".attn.o_proj.weight"])
+        h = P.rmsnorm(x, w[name + ".n2.weight"], eps)
+        x = x + P.linear(P.swiglu(P.linear(h, w[name + ".mlp.gate_proj.weight"]), P.linear(h, w[name + ".mlp.up_proj.weight"])),
+                         w[name + ".mlp.down_proj.weight"])
+    return P.linear(P.rmsnorm(x, w["final.weight"], eps), w["head.weight"])
+
+
+@pytest.mark.parametrize("dtype, execution", [("float32", "eager"), ("bfloat16", "eager"), ("bfloat16", "graph")])
+def test_attention_with_a_partial_rotary_embedding_and_a_scale_of_its_own(tmp_path, dtype, execution):
+    """The constants of a part are its parameters: a head of 24 coordinates (not a power of two) of which 8 turn, and
+    scores scaled by 0.31, through the framework's attention in portions beside decoded tokens."""
+    import plain_llama as P
+    from conftest import assert_close
+    from runtime.engine import load_model, ModelRunner, StepEntry
+    from runtime.engine.loading import build_from_config_dict
+    from runtime.weights import write_model_folder
+    cleanup = build_partial_rotary_toy()
+    try:
+        raw = {"model_type": "toy-partial-rotary-lm", "vocab_size": 59, "hidden_size": 48, "rotary_dim": 8, "score_scale": 0.31,
+               "rope_theta": 700.0, "max_position_embeddings": 96, "rms_norm_eps": 1e-6}
+        tmp_path.mkdir(exist_ok=True)
+        _, _, blueprint = build_from_config_dict(raw)
+        write_model_folder(tmp_path, raw, blueprint.tensor_specs(), seed=17, dtype=torch.float32 if dtype == "float32" else torch.bfloat16, std=0.15)
+        cfg, w = P.read_folder(tmp_path)
+        model = load_model(tmp_path, dtype=dtype)
+        runner = ModelRunner(model, n_pages=16, page_size=8, max_requests=2, execution=execution)
+        tokens = {"x": np.random.default_rng(8).integers(0, 59, 44).tolist(), "y": np.random.default_rng(9).integers(0, 59, 23).tolist()}
+        want = {k: plain_partial_rotary_toy(raw, w, v) for k, v in tokens.items()}
+        runner.create("x"); runner.create("y")
+        got, fed = {"x": [], "y": []}, {"x": 0, "y": 0}
+        for step in [[("x", 19), ("y", 2)], [("x", 1), ("y", 11)], [("x", 1), ("y", 1)], [("x", 23), ("y", 9)]]:
+            entries = [StepEntry(k, tokens[k][fed[k]:fed[k] + n], list(range(n))) for k, n in step]
+            out = runner.step(entries).float().cpu().numpy()
+            row = 0
+            for k, n in step:
+                got[k].append(out[row:row + n]); row += n; fed[k] += n
+        for k in tokens:
+            assert_close(np.concatenate(got[k]), want[k], dtype, f"request {k}")
+        # both constants matter: with all 24 coordinates turned, or with the usual scale, the logits are others
+        assert np.abs(plain_partial_rotary_toy(dict(raw, rotary_dim=24), w, tokens["x"]) - want["x"]).max() > 1e-3
+        assert np.abs(plain_partial_rotary_toy(dict(raw, score_scale=1 / np.sqrt(24)), w, tokens["x"]) - want["x"]).max() > 1e-3
+        runner.cache.check()
+    finally:
+        cleanup()

@@ -799,3 +799,45 @@ def test_attention_with_a_partial_rotary_embedding_and_a_scale_of_its_own(tmp_pa
         runner.cache.check()
     finally:
         cleanup()
+
+
+@pytest.mark.parametrize("execution, overlap", [("eager", False), ("graph", True)])
+def test_scheduler_generates_with_a_model_of_two_page_groups(tmp_path, execution, overlap):
+    """The entry point over the model with windowed and full layers: requests admitted by what each group of pages
+    can promise, prompts cut into portions, greedy tokens equal to the plain implementation's, every page given back."""
+    import plain_llama as P
+    from runtime.engine.loading import build_from_config_dict
+    from runtime.engine.scheduler import Engine
+    from runtime.weights import write_model_folder
+    cleanup = build_window_toy()
+    try:
+        raw = {"model_type": "toy-window-lm", "vocab_size": 71, "hidden_size": 40, "heads": 6, "kv_heads": 2, "head_dim": 16,
+               "window": 20, "intermediate_size": 48, "rope_theta": 3000.0, "max_position_embeddings": 256, "rms_norm_eps": 1e-5}
+        tmp_path.mkdir(exist_ok=True)
+        _, _, blueprint = build_from_config_dict(raw)
+        write_model_folder(tmp_path, raw, blueprint.tensor_specs(), seed=13, dtype=torch.float32, std=0.3)
+        cfg, w = P.read_folder(tmp_path)
+        prompts = [np.random.default_rng(20 + i).integers(0, 71, n).tolist() for i, n in enumerate((37, 5, 52, 18))]
+
+        def plain_greedy(prompt, steps):
+            tokens, new = list(prompt), []
+            for _ in range(steps):
+                row = plain_window_toy(raw, w, tokens)[-1]
+                top = np.sort(row)[-2:]
+                assert top[1] - top[0] > 1e-3, "a near-tie in the plain logits: choose other weights"
+                new.append(int(row.argmax())); tokens.append(new[-1])
+            return new
+
+        want = [plain_greedy(p, 9) for p in prompts]
+        engine = Engine.from_folder(tmp_path, dtype="float32", pages=12, page_size=8, execution=execution, max_active=3,
+                                    token_budget=24, prefill_chunk=16, policy="decode_first", overlap=overlap)
+        got = engine.generate(prompts, max_new_tokens=9)
+        assert got == want
+        cache = engine.runner.cache
+        cache.check()
+        assert all(g.pool.used == 0 for g in cache.groups) and len(cache.groups) == 2
+        # 12 pages of 8 keys a group: the longest request (52 + 8 keys) takes 8 of the group that keeps all keys, so
+        # the four requests cannot all have been live at once
+        assert max(step["active"] for step in engine.trace) <= 3
+    finally:
+        cleanup()

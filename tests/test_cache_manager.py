@@ -314,3 +314,32 @@ def test_pages_that_fit_the_free_memory():
     assert pages_that_fit({0: None}, 16, 2, 5) == 1                          # no site keeps keys: nothing to size
     with pytest.raises(MemoryError):
         pages_that_fit(needs, 16, 2, per_page - 1, fraction=1.0)
+
+
+def test_fork_of_a_request_whose_window_has_passed_pages():
+    """A fork copies the block tables as they are: the places of pages that a window has passed stay empty in the copy,
+    the live pages are shared, the page being written is copied once by whoever writes first, and both requests go on
+    giving pages back as their windows move."""
+    window = KVNeed(1, 8, window=8)
+    m = CacheManager({0: KVNeed(1, 8), 1: window}, {KVNeed(1, 8): 40, window: 12}, 4, 4)
+    m.create("a")
+    for n in (13, 1, 1, 9, 1):
+        m.append_many([("a", n)])
+        m.check()
+    full, windowed = m.groups
+    assert windowed.tables["a"][:4] == [-1] * 4 and all(p >= 0 for p in windowed.tables["a"][4:])
+    m.fork("a", "b")
+    m.check()
+    assert windowed.tables["b"] == windowed.tables["a"] and full.tables["b"] == full.tables["a"]
+    shared = [p for p in windowed.tables["a"] if p >= 0]
+    assert all(windowed.pool.refs[p] == 2 for p in shared)
+    for n in (1, 1, 6, 1):
+        m.append_many([("a", n), ("b", n)])
+        m.check()
+    # position 25 was in a shared page of both groups: one of the two got a copy, the other kept the page
+    assert full.tables["a"][6] != full.tables["b"][6] and full.tables["a"][:6] == full.tables["b"][:6]
+    assert windowed.tables["a"].count(-1) == windowed.tables["b"].count(-1) == 6
+    assert not set(p for p in windowed.tables["a"] if p >= 0) & set(p for p in windowed.tables["b"] if p >= 0)
+    m.release("a"); m.check()
+    m.release("b"); m.check()
+    assert [g.pool.used for g in m.groups] == [0, 0]

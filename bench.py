@@ -147,6 +147,27 @@ def copy_bandwidth():
     return 2 * n / statistics.median(times) / 1e9
 
 
+def read_bandwidth():
+    """GB/s of a kernel that reads 2 GiB once and does nothing else (the library's own stream_read), the median of
+    five: what decode steps, which read weights and cache and write next to nothing, could get from this GPU."""
+    import statistics
+    import torch
+    from runtime.kernels import ops
+    n = 2 << 30
+    a = torch.empty(n, dtype=torch.uint8, device="cuda")
+    a.zero_()
+    sink = torch.zeros(1, dtype=torch.int32, device="cuda")
+    ops.stream_read(a, sink)
+    times = []
+    for _ in range(5):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        ops.stream_read(a, sink)
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t0)
+    return n / statistics.median(times) / 1e9
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -218,6 +239,7 @@ def main():
     main_r = results[args.batch]
     peak = PEAK_TFLOPS["bf16" if args.dtype == "bfloat16" else "fp32"] * 1e12
     copy_gbps = copy_bandwidth()
+    read_gbps = read_bandwidth()
     matmul_tflops = library_matmul_tflops()
     points = {f"decode_b{b}": round(results[b]["tokens_per_s"], 1) for b in batches if b != args.batch}
     line = {
@@ -234,7 +256,7 @@ def main():
                     "frac": round(pf_flops / pf / peak, 5), "peak_tflops": peak / 1e12,
                     "measured_library_matmul_tflops": round(matmul_tflops, 1)},
         "roofline": {"bound": "hbm", "achieved": round(main_r["gbps"], 1), "peak": HBM_GBPS, "unit": "GB/s",
-                     "frac": round(main_r["gbps"] / HBM_GBPS, 5), "measured_copy": round(copy_gbps, 1)},
+                     "frac": round(main_r["gbps"] / HBM_GBPS, 5), "measured_copy": round(copy_gbps, 1), "measured_read": round(read_gbps, 1)},
         "points": points,
         "points_roofline_frac": {f"decode_b{b}": round(results[b]["gbps"] / HBM_GBPS, 5) for b in batches if b != args.batch},
         "method": {"repeats": repeats, "statistic": "median", "ms_per_step_of_repeats": main_r["ms_all"], "clock": "host, synchronised",

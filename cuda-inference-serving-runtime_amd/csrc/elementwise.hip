@@ -634,3 +634,32 @@ extern "C" int cisr_idle(int blocks, hipStream_t stream) {
     idle_kernel<<<(unsigned)blocks, 256, 0, stream>>>();
     return CISR_LAUNCH_CHECK();
 }
+
+// A kernel that only reads: every block walks a contiguous run of 16-byte words, eight loads a lane in flight, and
+// folds them into one word that is written only if it has a value no data gives.  What this GPU's memory gives a
+// kernel that streams weights and does nothing else (the benchmark reports it beside the published peak).
+typedef unsigned int read_word_t __attribute__((ext_vector_type(4)));
+__global__ void __launch_bounds__(256) stream_read_kernel(const read_word_t* __restrict__ src, long long words, unsigned* __restrict__ sink) {
+    const long long per = words / gridDim.x;                       // (a remainder of fewer words than blocks is left out)
+    const read_word_t* p = src + (long long)blockIdx.x * per;
+    read_word_t acc = {0u, 0u, 0u, 0u};
+    constexpr int U = 8;
+    long long i = threadIdx.x;
+    for (; i + (long long)(U - 1) * 256 < per; i += (long long)U * 256) {
+        read_word_t v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) v[u] = __builtin_nontemporal_load(p + i + (long long)u * 256);
+#pragma unroll
+        for (int u = 0; u < U; ++u) acc ^= v[u];
+    }
+    for (; i < per; i += 256) acc ^= p[i];
+    if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x9e3779b9u && sink) sink[0] = acc.x;
+}
+
+// Reads `bytes` (a multiple of 16, 16-byte aligned) once with `blocks` blocks; `sink`: 4 bytes that are hardly ever written.
+extern "C" int cisr_stream_read(const void* src, long long bytes, void* sink, int blocks, hipStream_t stream) {
+    if (bytes <= 0 || blocks <= 0) return 0;
+    if (bytes % 16 || ((uintptr_t)src) % 16 || !sink) return (int)hipErrorInvalidValue;
+    stream_read_kernel<<<(unsigned)blocks, 256, 0, stream>>>((const read_word_t*)src, bytes / 16, (unsigned*)sink);
+    return CISR_LAUNCH_CHECK();
+}

@@ -48,6 +48,7 @@ def _declare(h):
         "cisr_page_copy": [p, p, p, i, i, ll, ll, p],
         "cisr_f32_to_bf16": [p, p, ll, p],
         "cisr_idle": [i, p],
+        "cisr_stream_read": [p, ll, p, i, p],
         "cisr_attn_rowwise": [p, i, p, p, p, p, p, p, p, p, i, i, i, i, i, i, i, f, i, i, p],
         "cisr_gemm_f32": [p, i, p, i, p, i, p, i, i, i, i, p],
         "cisr_gemm_bf16": [p, i, p, i, p, i, p, i, i, i, i, i, p],
@@ -270,6 +271,15 @@ def f32_to_bf16(x, out):
 def idle(blocks=1):
     """Launches a kernel of `blocks` blocks that does nothing (the cost of a launch, for measurement)."""
     _check(lib().cisr_idle(int(blocks), _stream()), "idle")
+
+
+def stream_read(buffer, sink, blocks=512):
+    """Reads every byte of `buffer` once and keeps nothing (the read bandwidth of the memory, for measurement).
+    `sink`: a GPU tensor of at least 4 bytes."""
+    nbytes = buffer.numel() * buffer.element_size()
+    if not buffer.is_contiguous() or nbytes % 16 or buffer.data_ptr() % 16:
+        raise KernelError("stream_read: a contiguous buffer of a multiple of 16 bytes, 16-byte aligned")
+    _check(lib().cisr_stream_read(buffer.data_ptr(), nbytes, _dev(sink, "sink"), int(blocks), _stream()), "stream_read")
 
 
 def attention_rowwise(q, q_row_stride, kcache, vcache, tables, seg_of_row, positions, out, heads, kv_heads, dim,

@@ -636,6 +636,19 @@ def test_attention_mfma_ignores_what_unseen_slots_hold(ops):
         kt[0], vt[0] = k0, v0
 
 
+def test_stream_read_reads_and_writes_nothing(ops):
+    """The read-bandwidth probe of the benchmark: any size that is a multiple of 16 bytes, any number of blocks; it
+    leaves its sink alone (the folded word never has the value that would be written)."""
+    sink = torch.zeros(4, dtype=torch.int32, device=DEV)
+    for nbytes, blocks in ((16, 1), (4096, 3), (1 << 20, 512), (16 * 100003, 7), (48, 256)):
+        buf = torch.arange(nbytes, dtype=torch.int64, device=DEV).to(torch.uint8)
+        ops.stream_read(buf, sink, blocks)
+    torch.cuda.synchronize()
+    assert (sink == 0).all()
+    with pytest.raises(ops.KernelError):
+        ops.stream_read(torch.zeros(24, dtype=torch.uint8, device=DEV), sink)
+
+
 def test_gemm_skinny_and_fused_swiglu(ops):
     """Few rows of bf16 run the weight-streaming kernel: every row count up to 64, output widths off
     the 16-column tile, float/bf16 outputs, residual, and the fused SwiGLU against the two-kernel path."""

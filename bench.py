@@ -309,7 +309,9 @@ def main():
 def launch_floor(args):
     """Microseconds a kernel of a captured chain costs when it computes nothing: 1,000 launches of an empty kernel
     (one block, and one block a compute unit) in one graph, replayed; the median of 20 replays.  A decode step of
-    L layers is 5 L + 5 kernels, so this times that count is the part of a step that no kernel work can remove."""
+    L layers is 5 L + 4 kernels, so this times that count is the part of a step that no kernel work can remove.
+    Beside it, what the other way to order a step's parts costs: a meeting of all blocks inside one kernel (counters
+    in memory, 200 meetings, the median of 5 runs), alone and with 8 x 576 floats passed from all blocks to all."""
     import statistics
     import torch
     from runtime.config import preset
@@ -333,8 +335,22 @@ def launch_floor(args):
             torch.cuda.synchronize()
             times.append(time.perf_counter() - t0)
         out[name] = round(statistics.median(times[3:]) / chain * 1e6, 3)
+    # a meeting of all blocks inside one kernel, which a step fused into fewer kernels would need instead of a launch
+    meeting = {}
+    for name, blocks, exchange in (("128_blocks", 128, 0), ("256_blocks", 256, 0), ("256_blocks_passing_18_kb", 256, 8 * 576)):
+        rounds, times = 200, []
+        for _ in range(5 + 1):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            words = ops.grid_meet(blocks, rounds, exchange)
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t0)
+            if int(words[-1]) or int(words[0]) != rounds * (blocks // 32):
+                raise SystemExit(f"grid_meet: {blocks} blocks did not all meet ({int(words[0])} arrivals, flag {int(words[-1])})")
+        meeting[name] = round(statistics.median(times[1:]) / rounds * 1e6, 2)
+    out["meeting_inside_a_kernel"] = meeting
     layers = preset(args.model)["num_hidden_layers"]
-    kernels = 5 * layers + 5
+    kernels = 5 * layers + 4
     print(json.dumps({"metric": "microseconds a kernel that does nothing costs in a captured chain", "value": out["one_block"],
                       "unit": "us", "higher_is_better": False, "n_gpus": 1, "chain": chain, "replays": 20, "us_per_kernel": out,
                       "kernels_of_a_decode_step": kernels, "model": args.model,

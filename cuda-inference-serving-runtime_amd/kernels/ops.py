@@ -49,6 +49,7 @@ def _declare(h):
         "cisr_f32_to_bf16": [p, p, ll, p],
         "cisr_idle": [i, p],
         "cisr_stream_read": [p, ll, p, i, p],
+        "cisr_grid_meet": [p, p, i, i, i, C.c_uint, p],
         "cisr_attn_rowwise": [p, i, p, p, p, p, p, p, p, p, i, i, i, i, i, i, i, f, i, i, p],
         "cisr_gemm_f32": [p, i, p, i, p, i, p, i, i, i, i, p],
         "cisr_gemm_bf16": [p, i, p, i, p, i, p, i, i, i, i, i, p],
@@ -280,6 +281,21 @@ def stream_read(buffer, sink, blocks=512):
     if not buffer.is_contiguous() or nbytes % 16 or buffer.data_ptr() % 16:
         raise KernelError("stream_read: a contiguous buffer of a multiple of 16 bytes, 16-byte aligned")
     _check(lib().cisr_stream_read(buffer.data_ptr(), nbytes, _dev(sink, "sink"), int(blocks), _stream()), "stream_read")
+
+
+def grid_meet(blocks, rounds, exchange=0, spin_limit=1 << 22):
+    """One kernel of `blocks` blocks (a multiple of 32, at most 512) that all meet `rounds` times, passing `exchange`
+    floats through memory at each meeting (what a barrier over the whole grid costs beside a launch, for measurement).
+    Returns the words it counted in: [0] the number of groups of 32 blocks that arrived, over all rounds, [-1] is set
+    when a block gave up waiting after `spin_limit` polls."""
+    if blocks <= 0 or blocks % 32 or blocks > 512 or rounds * blocks >= 1 << 31 or exchange < 0:
+        raise KernelError(f"grid_meet: {blocks} blocks must be a multiple of 32, at most 512, and {rounds} rounds few enough to count")
+    device = torch.device("cuda", torch.cuda.current_device())
+    words = torch.zeros(1024, dtype=torch.int32, device=device)
+    passed = torch.empty(max(2 * exchange, 1), dtype=torch.float32, device=device)
+    _check(lib().cisr_grid_meet(words.data_ptr(), passed.data_ptr(), int(exchange), int(blocks), int(rounds), int(spin_limit),
+                                _stream()), "grid_meet")
+    return words
 
 
 def attention_rowwise(q, q_row_stride, kcache, vcache, tables, seg_of_row, positions, out, heads, kv_heads, dim,

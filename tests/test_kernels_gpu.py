@@ -1211,3 +1211,19 @@ def test_kernels_refuse_what_they_cannot_take(ops):
         ops.rmsnorm(rnd(2, 8), rnd(9), torch.empty(2, 8, device=DEV), 1e-5)
     with pytest.raises(KernelError):
         ops.embedding(torch.zeros(2, dtype=torch.int64, device=DEV), rnd(4, 8), torch.empty(2, 8, device=DEV))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("blocks,exchange", [(32, 0), (256, 0), (96, 500)])
+def test_grid_meet_counts_every_group_every_round(ops, blocks, exchange):
+    from runtime.kernels.ops import KernelError
+    rounds = 50
+    words = ops.grid_meet(blocks, rounds, exchange)
+    torch.cuda.synchronize()
+    assert int(words[-1]) == 0                              # no block gave up waiting
+    assert int(words[0]) == rounds * (blocks // 32)         # every group arrived in every round
+    groups = blocks // 32
+    for g in range(groups):
+        assert int(words[16 * (1 + g)]) == rounds * 32
+    with pytest.raises(KernelError, match="multiple of 32"):
+        ops.grid_meet(48, 1)

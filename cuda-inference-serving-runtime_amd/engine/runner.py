@@ -66,7 +66,7 @@ class ModelRunner:
         self.execution = execution
         self.programs, self.program_capacity = {}, 16
         self.block_tiles = None    # long portions through LDS-shared tiles of 64 x this items: None = by the number of blocks
-        # long portions of long contexts through 32 x 32 tiles, 64 x this items a block (1, 2, 4): None = by size, 0 = never
+        # long portions of long contexts through 32 x 32 tiles, 64 x this items a block (1, 2, 3, 4): None = by size, 0 = never
         self.square_tiles = int(os.environ["CISR_SQUARE_TILES"]) if os.environ.get("CISR_SQUARE_TILES") else None
         self.square_halves = None  # two halves a block in that form (even and odd steps): None = by the number of blocks, 1, 2
         self.tile_waves = int(os.environ.get("CISR_TILE_WAVES", "4"))   # wavefronts that share one tile's keys
@@ -525,7 +525,11 @@ class ModelRunner:
                 if self.square_tiles is not None:
                     n = self.square_tiles
                 elif span >= 1024 and blocks >= 512:
-                    n = 4 if blocks >= 2048 and head_dim <= 64 else 2
+                    # from 2,048 blocks of 64 items on: 192 items, six computing waves beside the two that copy (eight waves:
+                    # a compute unit holds two such blocks with small heads, one with large, and no wave slot stays empty).
+                    # 32 heads of 64 at 16k rows: 1.42 ms against 1.46 with 256 items and 1.54 with 128; 9 heads over 3 at
+                    # 32k: 1.49 against 1.58 and 1.61; 32 heads of 128 over 8 at 8k: 0.60 against 0.63 with 128 items
+                    n = 3 if blocks >= 2048 else 2
                 elif span >= 1024 and blocks >= 128:
                     # (fewer blocks than compute units and a thousand keys: 64-item blocks, in two halves; 1,024 rows of
                     # 12 heads of 128 take 25 us against 35 as LDS block tiles, of 16 heads of 64 over 4: 17 against 18)

@@ -675,7 +675,7 @@ def attention_mfma(q, q_row_stride, kcache, vcache, tables, seg_of_row, position
     fn = _attention_entry(dpad)
     po = pm = tp = None
     if tasks is not None:
-        if item_tiles not in ((1, 2, 4) if block_tiles == 32 else (1, 2)) or (item_tiles == 2 and dim > 64 and not block_tiles):
+        if item_tiles not in ((1, 2, 3, 4) if block_tiles == 32 else (1, 2)) or (item_tiles == 2 and dim > 64 and not block_tiles):
             raise KernelError("attention_mfma: two item tiles a wave need a head size of at most 64")
         if block_tiles and dpad > 128:
             raise KernelError("attention_mfma: block tiles need a head size of at most 128")
@@ -687,11 +687,11 @@ def attention_mfma(q, q_row_stride, kcache, vcache, tables, seg_of_row, position
                 raise KernelError("attention_mfma: the output must be fewer than 2^31 elements (32-bit offsets)")
             if page_size < 8 or dpad > 128:
                 raise KernelError("attention_mfma: 32 x 32 block tiles need pages of at least 8 keys and a head size of at most 128")
-            if key_groups not in (1, 2) or (key_groups == 2 and item_tiles == 4):
+            if key_groups not in (1, 2) or (key_groups == 2 and item_tiles >= 3):
                 raise KernelError("attention_mfma: one or two key groups, two with 64 or 128 items a block")
             if dpad > 64 and (item_tiles == 4 or (item_tiles == 2 and key_groups == 2)):
                 raise KernelError("attention_mfma: blocks of more than eight waves need a head size of at most 64")
-            mode = {(1, 1): 6, (2, 1): 5, (4, 1): 7, (1, 2): 8, (2, 2): 9}[(item_tiles, key_groups)]
+            mode = {(1, 1): 6, (2, 1): 5, (3, 1): 10, (4, 1): 7, (1, 2): 8, (2, 2): 9}[(item_tiles, key_groups)]
         tp = _dev(tasks, "tasks", torch.int32, (n_tasks, 4))
     else:
         n_tasks, mode = rows, 1

@@ -405,7 +405,7 @@ def test_long_portions_through_block_tiles_match_the_plain_model(folders, name, 
 
 
 @pytest.mark.parametrize("name", ["a", "c"])
-@pytest.mark.parametrize("square, halves", [(1, 1), (2, 1), (4, 1), (1, 2), (2, 2)])
+@pytest.mark.parametrize("square, halves", [(1, 1), (2, 1), (3, 1), (4, 1), (1, 2), (2, 2)])
 def test_long_portions_through_square_tiles_match_the_plain_model(folders, name, square, halves):
     """Long portions of long contexts run on the 32 x 32 matrix instruction with waves of their own for the copies;
     forced here on small models: a whole prompt, then a second portion beside another request, then graph replays."""

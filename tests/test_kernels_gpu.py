@@ -376,7 +376,7 @@ def run_mfma(ops, qt, kt, vt, tables, rows, page_size, mode, splits=1, window=No
     tasks = None
     ws = (torch.empty(T * heads * splits * dim, device=DEV), torch.empty(T * heads * splits * 2, device=DEV))
     # ("square...": blocks on the 32 x 32 instruction; "...halves": two halves a block for the even and the odd steps)
-    items_of = {"tiles": 16, "tiles2": 32, "block": 64, "block2": 128, "square": 64, "square2": 128, "square4": 256,
+    items_of = {"tiles": 16, "tiles2": 32, "block": 64, "block2": 128, "square": 64, "square2": 128, "square3": 192, "square4": 256,
                 "square_halves": 64, "square2_halves": 128}
     if mode in items_of:
         group = heads // kv_heads
@@ -392,7 +392,7 @@ def run_mfma(ops, qt, kt, vt, tables, rows, page_size, mode, splits=1, window=No
     ops.attention_mfma(qt.reshape(T, heads * dim), heads * dim, kt, vt, tables, seg, pos, out, heads, kv_heads, dim,
                        page_size, window, scale if scale is not None else 1 / math.sqrt(dim), tasks, splits, ws, waves,
                        block_tiles=32 if mode.startswith("square") else mode.startswith("block"),
-                       item_tiles=(4 if mode == "square4" else 2 if mode in ("tiles2", "block2", "square2", "square2_halves") else 1),
+                       item_tiles=(4 if mode == "square4" else 3 if mode == "square3" else 2 if mode in ("tiles2", "block2", "square2", "square2_halves") else 1),
                        key_groups=2 if mode.endswith("_halves") else 1,
                        row_ids=None if row_ids is None else torch.tensor(row_ids, dtype=torch.int32, device=DEV))
     return f64(out).reshape(T, heads, dim)
@@ -403,7 +403,7 @@ MFMA_TOL = dict(rtol=2e-2, atol=2e-2)
 
 def square_modes(dim):
     """The forms of the 32 x 32 kernel that take this head size (blocks of more than eight waves: up to 64)."""
-    return ("square", "square2", "square_halves") + (("square4", "square2_halves") if dim <= 64 else ())
+    return ("square", "square2", "square3", "square_halves") + (("square4", "square2_halves") if dim <= 64 else ())
 
 
 @pytest.mark.parametrize("heads, kv_heads, dim, page_size", [
@@ -497,7 +497,7 @@ def test_attention_mfma_tiles(ops, heads, kv_heads, dim, page_size):
     if dim > 64:
         with pytest.raises(ops.KernelError):
             run_mfma(ops, qt, kt, vt, tables, rows, page_size, "square4")
-    for mode in square_modes(dim):                                                       # 64 / 128 / 256 items on the 32 x 32 instruction
+    for mode in square_modes(dim):                                                       # 64 / 128 / 192 / 256 items on the 32 x 32 instruction
         for given in (False, True):
             got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, mode, positions_given=given)
             np.testing.assert_allclose(got, want, **MFMA_TOL, err_msg=f"{mode} positions given: {given}")

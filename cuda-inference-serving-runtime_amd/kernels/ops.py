@@ -102,7 +102,15 @@ def prepare(head_dims=(), dtype=None):
     lib()
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_current_device = getattr(torch._C, "_cuda_getDevice", None)
+
+
 def _stream():
+    """The handle of the current stream of the current device.  Every launch asks for it: torch's short way where it has
+    one (a prompt step run kernel by kernel asks 240 times; `torch.cuda.current_stream()` takes 9 us a call, 2 ms a step)."""
+    if _raw_stream is not None and _current_device is not None:
+        return _raw_stream(_current_device())
     return torch.cuda.current_stream().cuda_stream
 
 

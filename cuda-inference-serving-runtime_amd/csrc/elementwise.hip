@@ -625,6 +625,27 @@ extern "C" int cisr_f32_to_bf16(const float* x, void* y, long long n, hipStream_
     return CISR_LAUNCH_CHECK();
 }
 
+// ------------------------------------------------------------- bias
+// x[r][c] += bias[c] (added in float, rounded once to x's type): the projections of an architecture with biases run
+// their product as it is and add the bias here, before whatever reads the rows next.
+template <typename TX, typename TB>
+__global__ void bias_add_kernel(TX* __restrict__ x, const TB* __restrict__ bias, size_t n, int cols) {
+    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) store_f32(x + i, load_f32(x + i) + load_f32(bias + i % cols));
+}
+
+extern "C" int cisr_bias_add(void* x, const void* bias, long long rows, int cols, int x_dtype, int bias_dtype, hipStream_t stream) {
+    if (rows <= 0 || cols <= 0) return 0;
+    const size_t n = (size_t)rows * cols;
+    if ((n + 255) / 256 > 0x7fffffffull) return (int)hipErrorInvalidValue;
+    const unsigned blocks = (unsigned)((n + 255) / 256);
+    if (x_dtype == DT_F32 && bias_dtype == DT_F32) bias_add_kernel<float, float><<<blocks, 256, 0, stream>>>((float*)x, (const float*)bias, n, cols);
+    else if (x_dtype == DT_F32) bias_add_kernel<float, bf16_t><<<blocks, 256, 0, stream>>>((float*)x, (const bf16_t*)bias, n, cols);
+    else if (bias_dtype == DT_F32) bias_add_kernel<bf16_t, float><<<blocks, 256, 0, stream>>>((bf16_t*)x, (const float*)bias, n, cols);
+    else bias_add_kernel<bf16_t, bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)x, (const bf16_t*)bias, n, cols);
+    return CISR_LAUNCH_CHECK();
+}
+
 // A kernel that does nothing: what a launch costs in a chain of kernels when nothing is computed, the floor
 // under every kernel of a decode step (measured by the benchmark's "floor" workload).
 __global__ void idle_kernel() {}

@@ -48,6 +48,7 @@ def _declare(h):
         "cisr_page_copy": [p, p, p, i, i, ll, ll, p],
         "cisr_f32_to_bf16": [p, p, ll, p],
         "cisr_idle": [i, p],
+        "cisr_bias_add": [p, p, ll, i, i, i, p],
         "cisr_stream_read": [p, ll, p, i, p],
         "cisr_grid_meet": [p, p, i, i, i, C.c_uint, p],
         "cisr_attn_rowwise": [p, i, p, p, p, p, p, p, p, p, i, i, i, i, i, i, i, f, i, i, p],
@@ -230,6 +231,14 @@ def swiglu(gate_up, out):
     _check(lib().cisr_swiglu(_dev(gate_up, "gate_up"), _dev(out, "out", gate_up.dtype, (rows, inter)), rows, inter,
                              _storage(gate_up, "gate_up"), _stream()), "swiglu")
     return out
+
+
+def bias_add(x, bias):
+    """x[r, c] += bias[c], in place (added in float).  x [T, N] float or bf16, contiguous; bias [N] float or bf16."""
+    rows, cols = x.shape
+    _check(lib().cisr_bias_add(_dev(x, "x"), _dev(bias, "bias", None, (cols,)), rows, cols, _storage(x, "x"), _storage(bias, "bias"),
+                               _stream()), "bias_add")
+    return x
 
 
 def rope_scatter(qkv, positions, slots, cos, sin, kcache, vcache, heads, kv_heads, dim, page_size, interleaved=False):

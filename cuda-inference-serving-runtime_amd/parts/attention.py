@@ -7,8 +7,11 @@ cached keys up to its own position (or the last `window` of them), scale
 residual (reference: runtime/model.py:110-115).  The three projections run as
 one product against the concatenated weight [q; k; v] (a layout choice only).
 
-A mixer built with `reads_site_of` set has no k/v projections: it attends to
-the cache another layer wrote.
+A mixer built with `own_kv` False has no k/v projections: it attends to
+the cache another layer wrote.  With `bias` the q/k/v projections add
+`<name>.{q,k,v}_proj.bias` before the position encoding, with `out_bias` the output
+projection adds `<name>.o_proj.bias`: the products run as they are and a small kernel
+adds the bias (the fused projection kernels have no bias and are not used then).
 """
 import math
 
@@ -20,7 +23,8 @@ from .base import Mixer, TensorSpec, matrix_operand, register_part
 
 
 class PagedAttention(Mixer):
-    def __init__(self, name, hidden, heads, kv_heads, head_dim, position, window=None, scale=None, own_kv=True):
+    def __init__(self, name, hidden, heads, kv_heads, head_dim, position, window=None, scale=None, own_kv=True,
+                 bias=False, out_bias=False):
         if heads % kv_heads:
             raise ValueError(f"{heads} query heads are not a multiple of {kv_heads} key/value heads")
         if head_dim % 2 or head_dim > 256:
@@ -28,7 +32,8 @@ class PagedAttention(Mixer):
         self.name, self.hidden, self.heads, self.kv_heads, self.head_dim = name, hidden, heads, kv_heads, head_dim
         self.position, self.window, self.own_kv = position, window, own_kv
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)
-        self.w_in = self.w_out = None
+        self.bias, self.out_bias = bool(bias), bool(out_bias)
+        self.w_in = self.w_out = self.b_in = self.b_out = None
 
     def cache_need(self):
         return KVNeed(self.kv_heads, self.head_dim, self.window) if self.own_kv else None
@@ -42,13 +47,24 @@ class PagedAttention(Mixer):
         if self.own_kv:
             specs += [TensorSpec(f"{n}.k_proj.weight", (self.kv_heads * D, H)),
                       TensorSpec(f"{n}.v_proj.weight", (self.kv_heads * D, H))]
-        return specs + [TensorSpec(f"{n}.o_proj.weight", (H, self.heads * D))]
+        specs.append(TensorSpec(f"{n}.o_proj.weight", (H, self.heads * D)))
+        if self.bias:
+            specs.append(TensorSpec(f"{n}.q_proj.bias", (self.heads * D,)))
+            if self.own_kv:
+                specs += [TensorSpec(f"{n}.k_proj.bias", (self.kv_heads * D,)), TensorSpec(f"{n}.v_proj.bias", (self.kv_heads * D,))]
+        if self.out_bias:
+            specs.append(TensorSpec(f"{n}.o_proj.bias", (H,)))
+        return specs
 
     def bind(self, tensors, dtype):
         names = ["q_proj"] + (["k_proj", "v_proj"] if self.own_kv else [])
         parts = [matrix_operand(tensors[f"{self.name}.{p}.weight"], dtype) for p in names]
         self.w_in = torch.cat(parts, dim=0).contiguous() if len(parts) > 1 else parts[0]
         self.w_out = matrix_operand(tensors[f"{self.name}.o_proj.weight"], dtype)
+        if self.bias:   # (a bias keeps the type it is stored in; it is added in float)
+            self.b_in = torch.cat([tensors[f"{self.name}.{p}.bias"] for p in names], dim=0).contiguous()
+        if self.out_bias:
+            self.b_out = tensors[f"{self.name}.o_proj.bias"].contiguous()
 
     def prepare(self, device, dtype):
         self.position.prepare(device, dtype)
@@ -60,7 +76,7 @@ class PagedAttention(Mixer):
     def _fused_projection_ok(self, a, normed):
         cos, _ = self.position.tables()
         # (the fused kernels turn split-half pairs only; another pairing takes the general rotary kernel)
-        return not self._interleaved and ops.qkv_rope_fused_ok(a, self.w_in, self.head_dim, cos, normed)
+        return not self._interleaved and not self.bias and ops.qkv_rope_fused_ok(a, self.w_in, self.head_dim, cos, normed)
 
     def fuses_norm(self, norm, residual, ctx):
         return getattr(norm, "fusable_as", None) == "rms" and self._fused_projection_ok(residual, True)
@@ -85,6 +101,8 @@ class PagedAttention(Mixer):
             q_stride = (nh + (2 * nkv if self.own_kv else 0)) * D
             q = ctx.buffer("attn.qkv", (T, q_stride), ctx.dtype)
             ops.gemm(h, self.w_in, q)
+            if self.b_in is not None:
+                ops.bias_add(q, self.b_in)
             ops.rope_scatter(q, ctx.positions, slots, cos, sin, kcache_w, vcache_w, nh, nkv, D, view.page_size,
                              interleaved=self._interleaved)
         out = ctx.buffer("attn.out", (T, nh * D), ctx.dtype)
@@ -92,8 +110,12 @@ class PagedAttention(Mixer):
         unmerged = ctx.attend(q, q_stride, kcache, vcache, view, out, nh, nkv, D, self.window, self.scale,
                               defer_merge=lambda splits: ops.gemm_merged_ok(T, self.w_out, nh, D, splits))
         if unmerged is not None:
-            return ops.gemm_merged(unmerged, nh, D, self.w_out, residual, residual)
-        return ctx.add_product(out, self.w_out, residual)
+            residual = ops.gemm_merged(unmerged, nh, D, self.w_out, residual, residual)
+        else:
+            residual = ctx.add_product(out, self.w_out, residual)
+        if self.b_out is not None:
+            ops.bias_add(residual, self.b_out)   # (sums commute: slices of the product that a later norm adds may still be out)
+        return residual
 
 
 register_part("mixer", "attention", PagedAttention)

@@ -1227,3 +1227,19 @@ def test_grid_meet_counts_every_group_every_round(ops, blocks, exchange):
         assert int(words[16 * (1 + g)]) == rounds * 32
     with pytest.raises(KernelError, match="multiple of 32"):
         ops.grid_meet(48, 1)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("x_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("bias_dtype", [torch.float32, torch.bfloat16])
+def test_bias_add(ops, x_dtype, bias_dtype):
+    for rows, cols in ((1, 7), (37, 576), (300, 1000)):
+        g = torch.Generator(device="cpu").manual_seed(rows + cols)
+        x = torch.randn(rows, cols, generator=g).to(x_dtype).to(DEV)
+        bias = torch.randn(cols, generator=g).to(bias_dtype).to(DEV)
+        want = (x.double() + bias.double()[None, :]).to(x_dtype)          # one rounding, to x's type
+        got = ops.bias_add(x.clone(), bias)
+        assert torch.equal(got, want), (rows, cols)
+    from runtime.kernels.ops import KernelError
+    with pytest.raises(KernelError, match="shape"):
+        ops.bias_add(torch.zeros(3, 5, device=DEV), torch.zeros(4, device=DEV))

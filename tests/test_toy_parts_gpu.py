@@ -801,6 +801,110 @@ def test_attention_with_a_partial_rotary_embedding_and_a_scale_of_its_own(tmp_pa
         cleanup()
 
 
+def build_biased_toy():
+    """The framework's attention and feed-forward with biases on their projections (no architecture of the family has
+    them): the first layer on all seven projections, the second on q/k/v only."""
+    from runtime import make_part, register_architecture
+    from runtime.config import unregister_architecture
+    from runtime.parts import TokenEmbedding, LMHead
+    from runtime.models import Model
+
+    @dataclass(frozen=True)
+    class BiasedConfig:
+        vocab_size: int
+        hidden_size: int
+        rope_theta: float
+        max_position_embeddings: int
+        rms_norm_eps: float
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(*(raw[k] for k in ("vocab_size", "hidden_size", "rope_theta", "max_position_embeddings", "rms_norm_eps")))
+
+    def build(c):
+        def rms(n): return make_part("norm", "rmsnorm", name=n, dim=c.hidden_size, eps=c.rms_norm_eps)
+        position = make_part("position", "rotary", head_dim=16, theta=c.rope_theta, max_positions=c.max_position_embeddings)
+        def layer(n, out_bias, mlp_bias):
+            return make_part("block", "prenorm", mixer_norm=rms(n + ".n1"),
+                             mixer=make_part("mixer", "attention", name=n + ".attn", hidden=c.hidden_size, heads=4, kv_heads=2,
+                                             head_dim=16, position=position, bias=True, out_bias=out_bias),
+                             ffn_norm=rms(n + ".n2"),
+                             ffn=make_part("ffn", "gated_mlp", name=n + ".mlp", hidden=c.hidden_size, intermediate=56, bias=mlp_bias))
+        return Model(c, TokenEmbedding("embed", c.vocab_size, c.hidden_size), [layer("l0", True, True), layer("l1", False, False)],
+                     rms("final"), LMHead("head", c.vocab_size, c.hidden_size))
+
+    register_architecture("toy-biased-lm", BiasedConfig, build)
+    return lambda: unregister_architecture("toy-biased-lm")
+
+
+def plain_biased_toy(raw, w, tokens, without=()):
+    """`without`: names of biases taken as zero."""
+    import plain_llama as P
+    eps, theta = raw["rms_norm_eps"], raw["rope_theta"]
+    T, nh, nkv, D = len(tokens), 4, 2, 16
+    pos = np.arange(T)
+
+    def lin(x, name):
+        y = P.linear(x, w[name + ".weight"])
+        if name + ".bias" in w and name + ".bias" not in without:
+            y = y + np.asarray(w[name + ".bias"], np.float64)
+        return y
+
+    x = np.asarray(w["embed.weight"], np.float64)[tokens]
+    for name in ("l0", "l1"):
+        h = P.rmsnorm(x, w[name + ".n1.weight"], eps)
+        q = P.rope(lin(h, name + ".attn.q_proj").reshape(T, nh, D), pos, theta)
+        k = P.rope(lin(h, name + ".attn.k_proj").reshape(T, nkv, D), pos, theta)
+        v = lin(h, name + ".attn.v_proj").reshape(T, nkv, D)
+        k, v = np.repeat(k, nh // nkv, axis=1), np.repeat(v, nh // nkv, axis=1)
+        x = x + lin(P.causal_attention(q, k, v).reshape(T, nh * D), name + ".attn.o_proj")
+        h = P.rmsnorm(x, w[name + ".n2.weight"], eps)
+        x = x + lin(P.swiglu(lin(h, name + ".mlp.gate_proj"), lin(h, name + ".mlp.up_proj")), name + ".mlp.down_proj")
+    return P.linear(P.rmsnorm(x, w["final.weight"], eps), w["head.weight"])
+
+
+@pytest.mark.parametrize("dtype, execution", [("float32", "eager"), ("bfloat16", "eager"), ("bfloat16", "graph")])
+def test_projections_with_biases(tmp_path, dtype, execution):
+    """A bias is a parameter of the framework's own attention and feed-forward: the products run as they are, a small
+    kernel adds the bias before the rotary embedding, the activation or the residual sum; portions beside decoded tokens."""
+    import plain_llama as P
+    from conftest import assert_close
+    from runtime.engine import load_model, ModelRunner, StepEntry
+    from runtime.engine.loading import build_from_config_dict
+    from runtime.weights import write_model_folder
+    cleanup = build_biased_toy()
+    try:
+        raw = {"model_type": "toy-biased-lm", "vocab_size": 67, "hidden_size": 40, "rope_theta": 900.0,
+               "max_position_embeddings": 96, "rms_norm_eps": 1e-6}
+        tmp_path.mkdir(exist_ok=True)
+        _, _, blueprint = build_from_config_dict(raw)
+        names = [spec.name for spec in blueprint.tensor_specs()]
+        assert sum(n.endswith(".bias") for n in names) == 7 + 3
+        write_model_folder(tmp_path, raw, blueprint.tensor_specs(), seed=23, dtype=torch.float32 if dtype == "float32" else torch.bfloat16, std=0.15)
+        cfg, w = P.read_folder(tmp_path)
+        model = load_model(tmp_path, dtype=dtype)
+        runner = ModelRunner(model, n_pages=16, page_size=8, max_requests=2, execution=execution)
+        tokens = {"x": np.random.default_rng(18).integers(0, 67, 41).tolist(), "y": np.random.default_rng(19).integers(0, 67, 25).tolist()}
+        want = {k: plain_biased_toy(raw, w, v) for k, v in tokens.items()}
+        runner.create("x"); runner.create("y")
+        got, fed = {"x": [], "y": []}, {"x": 0, "y": 0}
+        for step in [[("x", 17), ("y", 2)], [("x", 1), ("y", 12)], [("x", 1), ("y", 1)], [("x", 22), ("y", 10)]]:
+            entries = [StepEntry(k, tokens[k][fed[k]:fed[k] + n], list(range(n))) for k, n in step]
+            out = runner.step(entries).float().cpu().numpy()
+            row = 0
+            for k, n in step:
+                got[k].append(out[row:row + n]); row += n; fed[k] += n
+        for k in tokens:
+            assert_close(np.concatenate(got[k]), want[k], dtype, f"request {k}")
+        # every kind of bias matters: with one of them taken as zero the logits are others
+        for name in ("l0.attn.q_proj.bias", "l0.attn.k_proj.bias", "l1.attn.v_proj.bias", "l0.attn.o_proj.bias",
+                     "l0.mlp.gate_proj.bias", "l0.mlp.up_proj.bias", "l0.mlp.down_proj.bias"):
+            assert np.abs(plain_biased_toy(raw, w, tokens["x"], without=(name,)) - want["x"]).max() > 1e-3, name
+        runner.cache.check()
+    finally:
+        cleanup()
+
+
 @pytest.mark.parametrize("execution, overlap", [("eager", False), ("graph", True)])
 def test_scheduler_generates_with_a_model_of_two_page_groups(tmp_path, execution, overlap):
     """The entry point over the model with windowed and full layers: requests admitted by what each group of pages

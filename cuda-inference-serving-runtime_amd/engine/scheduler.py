@@ -334,7 +334,12 @@ class Engine:
             # a model whose mixers keep no keys has nothing to size)
             widths = [need.kv_heads * need.head_dim for need in model.cache_needs().values() if need is not None]
             if widths:
-                addressable = min(addressable, (2 ** 31 - 1) // (max(widths) * page_size))
+                by_offsets = (2 ** 31 - 1) // (max(widths) * page_size)
+                if by_offsets < addressable:
+                    import sys
+                    print(f"[runtime] the pool is limited to {by_offsets} pages a layer by the kernels' 32-bit offsets "
+                          f"(the requests could address {addressable})", file=sys.stderr)
+                    addressable = by_offsets
             pages = pages_that_fit(model.cache_needs(), page_size, 2 if dtype == "bfloat16" else 4, free, most=addressable)
         runner = ModelRunner(model, n_pages=pages, page_size=page_size, max_requests=max_requests, device=device,
                              execution=execution)

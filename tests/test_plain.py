@@ -149,7 +149,7 @@ def test_reference_toy_weights_vector(folders):
     # the reference's own model test (tests/test_model.py:8-26) feeds tokens
     # [1,9,5,7,3] through its default toy configuration; its weights come from
     # numpy's default_rng(42) (runtime/model.py:38-55).  Rebuilt here, the plain
-    # forward must agree with the composition written in that test.
+    # forward must agree with the computation of that test written out a second time.
     c = dict(vocab_size=128, hidden_size=64, intermediate_size=128, num_hidden_layers=2, num_attention_heads=4,
              num_key_value_heads=2, rms_norm_eps=1e-5, rope_theta=10000.0, tie_word_embeddings=False)
     rng = np.random.default_rng(42)
@@ -171,19 +171,38 @@ def test_reference_toy_weights_vector(folders):
         matrix(p + "mlp.down_proj.weight", 64, 128)
     tokens = [1, 9, 5, 7, 3]
     got = P.forward(c, w, tokens)
-    # the same computation in the order of the reference's test, in float64
+    # the same computation written a second time from the formulas, sharing nothing with the plain module: the norm
+    # spelled out, the rotary embedding as a complex rotation, attention as one masked softmax matrix per head
+    def norm(z, weight):
+        return z / np.sqrt((z * z).mean(-1, keepdims=True) + 1e-5) * weight.astype(np.float64)
+
+    def turn(z):   # z [T, heads, dim]: coordinates (i, i + dim/2) are the real and imaginary part of one number
+        half = dim // 2
+        angle = np.arange(5)[:, None] * 10000.0 ** (-2.0 * np.arange(half) / dim)[None, :]
+        zc = (z[..., :half] + 1j * z[..., half:]) * np.exp(1j * angle)[:, None, :]
+        return np.concatenate([zc.real, zc.imag], axis=-1)
+
+    def attend(q, k, v):   # q [T, 4, dim], k and v [T, 2, dim]: query head h reads key head h // 2
+        out = np.zeros_like(q)
+        for h in range(4):
+            scores = q[:, h] @ k[:, h // 2].T / np.sqrt(dim)
+            scores[np.triu_indices(5, 1)] = -np.inf
+            weights = np.exp(scores - scores.max(-1, keepdims=True))
+            out[:, h] = (weights / weights.sum(-1, keepdims=True)) @ v[:, h // 2]
+        return out
+
     x = w["model.embed_tokens.weight"][tokens].astype(np.float64)
     for layer in range(2):
         p = f"model.layers.{layer}."
         lin = lambda z, n: z @ w[p + n + ".weight"].astype(np.float64).T
-        h = P.rmsnorm(x, w[p + "input_layernorm.weight"], 1e-5)
-        q = P.rope(lin(h, "self_attn.q_proj").reshape(-1, 4, dim), range(5), 10000.0)
-        k = P.rope(lin(h, "self_attn.k_proj").reshape(-1, 2, dim), range(5), 10000.0)
+        h = norm(x, w[p + "input_layernorm.weight"])
+        q = turn(lin(h, "self_attn.q_proj").reshape(-1, 4, dim))
+        k = turn(lin(h, "self_attn.k_proj").reshape(-1, 2, dim))
         v = lin(h, "self_attn.v_proj").reshape(-1, 2, dim)
-        x = x + lin(P.causal_attention(q, k, v).reshape(-1, 64), "self_attn.o_proj")
-        h = P.rmsnorm(x, w[p + "post_attention_layernorm.weight"], 1e-5)
+        x = x + lin(attend(q, k, v).reshape(-1, 64), "self_attn.o_proj")
+        h = norm(x, w[p + "post_attention_layernorm.weight"])
         g = lin(h, "mlp.gate_proj")
         x = x + lin(g / (1 + np.exp(-g)) * lin(h, "mlp.up_proj"), "mlp.down_proj")
-    expected = P.rmsnorm(x, w["model.norm.weight"], 1e-5) @ w["lm_head.weight"].astype(np.float64).T
+    expected = norm(x, w["model.norm.weight"]) @ w["lm_head.weight"].astype(np.float64).T
     np.testing.assert_allclose(got, expected, atol=1e-12)
     assert got.shape == (5, 128) and np.abs(got).max() > 0.5  # real-sized logits, not a degenerate case

@@ -538,7 +538,9 @@ class ModelRunner:
                     # about one block a compute unit: the time is the longest tile's chain of steps, which two halves a
                     # block cut in two (2,048 rows at the 135M sizes 31.6 -> 28.4 us, 4,096 rows 64 -> 55; with more
                     # blocks than that the halves only crowd the compute units: 46 -> 68 us at the 1.7B sizes)
-                    few = -(-blocks // n) <= 320
+                    # (up to 511 blocks of 64 items when the chain is long: 3,072 rows at the 135M sizes, 441 blocks,
+                    # 35.6 us against 43.4; 16 heads over 4 at 1,536 rows 22.1 against 25.4; at 1,000 rows the halves lose)
+                    few = -(-blocks // n) <= 320 or (n == 1 and span >= 1536)
                     fits = n == 1 or (n == 2 and head_dim <= 64)
                     halves = 2 if (few and fits if self.square_halves is None else self.square_halves == 2 and fits) else 1
                     return "square", n, halves

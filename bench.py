@@ -192,11 +192,12 @@ def main():
     ap.add_argument("--overlap", type=int, default=1, choices=[0, 1],
                     help="1: picked tokens stay on the device and a step is launched before the tokens of the one "
                          "before are read, as the scheduler's overlapped ticks do; 0: every step waits for its tokens")
-    ap.add_argument("--workload", default="decode", choices=["decode", "serving", "floor", "attention"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "serving", "floor", "attention", "attention_forms"],
                     help="decode: fixed batch after whole prompts (the default, timed per step); serving: --requests "
                          "requests with prompts of 128..--prompt tokens and --new-tokens each through the scheduler; "
                          "floor: a captured chain of kernels that do nothing (what a launch costs); attention: the attention kernel "
-                         "alone over whole prompts of --attention-rows rows at the family's head shapes")
+                         "alone over whole prompts of --attention-rows rows at the family's head shapes; attention_forms: every form "
+                         "of that kernel at a grid of head shapes and --attention-rows, beside the form the engine picks")
     ap.add_argument("--attention-rows", default="2048,7936", help="attention workload: prompt lengths (comma separated)")
     ap.add_argument("--requests", type=int, default=64)
     ap.add_argument("--new-tokens", type=int, default=256)
@@ -213,6 +214,8 @@ def main():
 
     if args.workload == "floor":
         return launch_floor(args)
+    if args.workload == "attention_forms":
+        return attention_forms(args)
     if args.workload == "attention":
         return prompt_attention(args)
     raw = preset(args.model)
@@ -358,65 +361,114 @@ def launch_floor(args):
     return 0
 
 
+def _time_attention(heads, kv_heads, D, T, P, form, calls=20):
+    """Microseconds of one call of the prompt attention kernel in `form` (kind, n, halves): causal attention of T rows
+    over their own T keys in a paged cache; `calls` calls in one captured graph, the median of five replays."""
+    import statistics
+    import numpy as np
+    import torch
+    from runtime.engine.context import fill_tasks
+    from runtime.kernels import ops
+    dev = torch.device("cuda:0")
+    kind, n, halves = form
+    pages = -(-T // P)
+    q = torch.randn(T, heads * D, device=dev).bfloat16()
+    K = torch.randn(pages, kv_heads, P, D, device=dev).bfloat16()
+    V = torch.randn(pages, kv_heads, D, P, device=dev).bfloat16()
+    tables = torch.arange(pages, dtype=torch.int32, device=dev).reshape(1, pages)
+    seg = torch.zeros(T, dtype=torch.int32, device=dev)
+    pos = torch.arange(T, dtype=torch.int32, device=dev)
+    o = torch.empty(T, heads * D, device=dev, dtype=torch.bfloat16)
+    rows_per_tile = (16 if kind == "tiles" else 64) * n // min(heads // kv_heads, 16)
+    host = np.full((-(-T // rows_per_tile), 4), -1, dtype=np.int32)
+    fill_tasks(host, [T], rows_per_tile, [0])
+    tasks = torch.from_numpy(host).to(dev)
+
+    def run():
+        ops.attention_mfma(q, heads * D, K, V, tables, seg, pos, o, heads, kv_heads, D, P, None, D ** -0.5, tasks,
+                           block_tiles={"tiles": False, "block": True, "square": 32}[kind], item_tiles=n, key_groups=halves)
+    stream, graph = torch.cuda.Stream(), torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        run(); stream.synchronize()
+        with torch.cuda.graph(graph, stream=stream):
+            for _ in range(calls):
+                run()
+    times = []
+    for _ in range(6):
+        torch.cuda.synchronize(); t0 = time.perf_counter()
+        graph.replay()
+        torch.cuda.synchronize(); times.append((time.perf_counter() - t0) / calls)
+    return statistics.median(times[1:]) * 1e6
+
+
+def _form_chooser():
+    from runtime.engine import ModelRunner
+    chooser = ModelRunner.__new__(ModelRunner)          # only its tiling rule is used
+    chooser.square_tiles = chooser.block_tiles = chooser.square_halves = None
+    chooser.item_tiles = 2
+    return chooser
+
+
+def _form_name(form):
+    kind, n, halves = form
+    return f"{kind} x{n}" + (", two halves" if halves == 2 else "")
+
+
 def prompt_attention(args):
     """The attention kernel alone on whole prompts: causal attention of T rows over their own T keys in a paged cache, at
     the head shapes of the three family members, in the form the engine chooses for that size.  Twenty calls in one
     captured graph, the median of five replays; flops are those of the causal half, 4 T (T + 1) / 2 x head size x heads."""
-    import statistics
-    import numpy as np
-    import torch
     from runtime.config import preset
-    from runtime.engine import ModelRunner
-    from runtime.engine.context import fill_tasks
-    from runtime.kernels import ops
-    dev = torch.device("cuda:0")
     P = args.page_size
     out = {}
-    chooser = ModelRunner.__new__(ModelRunner)          # only its tiling rule is used
-    chooser.square_tiles = chooser.block_tiles = chooser.square_halves = None
-    chooser.item_tiles = 2
+    chooser = _form_chooser()
     for name in ("smollm2-135m", "smollm2-1.7b", "llama-3-8b"):
         raw = preset(name)
         heads, kv_heads = raw["num_attention_heads"], raw["num_key_value_heads"]
         D = raw.get("head_dim") or raw["hidden_size"] // heads
         for T in [int(t) for t in args.attention_rows.split(",") if t]:
-            pages = -(-T // P)
-            q = torch.randn(T, heads * D, device=dev).bfloat16()
-            K = torch.randn(pages, kv_heads, P, D, device=dev).bfloat16()
-            V = torch.randn(pages, kv_heads, D, P, device=dev).bfloat16()
-            tables = torch.arange(pages, dtype=torch.int32, device=dev).reshape(1, pages)
-            seg = torch.zeros(T, dtype=torch.int32, device=dev)
-            pos = torch.arange(T, dtype=torch.int32, device=dev)
-            o = torch.empty(T, heads * D, device=dev, dtype=torch.bfloat16)
-            kind, n, halves = chooser.prompt_attention_form(T, 1, T, heads, kv_heads, D, P)
-            rows_per_tile = (16 if kind == "tiles" else 64) * n // min(heads // kv_heads, 16)
-            host = np.full((-(-T // rows_per_tile), 4), -1, dtype=np.int32)
-            fill_tasks(host, [T], rows_per_tile, [0])
-            tasks = torch.from_numpy(host).to(dev)
-
-            def run():
-                ops.attention_mfma(q, heads * D, K, V, tables, seg, pos, o, heads, kv_heads, D, P, None, D ** -0.5, tasks,
-                                   block_tiles={"tiles": False, "block": True, "square": 32}[kind], item_tiles=n, key_groups=halves)
-            calls = 20
-            stream, graph = torch.cuda.Stream(), torch.cuda.CUDAGraph()
-            with torch.cuda.stream(stream):
-                run(); stream.synchronize()
-                with torch.cuda.graph(graph, stream=stream):
-                    for _ in range(calls):
-                        run()
-            times = []
-            for _ in range(6):
-                torch.cuda.synchronize(); t0 = time.perf_counter()
-                graph.replay()
-                torch.cuda.synchronize(); times.append((time.perf_counter() - t0) / calls)
-            us = statistics.median(times[1:]) * 1e6
+            form = chooser.prompt_attention_form(T, 1, T, heads, kv_heads, D, P)
+            us = _time_attention(heads, kv_heads, D, T, P, form)
             flops = 4 * T * (T + 1) / 2 * D * heads
-            out[f"{name}_{T}"] = {"heads": heads, "kv_heads": kv_heads, "head_dim": D, "rows": T, "form": f"{kind} x{n}" + (", two halves" if halves == 2 else ""),
+            out[f"{name}_{T}"] = {"heads": heads, "kv_heads": kv_heads, "head_dim": D, "rows": T, "form": _form_name(form),
                                   "us": round(us, 1), "pflops": round(flops / us / 1e9, 3),
                                   "frac_of_bf16_peak": round(flops / us / 1e6 / PEAK_TFLOPS["bf16"], 4)}
     print(json.dumps({"metric": "prompt attention alone, PFLOP/s of the causal half (bf16, paged cache, page size %d)" % P,
                       "unit": "PFLOP/s", "n_gpus": 1, "value": out["smollm2-1.7b_%s" % args.attention_rows.split(",")[0]]["pflops"],
                       "higher_is_better": True, "shapes": out}))
+    return 0
+
+
+def attention_forms(args):
+    """Every form of the prompt attention kernel at a grid of head shapes (heads/key heads x head size, the family's and
+    others) and prompt lengths, beside the form the engine's rule picks: one line a point on stderr, then one JSON line
+    with the worst and the mean loss of the rule against the best form of each point."""
+    P = args.page_size
+    chooser = _form_chooser()
+    forms = [("tiles", 1, 1), ("tiles", 2, 1), ("block", 1, 1), ("block", 2, 1), ("square", 1, 1), ("square", 2, 1),
+             ("square", 3, 1), ("square", 4, 1), ("square", 1, 2), ("square", 2, 2)]
+
+    def takes(form, D, T):
+        kind, n, halves = form
+        if kind == "tiles":
+            return T <= 4096 and (n == 1 or D <= 64)      # (far from the best beyond that, and slow to measure)
+        return kind == "block" or D <= 64 or not (n == 4 or (n == 2 and halves == 2))
+    shapes = [(9, 3, 64), (32, 32, 64), (32, 8, 128), (16, 4, 64), (12, 12, 128), (8, 8, 64), (24, 8, 96), (64, 8, 128)]
+    points, losses = {}, []
+    for heads, kv_heads, D in shapes:
+        for T in [int(t) for t in args.attention_rows.split(",") if t]:
+            us = {form: _time_attention(heads, kv_heads, D, T, P, form, calls=8) for form in forms if takes(form, D, T)}
+            pick = tuple(chooser.prompt_attention_form(T, 1, T, heads, kv_heads, D, P))
+            best = min(us, key=us.get)
+            loss = us[pick] / us[best] - 1
+            losses.append(loss)
+            points[f"{heads}/{kv_heads}x{D}_{T}"] = {"pick": _form_name(pick), "pick_us": round(us[pick], 1), "best": _form_name(best),
+                                                    "best_us": round(us[best], 1), "loss": round(loss, 3)}
+            print(f"{heads:2d}/{kv_heads:2d} x {D:3d}  {T:5d} rows  pick {_form_name(pick):22s} {us[pick]:7.1f} us   best {_form_name(best):22s} "
+                  f"{us[best]:7.1f} us   " + "  ".join(f"{_form_name(f)}: {v:.0f}" for f, v in us.items()), file=sys.stderr, flush=True)
+    print(json.dumps({"metric": "loss of the rule that picks the prompt attention form against the best form of each point",
+                      "unit": "fraction", "n_gpus": 1, "value": round(max(losses), 3), "higher_is_better": False,
+                      "mean": round(sum(losses) / len(losses), 4), "points": points}))
     return 0
 
 

@@ -529,7 +529,9 @@ class ModelRunner:
                     # a compute unit holds two such blocks with small heads, one with large, and no wave slot stays empty).
                     # 32 heads of 64 at 16k rows: 1.42 ms against 1.46 with 256 items and 1.54 with 128; 9 heads over 3 at
                     # 32k: 1.49 against 1.58 and 1.61; 32 heads of 128 over 8 at 8k: 0.60 against 0.63 with 128 items
-                    n = 3 if blocks >= 2048 else 2
+                    # (heads of more than 64 coordinates, one computing wave a SIMD: already from 1,100 blocks on; 32 heads
+                    # of 128 over 8 at 3,072 rows, 1,536 blocks: 106 us against 123; 24 heads of 96 over 8: 72 against 84)
+                    n = 3 if blocks >= (2048 if head_dim <= 64 else 1100) else 2
                 elif span >= 1024 and blocks >= 128:
                     # (fewer blocks than compute units and a thousand keys: 64-item blocks, in two halves; 1,024 rows of
                     # 12 heads of 128 take 25 us against 35 as LDS block tiles, of 16 heads of 64 over 4: 17 against 18)
@@ -540,7 +542,10 @@ class ModelRunner:
                     # blocks than that the halves only crowd the compute units: 46 -> 68 us at the 1.7B sizes)
                     # (up to 511 blocks of 64 items when the chain is long: 3,072 rows at the 135M sizes, 441 blocks,
                     # 35.6 us against 43.4; 16 heads over 4 at 1,536 rows 22.1 against 25.4; at 1,000 rows the halves lose)
-                    few = -(-blocks // n) <= 320 or (n == 1 and span >= 1536)
+                    # and up to 512 blocks of 128 items from 3,072 keys on: 8 heads of 64 at 6,144 rows 71 against 89,
+                    # 9 over 3 at 6,144 rows 76 against 92, 16 over 4 at 3,072 rows 42 against 50
+                    few = (-(-blocks // n) <= 320 or (n == 1 and span >= 1536)
+                           or (n == 2 and -(-blocks // n) <= 512 and span >= 3072))
                     fits = n == 1 or (n == 2 and head_dim <= 64)
                     halves = 2 if (few and fits if self.square_halves is None else self.square_halves == 2 and fits) else 1
                     return "square", n, halves

@@ -192,12 +192,14 @@ def main():
     ap.add_argument("--overlap", type=int, default=1, choices=[0, 1],
                     help="1: picked tokens stay on the device and a step is launched before the tokens of the one "
                          "before are read, as the scheduler's overlapped ticks do; 0: every step waits for its tokens")
-    ap.add_argument("--workload", default="decode", choices=["decode", "serving", "floor", "attention", "attention_forms"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "serving", "floor", "attention", "attention_forms", "decode_attention_shapes"],
                     help="decode: fixed batch after whole prompts (the default, timed per step); serving: --requests "
                          "requests with prompts of 128..--prompt tokens and --new-tokens each through the scheduler; "
                          "floor: a captured chain of kernels that do nothing (what a launch costs); attention: the attention kernel "
                          "alone over whole prompts of --attention-rows rows at the family's head shapes; attention_forms: every form "
-                         "of that kernel at a grid of head shapes and --attention-rows, beside the form the engine picks")
+                         "of that kernel at a grid of head shapes and --attention-rows, beside the form the engine picks; "
+                         "decode_attention_shapes: every launch shape of the decode attention kernel at a grid of requests and "
+                         "contexts, beside the one the engine picks")
     ap.add_argument("--attention-rows", default="2048,7936", help="attention workload: prompt lengths (comma separated)")
     ap.add_argument("--requests", type=int, default=64)
     ap.add_argument("--new-tokens", type=int, default=256)
@@ -216,6 +218,8 @@ def main():
         return launch_floor(args)
     if args.workload == "attention_forms":
         return attention_forms(args)
+    if args.workload == "decode_attention_shapes":
+        return decode_attention_shapes(args)
     if args.workload == "attention":
         return prompt_attention(args)
     raw = preset(args.model)
@@ -467,6 +471,80 @@ def attention_forms(args):
             print(f"{heads:2d}/{kv_heads:2d} x {D:3d}  {T:5d} rows  pick {_form_name(pick):22s} {us[pick]:7.1f} us   best {_form_name(best):22s} "
                   f"{us[best]:7.1f} us   " + "  ".join(f"{_form_name(f)}: {v:.0f}" for f, v in us.items()), file=sys.stderr, flush=True)
     print(json.dumps({"metric": "loss of the rule that picks the prompt attention form against the best form of each point",
+                      "unit": "fraction", "n_gpus": 1, "value": round(max(losses), 3), "higher_is_better": False,
+                      "mean": round(sum(losses) / len(losses), 4), "points": points}))
+    return 0
+
+
+def decode_attention_shapes(args):
+    """The decode attention kernel alone (one row a request, bf16, paged cache with scattered pages) at the family's head
+    shapes over a grid of requests and contexts: every launch shape (wavefronts a block x blocks along the keys, with the
+    merge kernel when the keys are split) beside the one `ModelRunner._rows_launch` picks.  Keys and values of up to
+    eight layers take turns, so that nothing is read from a cache twice in a row.  One line a point on stderr, then one
+    JSON line with the worst and the mean loss of the rule."""
+    import math
+    import torch
+    from runtime.config import preset
+    from runtime.engine import ModelRunner
+    from runtime.kernels import ops
+    dev, P = torch.device("cuda:0"), args.page_size
+    points, losses = {}, []
+    for name in ("smollm2-135m", "smollm2-1.7b", "llama-3-8b"):
+        raw = preset(name)
+        heads, kv = raw["num_attention_heads"], raw["num_key_value_heads"]
+        D = raw.get("head_dim") or raw["hidden_size"] // heads
+        group = heads // kv
+        per_chunk = min(group, 16)
+        for C in (512, 2048, 8192, 32768):
+            for B in (1, 4, 8, 16, 32, 64, 128):
+                if B * C * kv * D * 4 > 6 << 30:
+                    continue
+                pages_per = -(-C // P)
+                n_pages = B * pages_per
+                copies = int(max(1, min(8, (600 << 20) // (n_pages * kv * P * D * 4))))
+                ks = [torch.randn(n_pages, kv, P, D, device=dev).bfloat16() for _ in range(copies)]
+                vs = [torch.randn(n_pages, kv, D, P, device=dev).bfloat16() for _ in range(copies)]
+                tables = torch.randperm(n_pages, device=dev).int().view(B, pages_per)
+                q = torch.randn(B, heads * D, device=dev).bfloat16()
+                seg = torch.arange(B, device=dev, dtype=torch.int32)
+                pos = torch.full((B,), C - 1, device=dev, dtype=torch.int32)
+                out = torch.empty(B, heads * D, device=dev).bfloat16()
+                blocks = B * kv * -(-group // per_chunk)
+                pick = tuple(ModelRunner._rows_launch(blocks, C, per_chunk, D))
+                shapes = {(w, n) for w in (4, 8) for n in (1, 2, 4, 8, 16, 32) if (n == 1 or n * 32 <= C) and blocks * n <= 16384} | {pick}
+                us = {}
+                for waves, splits in sorted(shapes):
+                    ws = (torch.empty(B * heads * splits * D, device=dev), torch.empty(B * heads * splits * 2, device=dev))
+
+                    def run(i):
+                        ops.attention_mfma(q, heads * D, ks[i], vs[i], tables, seg, pos, out, heads, kv, D, P, None, 1 / math.sqrt(D),
+                                           None, splits, ws, waves)
+                    calls = max(copies, 4)
+                    for i in range(copies):
+                        run(i)
+                    torch.cuda.synchronize()
+                    graph = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(graph):
+                        for i in range(calls):
+                            run(i % copies)
+                    graph.replay()
+                    torch.cuda.synchronize()
+                    times = []
+                    for _ in range(3):
+                        t0 = time.perf_counter()
+                        graph.replay()
+                        torch.cuda.synchronize()
+                        times.append((time.perf_counter() - t0) / calls * 1e6)
+                    us[(waves, splits)] = sorted(times)[1]
+                best = min(us, key=us.get)
+                loss = us[pick] / us[best] - 1
+                losses.append(loss)
+                label = lambda shape: f"{shape[0]} waves x {shape[1]}"
+                points[f"{name}_{B}x{C}"] = {"pick": label(pick), "pick_us": round(us[pick], 1), "best": label(best),
+                                             "best_us": round(us[best], 1), "loss": round(loss, 3)}
+                print(f"{name:13s} {B:3d} rows x {C:5d} keys  pick {label(pick):13s} {us[pick]:7.1f} us   best {label(best):13s} {us[best]:7.1f} us   "
+                      + "  ".join(f"{w}x{n}: {v:.1f}" for (w, n), v in sorted(us.items())), file=sys.stderr, flush=True)
+    print(json.dumps({"metric": "loss of the rule that picks the decode attention launch shape against the best shape of each point",
                       "unit": "fraction", "n_gpus": 1, "value": round(max(losses), 3), "higher_is_better": False,
                       "mean": round(sum(losses) / len(losses), 4), "points": points}))
     return 0

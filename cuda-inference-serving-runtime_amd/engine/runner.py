@@ -571,18 +571,22 @@ class ModelRunner:
         when that gives every compute unit at most one block."""
         steps = -(-span // 32)
         few = blocks < 128
-        # eight waves a block with few rows and small heads, except at long contexts (more than 4k), where three
-        # blocks of four waves a compute unit keep more loads in flight than the one block of eight that fits
-        # (4-6 % faster at 8 rows and 8k to 30k, 2 % slower at 2k to 4k; a single row keeps its eight)
-        waves = 8 if few and head_dim <= 64 and (steps <= 128 or blocks < 8) else 4
+        # eight waves a block with few rows and small heads (at 8k and 32k too, now that at most eight splits of few
+        # rows are merged by the product that follows: 4 rows at 8k 15.3 us against 16.3 with four waves, 8 rows at
+        # 32k 44.4 against 46.5)
+        waves = 8 if few and head_dim <= 64 else 4
+        if steps <= 2 * waves:
+            # two steps a wave: nothing to split (a second block along the keys and the merge cost 2 us of 8 to 10)
+            return waves, 1
         if few:
             # Few rows: split the keys until the blocks fill the GPU once: an eight-wave block fills a compute
             # unit (256 blocks; more start a second round: 16 splits of 8 rows at 2k to 4k are 10 % slower than
             # 8), four-wave blocks fit three a unit, of which two are worth having (512 blocks: a thousand are
             # 12 % slower at 30k, where each then lives for three steps a wave only).  A wave keeps at least one
             # 32-key step (with two, 8 rows at 2k have 4 splits and are 5 % slower).
+            # At most 32 splits: a single row of 8 key heads at 8k takes 23 us with 32 and 30 with 64.
             room = 256 if waves == 8 else 512
-            splits = int(max(1, min(steps // waves, room // blocks, 64)))
+            splits = int(max(1, min(steps // waves, room // blocks, 32)))
         elif head_dim <= 64 and 140 <= blocks <= 256:
             # enough rows to give most compute units one block of eight waves, and no more than one each: the
             # keys are not split and no merge follows (9-11 % faster than four waves and three or four splits at
@@ -591,8 +595,9 @@ class ModelRunner:
         else:
             # Many rows split until every compute unit has the blocks of four waves that its registers hold (three
             # with small heads, two otherwise: 3-5 % faster at 384 blocks of the 135M sizes than one block a unit;
-            # from 512 blocks on a split costs 3-8 %); a wave keeps at least two 32-key steps.
+            # from 512 blocks on a split costs 3-8 %); a wave keeps at least four 32-key steps (with two, 128 rows at
+            # 512 keys take 19.4 us against 16.5 unsplit).
             target = 768 if head_dim <= 64 else 512
             per = target // blocks if head_dim <= 64 and blocks > 256 else -(-target // blocks)
-            splits = int(max(1, min(steps // (waves * 2), per, 64)))
+            splits = int(max(1, min(steps // (waves * 4), per, 64)))
         return waves, splits

@@ -13,7 +13,7 @@ pytestmark = pytest.mark.gpu
 FAMILY = {
     "smollm2-135m": dict(num_hidden_layers=2, hidden_size=576, num_attention_heads=9, num_key_value_heads=3, head_dim=64,
                          intermediate_size=1536, vocab_size=3001, rope_theta=100000.0, rms_norm_eps=1e-5,
-                         tie_word_embeddings=True, max_position_embeddings=512),
+                         tie_word_embeddings=True, max_position_embeddings=768),
     "smollm2-1.7b": dict(num_hidden_layers=1, hidden_size=2048, num_attention_heads=32, num_key_value_heads=32, head_dim=64,
                          intermediate_size=8192, vocab_size=2003, rope_theta=130000.0, rms_norm_eps=1e-5,
                          tie_word_embeddings=True, max_position_embeddings=512),
@@ -87,16 +87,16 @@ def test_a_cut_across_the_library_threshold_changes_rounding_only(family_folders
 
 @pytest.mark.parametrize("execution", ["eager", "graph"])
 def test_decoding_at_a_context_whose_keys_are_split_over_blocks(family_folders, execution):
-    """From a context of about 500 keys on, a decode step of few rows splits every row's keys over blocks; at the
+    """From a context of about 550 keys on (more than two 32-key steps a wave), a decode step of few rows splits every row's keys over blocks; at the
     135M sizes the output projection then merges the blocks' partial results itself (no merge kernel).  Three requests
     of very different lengths decode together (the short one's later splits see no key at all), then one alone."""
     from runtime.engine import load_model, ModelRunner, StepEntry
     name = "smollm2-135m"
     folder = family_folders[name]
     V = FAMILY[name]["vocab_size"]
-    seqs = {"long": random_tokens(11, 506, V), "mid": random_tokens(12, 310, V), "short": random_tokens(13, 20, V)}
+    seqs = {"long": random_tokens(11, 700, V), "mid": random_tokens(12, 310, V), "short": random_tokens(13, 20, V)}
     model = load_model(folder, dtype="bfloat16")
-    runner = ModelRunner(model, n_pages=64, page_size=16, max_requests=4, execution=execution)
+    runner = ModelRunner(model, n_pages=80, page_size=16, max_requests=4, execution=execution)
     fed, got = {}, {k: [] for k in seqs}
     for k, toks in seqs.items():
         runner.create(k)

@@ -361,11 +361,19 @@ def attention_rowwise(q, q_row_stride, kcache, vcache, tables, seg_of_row, posit
 # residual sum included; the products of the 135M sizes, 0.7 to 3.5 MB, are as fast or faster here).  0 rows: never.
 LIBRARY_MIN_ROWS = int(os.environ.get("CISR_LIBRARY_MIN_ROWS", "65"))
 LIBRARY_MIN_BYTES = int(float(os.environ.get("CISR_LIBRARY_MIN_MB", "8")) * (1 << 20))
+LIBRARY_GATED_MIN_ROWS, LIBRARY_GATED_MIN_BYTES = 33, 64 << 20
 _library_scratch = {}   # (device, elements) -> bf16 buffers, never freed: captured programs keep their addresses
 
 
-def library_ok(m, w):
-    return (LIBRARY_MIN_ROWS > 0 and m >= LIBRARY_MIN_ROWS and w.dtype == torch.bfloat16 and w.is_contiguous()
+def library_ok(m, w, gated=False):
+    """`gated`: the product of gate and up, whose activation is a kernel of its own after the library's product.  With
+    weights of 64 MB and more it goes there from 33 rows on: 64 rows against the 8B sizes' 235 MB take 60.7 us there and
+    69.7 in the wide kernel here (58.4 against 63.0 at 33 rows; 23.0 against 26.5 at the 1.7B sizes), the activation
+    included; the other products of 33 to 64 rows are as fast here."""
+    least = LIBRARY_MIN_ROWS
+    if gated and w.numel() * 2 >= LIBRARY_GATED_MIN_BYTES:
+        least = min(least, LIBRARY_GATED_MIN_ROWS)
+    return (LIBRARY_MIN_ROWS > 0 and m >= least and w.dtype == torch.bfloat16 and w.is_contiguous()
             and w.numel() * 2 >= LIBRARY_MIN_BYTES)
 
 
@@ -589,7 +597,7 @@ def gemm_swiglu(a, w_gate_up, out, scratch=None, norm=None):
         return out
     if out.dtype != a.dtype or a.dtype != w_gate_up.dtype:
         raise KernelError("gemm_swiglu: dtypes differ")
-    if a.dtype == torch.bfloat16 and library_ok(m, w_gate_up) and a.is_contiguous():
+    if a.dtype == torch.bfloat16 and library_ok(m, w_gate_up, gated=True) and a.is_contiguous():
         product = _scratch_bf16(a.device, m, two_i)
         torch.mm(a, w_gate_up.t(), out=product)
         return swiglu(product, out)

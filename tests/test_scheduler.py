@@ -312,3 +312,44 @@ def test_overlapped_ticks_cancel_while_a_step_is_in_flight():
     assert len(e.requests["b"].generated) == 6 and not e.reserved
     e.runner.cache.check()
     assert e.runner.cache.free_pages() == [20]
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_workloads_finish_and_give_everything_back(seed):
+    """Random pools, limits, policies and windows; requests arrive while others run, some are cancelled, some are too
+    long for the context or the pool: every accepted request ends finished or cancelled, the engine comes to rest,
+    no page and no promise is left behind."""
+    import random
+    rng = random.Random(seed)
+    pages, page_size = rng.randint(6, 30), rng.choice([2, 4, 8])
+    max_requests, overlap = rng.randint(2, 8), rng.random() < 0.5
+    window = rng.choice([None, None, 8, 12])
+    runner = (OverlapRunner if overlap else FakeRunner)(pages=pages, page_size=page_size, max_requests=max_requests,
+                                                        max_context=rng.choice([32, 64, 96]))
+    if window is not None:   # a second group of layers that look back over a window: pages of their own
+        runner.cache = CacheManager({0: KVNeed(1, 8), 1: KVNeed(1, 8, window)}, pages, page_size, max_requests)
+    engine = make_engine(runner, max_active=rng.randint(1, 8), token_budget=rng.randint(2, 40), prefill_chunk=rng.randint(1, 16),
+                         policy=rng.choice(["serial", "chunked", "decode_first"]), overlap=overlap)
+    arriving = [(f"r{i}", [rng.randrange(50) for _ in range(rng.randint(1, 40))], rng.randint(1, 12), rng.choice([None, None, 7, (3, 9)]))
+                for i in range(rng.randint(1, 12))]
+    accepted, ticks = [], 0
+    while arriving or engine.waiting or engine.active or engine.inflight:
+        ticks += 1
+        assert ticks < 5000, "the engine does not come to rest"
+        if arriving and rng.random() < 0.4:
+            key, prompt, new, eos = arriving.pop()
+            try:
+                engine.submit(Request(key, prompt, new, eos))
+                accepted.append(key)
+            except ValueError:
+                pass          # refused at the door: longer than the context, or than the pool could ever hold
+        if accepted and rng.random() < 0.05:
+            engine.cancel(rng.choice(accepted))
+        engine.tick()
+    runner.cache.check()
+    assert not runner.cache.lengths and not engine.ledger.promised
+    for key in accepted:
+        request = engine.requests[key]
+        assert str(request.status) in ("finished", "cancelled")
+        if str(request.status) == "finished":
+            assert 1 <= len(request.generated) <= request.max_new_tokens

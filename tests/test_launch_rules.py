@@ -1,0 +1,51 @@
+"""The rules that pick a kernel's form are plain functions of sizes: their decisions at the points where
+measurements settled them (profiles/prompt_attention_forms_and_the_rule_that_picks.txt and
+profiles/decode_attention_launch_shapes_and_the_rule_that_picks.txt), so that a change of a rule shows."""
+import pytest
+
+from runtime.engine.runner import ModelRunner
+
+
+def chooser():
+    runner = ModelRunner.__new__(ModelRunner)          # only the rule is used
+    runner.square_tiles = runner.block_tiles = runner.square_halves = None
+    runner.item_tiles = 2
+    return runner
+
+
+@pytest.mark.parametrize("heads, kv_heads, dim, rows, form", [
+    (9, 3, 64, 2048, ("square", 1, 2)),       # about one block a compute unit: two halves a block
+    (9, 3, 64, 3072, ("square", 1, 2)),       # 441 blocks, a long chain: still halves
+    (9, 3, 64, 6144, ("square", 2, 2)),       # 440 blocks of 128 items from 3,072 keys on
+    (9, 3, 64, 8192, ("square", 2, 1)),
+    (32, 32, 64, 2048, ("square", 2, 1)),
+    (32, 32, 64, 4096, ("square", 3, 1)),     # 2,048 blocks of 64 items: 192 items a block
+    (32, 8, 128, 2048, ("square", 2, 1)),
+    (32, 8, 128, 3072, ("square", 3, 1)),     # large heads: 192 items from 1,100 blocks on
+    (16, 4, 64, 3072, ("square", 2, 2)),
+    (16, 4, 64, 6144, ("square", 2, 1)),      # 768 blocks of 128 items: the halves would crowd the compute units
+])
+def test_prompt_attention_form_at_measured_points(heads, kv_heads, dim, rows, form):
+    assert tuple(chooser().prompt_attention_form(rows, 1, rows, heads, kv_heads, dim, 16)) == form
+
+
+def test_prompt_attention_form_needs_long_portions_and_pages_of_eight_keys():
+    rule = chooser()
+    assert rule.prompt_attention_form(40, 8, 3000, 9, 3, 64, 16)[0] == "tiles"        # many short portions
+    assert rule.prompt_attention_form(2048, 1, 2048, 9, 3, 64, 4)[0] != "square"      # the copying waves take 8 keys of a page
+    assert rule.prompt_attention_form(2048, 1, 2048, 2, 2, 256, 16)[0] == "tiles"     # heads of more than 128 coordinates
+
+
+@pytest.mark.parametrize("blocks, keys, group, dim, launch", [
+    (3, 2048, 3, 64, (8, 8)),          # one request of the 135M sizes
+    (24, 2048, 3, 64, (8, 8)),         # eight
+    (192, 2048, 3, 64, (8, 1)),        # 64: one block of eight waves a compute unit, no split
+    (24, 8192, 3, 64, (8, 10)),        # eight waves at long contexts too
+    (24, 512, 3, 64, (8, 1)),          # two steps a wave: nothing to split
+    (384, 512, 3, 64, (4, 1)),
+    (8, 8192, 4, 128, (4, 32)),        # at most 32 splits
+    (64, 2048, 4, 128, (4, 8)),
+    (512, 2048, 4, 128, (4, 1)),
+])
+def test_decode_attention_launch_at_measured_points(blocks, keys, group, dim, launch):
+    assert tuple(ModelRunner._rows_launch(blocks, keys, group, dim)) == launch

@@ -32,9 +32,10 @@ class CacheManager:
     fast_decode = True   # steps of one token a request take a short path (tests switch it off to compare)
 
     def __init__(self, site_needs, n_pages, page_size, max_requests, state_needs=None,
-                 allocate_kv=None, allocate_state=None, copy_pages=None, zero_state=None, copy_state=None):
-        """site_needs: {site id: KVNeed}; state_needs: {site id: StateNeed}.
-        n_pages: pages per group (an int, or {KVNeed: int})."""
+                 allocate_pages=None, allocate_state=None, copy_pages=None, zero_state=None, copy_state=None):
+        """site_needs: {site id: need (KVNeed or another class with its methods)}; state_needs: {site id: StateNeed}.
+        n_pages: pages per group (an int, or {need: int}).  `allocate_pages(shape)` makes a group's device storage,
+        of the shape its need states."""
         self.page_size = page_size
         self.groups = []
         self.group_of_site = {}
@@ -44,8 +45,8 @@ class CacheManager:
         for gid, (need, sites) in enumerate(by_need.items()):
             pages = n_pages[need] if isinstance(n_pages, dict) else n_pages
             group = CacheGroup(need, sites, pages, page_size)
-            if allocate_kv is not None:
-                group.storage = allocate_kv(len(sites), pages, need.kv_heads, page_size, need.head_dim)
+            if allocate_pages is not None:
+                group.storage = allocate_pages(need.storage_shape(len(sites), pages, page_size))
             self.groups.append(group)
             for index, site in enumerate(sites):
                 self.group_of_site[site] = (gid, index)
@@ -152,7 +153,8 @@ class CacheManager:
         return result
 
     def commit(self, done):
-        """The step that fills the slots of `done` (append_many with commit=False) is on its way: the tokens count."""
+        """The step that fills the slots of `done` (append_many with commit=False) is on its way: the tokens count.
+        (On its way, not finished: later steps read the slots only because they are queued on the same stream.)"""
         for d in done:
             if self.lengths[d.request] != d.start:
                 raise RuntimeError(f"request {d.request!r} moved between its append and its commit")
@@ -160,9 +162,13 @@ class CacheManager:
         return done
 
     def abandon(self, done):
-        """The step of `done` (append_many with commit=False) was never launched: pages taken for its tokens go
-        back, the requests stand where they stood.  (A page copied for a write stays copied, pages that a window
-        had passed stay given back: neither changes what a later step reads.)"""
+        """The step of `done` (append_many with commit=False) was never launched, or failed on its way: pages taken
+        for its tokens go back, the requests' lengths and tables stand where they stood.  (A page copied for a write
+        stays copied, pages that a window had passed stay given back: neither changes what a later step reads.)
+        Kernels of the failed step may still be queued and write into pages that go back here, and the page copy of
+        a copy-on-write may still be on its way: whoever takes those pages next must be ordered behind them.  The
+        owner launches everything on ONE stream (ModelRunner refuses a step on another), which is that order.
+        Per-request state is not restored: see ModelRunner.step."""
         for d in done:
             keep = -(-self.lengths[d.request] // self.page_size)
             for group in self.groups:
@@ -211,13 +217,14 @@ class CacheManager:
         return self.groups[gid].tables[request]
 
     # -- views for mixers ---------------------------------------------------
-    def kv_of_site(self, site):
-        """(group id, keys [pages, kv_heads, P, D], values [pages, kv_heads, D, P]) of a site.
-        Values are stored transposed inside a page (same bytes per page as keys)."""
+    def pages_of_site(self, site):
+        """(group id, *views): the group a site's pages belong to and the site's own views of the group's storage,
+        as its need lays them out (KVNeed: keys [pages, kv_heads, P, D], values [pages, kv_heads, D, P])."""
         gid, index = self.group_of_site[site]
-        storage = self.groups[gid].storage
-        pages, kv_heads, psize, dim = storage.shape[2:]
-        return gid, storage[index, 0], storage[index, 1].view(pages, kv_heads, dim, psize)
+        group = self.groups[gid]
+        return (gid, *group.need.views(group.storage, index))
+
+    kv_of_site = pages_of_site
 
     # -- bookkeeping --------------------------------------------------------
     def check(self):
@@ -253,7 +260,7 @@ class CacheManager:
     def report(self):
         out = []
         for gid, g in enumerate(self.groups):
-            token_bytes = 2 * g.need.kv_heads * g.need.head_dim * len(g.sites)
+            token_bytes = g.need.elements_per_token() * len(g.sites)
             out.append({"group": gid, "sites": len(g.sites), "window": g.need.window, "pages": g.pool.n_pages,
                         "resident_pages": g.pool.used, "peak_pages": g.pool.peak, "free_pages": len(g.pool.free),
                         "shared_pages": sum(1 for r in g.pool.refs if r > 1), "requests": len(g.tables),
@@ -263,9 +270,9 @@ class CacheManager:
 
 def pages_that_fit(site_needs, page_size, itemsize, free_bytes, fraction=0.8, most=None):
     """How many pages a pool may have so that the caches of all sites take `fraction` of `free_bytes`:
-    a page index costs, in every site that keeps keys and values, 2 x kv_heads x page_size x head_dim
-    elements.  `most` caps the answer (more pages than the requests can ever address are of no use)."""
-    per_page = sum(2 * need.kv_heads * page_size * need.head_dim * itemsize for need in site_needs.values() if need is not None)
+    a page index costs, in every site that keeps pages, page_size times the elements its need takes a token.
+    `most` caps the answer (more pages than the requests can ever address are of no use)."""
+    per_page = sum(need.elements_per_token() * page_size * itemsize for need in site_needs.values() if need is not None)
     if per_page == 0:
         return 1
     pages = int(free_bytes * fraction) // per_page

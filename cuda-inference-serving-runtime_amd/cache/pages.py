@@ -26,10 +26,34 @@ class OutOfPages(MemoryError):
 
 @dataclass(frozen=True)
 class KVNeed:
-    """Keys and values per token: [kv_heads, head_dim] each; window None = all keys."""
+    """Keys and values per token: [kv_heads, head_dim] each; window None = all keys.
+
+    A need is what the cache manager knows of a mixer's pages.  The manager groups sites by equal needs and asks the
+    need, never itself, how the pages of a group are stored: any frozen dataclass with `window` and the four
+    methods below can stand here (keys and values of different widths, a compressed form, one tensor a token).
+    This one's layout is what the attention kernels of this package read: a page's keys as [kv_heads, page_size,
+    head_dim], its values transposed as [kv_heads, head_dim, page_size], keys of all pages first."""
     kv_heads: int
     head_dim: int
     window: Optional[int] = None
+
+    def elements_per_token(self):
+        """Cached elements a token takes in one site."""
+        return 2 * self.kv_heads * self.head_dim
+
+    def storage_shape(self, sites, pages, page_size):
+        """Shape of the one tensor that holds the pages of `sites` sites of a group."""
+        return (sites, 2, pages, self.kv_heads, page_size, self.head_dim)
+
+    def slabs(self, sites):
+        """Into how many contiguous runs of `pages` pages the storage divides (a page copy touches each)."""
+        return sites * 2
+
+    def views(self, storage, index):
+        """What a mixer reads and writes of site `index` of the group: (keys [pages, kv_heads, P, D],
+        values [pages, kv_heads, D, P])."""
+        pages, kv_heads, psize, dim = storage.shape[2:]
+        return storage[index, 0], storage[index, 1].view(pages, kv_heads, dim, psize)
 
 
 @dataclass(frozen=True)
@@ -85,7 +109,7 @@ class CacheGroup:
         self.tables = {}
         self.versions = {}   # request -> stamp of the last change of its table (stamps are never reused)
         self._stamp = 0
-        self.storage = None  # device tensor [sites, 2, pages, kv_heads, page_size, head_dim], set by the owner
+        self.storage = None  # device tensor of the shape the need states (storage_shape), set by the owner
 
     # -- planning -------------------------------------------------------
     def _dead_pages(self, request, length):

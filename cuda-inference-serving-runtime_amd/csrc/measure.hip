@@ -1,0 +1,106 @@
+// Kernels that only measure the machine: what a launch costs, what a meeting of all blocks inside one kernel costs,
+// what the memory gives a kernel that only reads.  A unit of its own (libcisr_measure): the engine never loads it;
+// `python -m runtime.measure` and the benchmark's read-bandwidth figure do.
+#include "common.h"
+
+// A kernel that does nothing: what a launch costs in a chain of kernels when nothing is computed, the floor
+// under every kernel of a decode step (measured by `python -m runtime.measure floor`).
+__global__ void idle_kernel() {}
+
+extern "C" int cisr_idle(int blocks, hipStream_t stream) {
+    if (blocks <= 0) return 0;
+    idle_kernel<<<(unsigned)blocks, 256, 0, stream>>>();
+    return CISR_LAUNCH_CHECK();
+}
+
+// A meeting of every block of a grid inside one kernel, as a decode step fused into fewer kernels would need between
+// its parts: what it costs beside the launch of a kernel (`python -m runtime.measure floor` reports both).  Blocks meet
+// in groups of 32 at a counter of their own, the last of a group goes on to the top counter, and everyone polls that
+// one; with `exchange` every block writes its share of that many floats before the meeting and reads all of them
+// after it, as activations would pass.  The wait is bounded: a block that waits too long sets the flag and leaves,
+// so every wave ends whatever happens.  `words`: 1024 zeroed 32-bit words (counters 64 bytes apart, the flag last).
+constexpr int MEET_GROUP = 32, MEET_WORDS = 1024, MEET_MAX_BLOCKS = 512;
+__global__ void __launch_bounds__(256) grid_meet_kernel(unsigned* __restrict__ words, float* __restrict__ passed, int exchange,
+                                                        int rounds, unsigned spin_limit) {
+    const unsigned groups = gridDim.x / MEET_GROUP;
+    unsigned* top = words;
+    unsigned* mine = words + 16 * (1 + blockIdx.x % groups);
+    unsigned* flag = words + MEET_WORDS - 1;
+    const int share = exchange / (int)gridDim.x;
+    float acc = 0.f;
+    __shared__ int gave_up;
+    if (threadIdx.x == 0) gave_up = 0;
+    for (int r = 0; r < rounds; ++r) {
+        float* side = passed + (size_t)(r & 1) * exchange;
+        for (int i = threadIdx.x; i < share; i += blockDim.x) side[blockIdx.x * share + i] = acc + (float)(r + i);
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            __atomic_thread_fence(__ATOMIC_RELEASE);
+            const unsigned before = __hip_atomic_fetch_add(mine, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (before + 1 == (unsigned)(r + 1) * MEET_GROUP) __hip_atomic_fetch_add(top, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            unsigned spins = 0;
+            while (__hip_atomic_load(top, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < (unsigned)(r + 1) * groups) {
+                if (++spins > spin_limit) { *flag = 1u; gave_up = 1; break; }
+                __builtin_amdgcn_s_sleep(1);
+            }
+            __atomic_thread_fence(__ATOMIC_ACQUIRE);
+        }
+        __syncthreads();
+        if (gave_up) break;
+        float part[4] = {0.f, 0.f, 0.f, 0.f};                  // (four sums, so that the loads of a lane do not wait for each other)
+        const int all = share * (int)gridDim.x;
+        int i = threadIdx.x;
+        for (; i + 3 * 256 < all; i += 4 * 256) {
+#pragma unroll
+            for (int u = 0; u < 4; ++u) part[u] += __builtin_nontemporal_load(side + i + u * 256);
+        }
+        for (; i < all; i += 256) part[0] += __builtin_nontemporal_load(side + i);
+        acc += (part[0] + part[1] + part[2] + part[3]) * 1e-9f;
+    }
+    if (acc == 123.456f) words[MEET_WORDS - 2] = 1u;
+}
+
+// `blocks`: a multiple of 32, at most 512 (all of them must be resident together: 256 threads and a few bytes of LDS each);
+// `passed`: 2 x exchange floats (may be null when exchange is 0).
+extern "C" int cisr_grid_meet(void* words, void* passed, int exchange, int blocks, int rounds, unsigned spin_limit, hipStream_t stream) {
+    if (rounds <= 0) return 0;
+    if (!words || blocks <= 0 || blocks % MEET_GROUP || blocks > MEET_MAX_BLOCKS || exchange < 0 || (exchange && !passed) ||
+        (long long)rounds * blocks >= (1ll << 31))
+        return (int)hipErrorInvalidValue;
+    // every block must be resident at once, or the first to arrive wait for blocks that cannot start
+    int device = 0, per_unit = 0, units = 0;
+    if (hipGetDevice(&device) != hipSuccess || hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess ||
+        hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_unit, grid_meet_kernel, 256, 0) != hipSuccess || (long long)per_unit * units < blocks)
+        return (int)hipErrorInvalidValue;
+    grid_meet_kernel<<<(unsigned)blocks, 256, 0, stream>>>((unsigned*)words, (float*)passed, exchange, rounds, spin_limit);
+    return CISR_LAUNCH_CHECK();
+}
+
+// A kernel that only reads: every block walks a contiguous run of 16-byte words, eight loads a lane in flight, and
+// folds them into one word that is written only if it has a value no data gives.  What this GPU's memory gives a
+// kernel that streams weights and does nothing else (the benchmark reports it beside the published peak).
+typedef unsigned int read_word_t __attribute__((ext_vector_type(4)));
+__global__ void __launch_bounds__(256) stream_read_kernel(const read_word_t* __restrict__ src, long long words, unsigned* __restrict__ sink) {
+    const long long per = words / gridDim.x;                       // (a remainder of fewer words than blocks is left out)
+    const read_word_t* p = src + (long long)blockIdx.x * per;
+    read_word_t acc = {0u, 0u, 0u, 0u};
+    constexpr int U = 8;
+    long long i = threadIdx.x;
+    for (; i + (long long)(U - 1) * 256 < per; i += (long long)U * 256) {
+        read_word_t v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) v[u] = __builtin_nontemporal_load(p + i + (long long)u * 256);
+#pragma unroll
+        for (int u = 0; u < U; ++u) acc ^= v[u];
+    }
+    for (; i < per; i += 256) acc ^= p[i];
+    if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x9e3779b9u && sink) sink[0] = acc.x;
+}
+
+// Reads `bytes` (a multiple of 16, 16-byte aligned) once with `blocks` blocks; `sink`: 4 bytes that are hardly ever written.
+extern "C" int cisr_stream_read(const void* src, long long bytes, void* sink, int blocks, hipStream_t stream) {
+    if (bytes <= 0 || blocks <= 0) return 0;
+    if (bytes % 16 || ((uintptr_t)src) % 16 || !sink) return (int)hipErrorInvalidValue;
+    stream_read_kernel<<<(unsigned)blocks, 256, 0, stream>>>((const read_word_t*)src, bytes / 16, (unsigned*)sink);
+    return CISR_LAUNCH_CHECK();
+}

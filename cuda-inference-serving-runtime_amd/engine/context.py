@@ -22,30 +22,30 @@ class GroupView:
     width: int
 
 
-def fill_tasks(tasks, counts, rows_per_tile, starts=None, skip_single=False):
-    """Write (segment, first row, rows, p) for tiles of at most `rows_per_tile` consecutive
-    rows of one segment into the int32 array tasks[n, 4]; returns how many were written.
-    With `starts` (the position of each segment's first row) p is the position of the tile's
-    first row plus one (a segment's rows have consecutive positions, so a kernel that reads p need
-    not wait for the positions array; p = 0 says "not given"), and the tiles are ordered by the
-    number of keys they attend to, most first: blocks are handed out in this order, and the
-    long ones must not be the last to start.  `skip_single`: segments of one row get no tile
-    (they are attended to by a launch of their own)."""
-    n = row = 0
-    for seg, count in enumerate(counts):
-        tiles = 0 if skip_single and count == 1 else -(-count // rows_per_tile)
-        firsts = np.arange(tiles, dtype=np.int64) * rows_per_tile
-        tasks[n:n + tiles, 0] = seg
-        tasks[n:n + tiles, 1] = row + firsts
-        tasks[n:n + tiles, 2] = np.minimum(rows_per_tile, count - firsts)
-        tasks[n:n + tiles, 3] = 0 if starts is None else int(starts[seg]) + firsts + 1
-        n += tiles
-        row += count
-    if starts is not None and n > 1:
-        first_row = np.concatenate(([0], np.cumsum(counts)))[tasks[:n, 0]]
-        keys = np.asarray(starts, dtype=np.int64)[tasks[:n, 0]] + (tasks[:n, 1] - first_row) + tasks[:n, 2]
-        tasks[:n] = tasks[:n][np.argsort(-keys, kind="stable")]
-    return n
+class StepArray:
+    """The interface of a per-step list that a part wants every step's metadata to carry, beside what every step
+    has (tokens, positions, segments, slots, block tables).  The step function lays such arrays out behind its own,
+    fills them on the host with the rest of the metadata and uploads everything in one copy; it never looks at what
+    they mean.  A part asks for one with `StepContext.step_array` (or names it beforehand in `step_arrays()`); from
+    then on every step carries it.  Implementations are small frozen dataclasses (they are dictionary keys):
+
+      words(rows, segments) -> int         int32 words for a step padded to that many rows and segments
+      launch_value(batch) -> int | None    what of the batch the part's launches depend on beside the array's
+                                           contents (the step function rounds it up and makes it part of the key
+                                           of a captured program); None: nothing
+      fill(out, batch, value) -> None      write the array (a NumPy int32 view of `words` entries) for `batch`;
+                                           `value` is the launch value, rounded up under a captured program
+    """
+
+
+@dataclass
+class Batch:
+    """A step's batch as the host sees it, for StepArray implementations."""
+    counts: list          # new tokens of each segment
+    starts: list          # position of each segment's first new token
+    first_row: object     # int32 [segments]: row of each segment's first token
+    decode_only: bool     # every segment brings exactly one token
+    launch_values: dict   # StepArray -> its launch value for this step
 
 
 class StepContext:
@@ -54,6 +54,7 @@ class StepContext:
         self.cache = runner.cache
         self.dtype = runner.model.dtype
         self.device = runner.device
+        self.scratch = runner.scratch   # the ScratchPool that products of this step use (ops.* take it as `scratch`)
         self.n_rows = self.n_segments = 0
         self.tokens = self.positions = self.seg_of_row = self.logit_rows = None
         self.seg_start = self.seg_first_pos = self.state_slots = None
@@ -63,9 +64,8 @@ class StepContext:
         self.max_context = 0      # host: largest position + 1 among the rows
         self.decode_only = False  # host: every segment brings exactly one token
         self.span_hint = 0        # host: context length that sizes attention launches (a bucket under capture)
-        self.tasks = {}           # rows per tile -> int32 [n, 4] task list on the device
-        self.single_rows = None   # int32 [S]: the rows of the one-token segments of a mixed step, then -1
-        self.n_single = 0         # host: how many entries of single_rows a launch of their own covers (0: none)
+        self.arrays = {}          # StepArray -> (int32 device view, launch value): what parts asked the metadata to carry
+        self.batch = None         # host: the Batch that the step arrays were filled from
         # A product whose partial sums are still to be added to the residual stream: (rows tensor, partials), set by a
         # part that was told it may (`next_norm`), taken by the norm that reads the rows next (or settled)
         self.unfinished = None
@@ -78,33 +78,30 @@ class StepContext:
         captured program; otherwise valid until the next step)."""
         return self.runner.workspace.get(name, shape, dtype, owner=self.owner)
 
-    def attention_tasks(self, rows_per_tile):
-        """int32 [n, 4] on the device: (segment, first row, rows, 0) for tiles of at most
-        `rows_per_tile` consecutive rows of one segment; entries with segment -1 are no tile.
-        The step's metadata holds the list for every tiling asked for before; a new tiling
-        is built and uploaded here once and travels with the metadata from the next step on."""
-        tasks = self.tasks.get(rows_per_tile)
-        if tasks is None:
+    def step_array(self, array):
+        """(int32 device tensor, launch value) of a StepArray.  The step's metadata holds every array asked for
+        before; a new one is built and uploaded here once and travels with the metadata from the next step on."""
+        got = self.arrays.get(array)
+        if got is None:
             if self.capturing:
-                raise RuntimeError(f"a task list of {rows_per_tile} rows a tile was first asked for under graph capture")
-            counts = [count for _, _, count in self.segments]
-            host = np.full((sum(-(-c // rows_per_tile) for c in counts), 4), -1, dtype=np.int32)
-            fill_tasks(host, counts, rows_per_tile, [start for _, start, _ in self.segments], skip_single=self.n_single > 0)
-            tasks = torch.from_numpy(host).to(self.device, non_blocking=False)
-            self.tasks[rows_per_tile] = tasks
-            if rows_per_tile not in self.runner.task_tilings:
-                self.runner.task_tilings.append(rows_per_tile)
-        return tasks
+                raise RuntimeError(f"the step array {array!r} was first asked for under graph capture")
+            value = array.launch_value(self.batch)
+            self.batch.launch_values[array] = value
+            host = np.zeros(array.words(self.n_rows, self.n_segments), dtype=np.int32)
+            array.fill(host, self.batch, value)
+            got = self.arrays[array] = (torch.from_numpy(host).to(self.device, non_blocking=False), value)
+            self.runner.carry(array)
+        return got
 
     def add_product(self, a, w, residual):
         """residual += a . w^T, in place.  Where the product is cut along its inner size and the norm that reads the
         residual next can add the slices itself (`next_norm`), they are left to it: one kernel fewer."""
         if getattr(self.next_norm, "adds_partials", False):
-            partials = ops.gemm_unfinished(a, w, residual)
+            partials = ops.gemm_unfinished(a, w, residual, scratch=self.scratch)
             if partials is not None:
                 self.leave_unfinished(residual, partials)
                 return residual
-        return ops.gemm(a, w, residual, residual=residual)
+        return ops.gemm(a, w, residual, residual=residual, scratch=self.scratch)
 
     def leave_unfinished(self, rows, partials):
         """`rows` lack the partial sums `partials` (ops.gemm_unfinished); whoever reads them next adds them."""
@@ -126,13 +123,6 @@ class StepContext:
         partials = self.take_unfinished(rows)
         if partials is not None:
             ops.add_partials(rows, partials)
-
-    def attend(self, q, q_row_stride, kcache, vcache, view, out, heads, kv_heads, head_dim, window, scale, defer_merge=None):
-        """out[r] = attention of row r's queries over its request's cache.  With `defer_merge` (see
-        ModelRunner.attention) the result may come back unmerged instead: (partial outputs, statistics, splits) for
-        ops.gemm_merged, `out` untouched; None means `out` holds the result."""
-        return self.runner.attention(self, q, q_row_stride, kcache, vcache, view, out, heads, kv_heads, head_dim, window, scale,
-                                     defer_merge=defer_merge)
 
 
 class Workspace:

@@ -5,6 +5,9 @@ generation uses.
 
 Input, one JSON object per line on standard input:
     {"step": 0, "entries": [{"id": "a", "tokens": [5, 17, 3], "want": [0, 2]}], "end": []}
+A step may also say "fork": [["a", "b"]]: before its entries run, request b starts as a copy of what a holds
+(pages shared, the partly filled last page copied at b's or a's next write; the reference's fork,
+runtime/cache.py:64-76, exercised by tests/test_execution.py:55-64).
 For a step in which something is wanted, ``<out>/<step>.f32`` receives the
 logits at the wanted places as little-endian float32 [wanted, vocab], in the
 order of the entries and of ``want``.  After every step ``done <step>`` is
@@ -39,6 +42,8 @@ def replay(model_dir, dtype, out_dir, max_tokens, lines, page_size=PAGE_SIZE, ec
         if not line:
             continue
         record = json.loads(line)
+        for source, target in record.get("fork", []):
+            runner.fork(source, target)
         entries = []
         for item in record.get("entries", []):
             if item["id"] not in runner.cache:
@@ -64,6 +69,7 @@ def main(argv=None):
     parser.add_argument("--out", required=True, help="folder for <step>.f32 files")
     parser.add_argument("--max-tokens", type=int, required=True,
                         help="most tokens live requests hold at any time (each rounded up to 64)")
+    parser.add_argument("--page-size", type=int, default=PAGE_SIZE, help="tokens a cache page (a power of two that divides 64)")
     parser.add_argument("--execution", choices=["eager", "graph"], default="eager",
                         help="eager: kernels launched one by one; graph: every step as a captured program")
     args = parser.parse_args(argv)
@@ -71,5 +77,7 @@ def main(argv=None):
     def echo(text):
         print(text, flush=True)
 
-    replay(args.model, args.dtype, args.out, args.max_tokens, sys.stdin, echo=echo, execution=args.execution)
+    if args.page_size <= 0 or 64 % args.page_size:
+        parser.error("--page-size must divide 64")
+    replay(args.model, args.dtype, args.out, args.max_tokens, sys.stdin, page_size=args.page_size, echo=echo, execution=args.execution)
     return 0

@@ -12,7 +12,6 @@ context limit, token range, page preflight, then execution
 (runtime/model.py:93-102).
 """
 import gc
-import os
 from dataclasses import dataclass, field
 from typing import List, Sequence
 
@@ -21,7 +20,7 @@ import torch
 
 from ..cache import CacheManager, OutOfPages
 from ..kernels import ops
-from .context import GroupView, StepContext, Workspace, fill_tasks
+from .context import Batch, GroupView, StepContext, Workspace
 
 
 @dataclass
@@ -55,42 +54,39 @@ def _bucket(n):
 
 
 class ModelRunner:
-    def __init__(self, model, n_pages, page_size=16, max_requests=64, device="cuda:0", execution="eager"):
+    def __init__(self, model, n_pages, page_size=16, max_requests=64, device="cuda:0", execution="eager", program_capacity=64):
         if not torch.cuda.is_available():
             raise RuntimeError("no GPU: the engine runs on an MI355X only and has no CPU path")
-        # fail now if the kernels are missing; a first call builds what this model needs, all at once
-        ops.prepare([need.head_dim for need in model.cache_needs().values() if need is not None], model.dtype)
+        # fail now if the kernels are missing; a first call builds what this model's parts say they need, all at once
+        ops.prepare(model.kernel_units())
         if execution not in ("eager", "graph"):
             raise ValueError(f"execution {execution!r} is not eager or graph")
         self.model = model
         self.execution = execution
-        self.programs, self.program_capacity = {}, 16
-        self.block_tiles = None    # long portions through LDS-shared tiles of 64 x this items: None = by the number of blocks
-        # long portions of long contexts through 32 x 32 tiles, 64 x this items a block (1, 2, 3, 4): None = by size, 0 = never
-        self.square_tiles = int(os.environ["CISR_SQUARE_TILES"]) if os.environ.get("CISR_SQUARE_TILES") else None
-        self.square_halves = None  # two halves a block in that form (even and odd steps): None = by the number of blocks, 1, 2
-        self.tile_waves = int(os.environ.get("CISR_TILE_WAVES", "4"))   # wavefronts that share one tile's keys
-        self.item_tiles = int(os.environ.get("CISR_ITEM_TILES", "2"))   # 16-item tiles a wave of long portions (small heads)
-        # In a mixed step a decoded token is a tile whose keys one block walks; from this context on the
-        # one-token segments get a launch of their own instead, which splits their keys over blocks
-        self.split_single_from = 4096
+        # captured programs, least recently used first.  A serving workload in portions makes a few dozen keys (rows,
+        # segments and wanted rows in buckets, contexts in powers of two); an evicted program costs a synchronisation and
+        # a capture when its key comes back, so the capacity is well above that and `report()` counts what happened.
+        self.programs, self.program_capacity = {}, int(program_capacity)
+        self.counters = {"steps": 0, "eager_steps": 0, "captures": 0, "replays": 0, "evictions": 0, "layouts": 0}
         self.device = torch.device(device)
+        self.stream = torch.cuda.current_stream(self.device)   # every step and every release is ordered on this stream
         self.page_size = page_size
         self.max_requests = max_requests
         dtype = model.dtype
 
-        def allocate_kv(sites, pages, kv_heads, psize, head_dim):
-            return torch.zeros((sites, 2, pages, kv_heads, psize, head_dim), dtype=dtype, device=self.device)
+        def allocate_pages(shape):
+            return torch.zeros(shape, dtype=dtype, device=self.device)
 
         def allocate_state(slots, shape, dt):
             return torch.zeros((slots, *shape), dtype=_TORCH_OF[dt], device=self.device)
 
         self.cache = CacheManager(model.cache_needs(), n_pages, page_size, max_requests,
-                                  state_needs=model.state_needs(), allocate_kv=allocate_kv,
+                                  state_needs=model.state_needs(), allocate_pages=allocate_pages,
                                   allocate_state=allocate_state, copy_pages=self._copy_pages,
                                   zero_state=lambda t, s: t[s].zero_(),
                                   copy_state=lambda t, a, b: t[b].copy_(t[a]))
         self.workspace = Workspace(self.device)
+        self.scratch = ops.ScratchPool()   # what products need beyond their operands (never shared with another runner)
         self.max_context = model.max_positions
         self.table_width = -(-self.max_context // page_size)
         self._staging = []
@@ -99,7 +95,8 @@ class ModelRunner:
         # host copies of the block tables by state slot, with the stamp of the table they were made from
         self._table_mirror = [(np.full((max_requests, self.table_width), -1, dtype=np.int32), [None] * max_requests)
                               for _ in self.cache.groups]
-        self.task_tilings = []   # rows-per-tile values that mixers have asked task lists for
+        # the step arrays that parts have asked every step's metadata to carry (context.StepArray), in layout order
+        self.carried = list(dict.fromkeys(model.step_arrays()))
         self.steps = 0
         # the token last picked on the device for each request, by state slot, and its copies on the way to the host
         self.picked = torch.zeros(max_requests, dtype=torch.int32, device=self.device)
@@ -107,6 +104,7 @@ class ModelRunner:
         self._picked_next = 0
         self._has_picked = set()
         self._last_wanted = None  # (requests, state slots on the host, state slots on the device) of the last step's logits
+        self._failed = set()      # requests whose state a failed step may have changed: they can only be released
 
     # -- requests -------------------------------------------------------------
     def create(self, request):
@@ -119,6 +117,7 @@ class ModelRunner:
         # later work that reuses the pages runs on the same stream, after every reader
         self.cache.release(request)
         self._has_picked.discard(request)
+        self._failed.discard(request)
 
     def length(self, request):
         return self.cache.length(request)
@@ -126,7 +125,12 @@ class ModelRunner:
     def _copy_pages(self, group, copies):
         src = torch.tensor([c[0] for c in copies], dtype=torch.int32, device=self.device)
         dst = torch.tensor([c[1] for c in copies], dtype=torch.int32, device=self.device)
-        ops.page_copy(group.storage, src, dst, group.storage.shape[0] * 2, group.pool.n_pages)
+        ops.page_copy(group.storage, src, dst, group.need.slabs(len(group.sites)), group.pool.n_pages)
+
+    def carry(self, array):
+        """From the next step on, every step's metadata holds the step array `array`."""
+        if array not in self.carried:
+            self.carried.append(array)
 
     # -- the step -------------------------------------------------------------
     def check(self, entries):
@@ -140,6 +144,9 @@ class ModelRunner:
             seen.add(e.request)
             if e.request not in lengths:
                 raise KeyError(f"unknown request {e.request!r}")
+            if e.request in self._failed:
+                raise RuntimeError(f"request {e.request!r} was in a step that failed after its kernels may have changed its "
+                                   f"state: it cannot be stepped again, only released")
             n = len(e.tokens)
             if n == 0:
                 raise ValueError(f"request {e.request!r} brings no tokens")
@@ -163,10 +170,18 @@ class ModelRunner:
 
     def step(self, entries: List[StepEntry]):
         """Float logits [sum(len(want)), vocab] on the GPU (valid until the next step)."""
+        if torch.cuda.current_stream(self.device) != self.stream:
+            # pages that a request gave back are used again without a wait, and copies on write are queued before the
+            # kernels that need them: both are right only because everything runs on one stream, in order
+            raise RuntimeError("a step must be launched on the stream that its runner was made on")
         self.check(entries)
         # slots first, the requests' lengths only once the step is launched (the reference commits after it has
         # submitted the work, runtime/execution.py:125-126): a step that fails on the way (a shape that a kernel
-        # refuses, no memory for a buffer) leaves every request where it stood, and can be tried again
+        # refuses, no memory for a buffer) leaves the length and the pages of every request where they stood.  With a
+        # cache of keys and values only, that is the whole of a request and the step can be tried again (what its
+        # kernels wrote lies beyond the lengths and is written again).  A per-request state is another matter: kernels
+        # launched before the failure may have updated it, and nothing keeps the old one, so the requests of such a
+        # model are marked failed and can only be released.
         done = self.cache.append_many([(e.request, len(e.tokens)) for e in entries], commit=False)  # OutOfPages changes nothing
         try:
             if self.execution == "graph":
@@ -174,11 +189,16 @@ class ModelRunner:
             else:
                 ctx = self._context(entries, done)
                 logits = self._forward(ctx, any(e.pending for e in entries))
+                self.counters["eager_steps"] += 1
         except BaseException:
             self.cache.abandon(done)
+            self._last_wanted = None          # the metadata of a step that never ran: nothing to pick from
+            if self.cache.state_needs:
+                self._failed.update(e.request for e in entries)
             raise
         self.cache.commit(done)
         self.steps += 1
+        self.counters["steps"] += 1
         if logits is None:
             return torch.empty((0, self.model.vocab_size), dtype=torch.float32, device=self.device)
         return logits
@@ -192,6 +212,8 @@ class ModelRunner:
         """Pick a token for each row of the last step's logits and leave it on the device, where a later
         step takes it from (StepEntry.pending); the host does not wait.  Returns PickedTokens, to be read
         before three more calls of this function."""
+        if self._last_wanted is None:
+            raise ValueError("the logits are not those of the last step (it failed, or none has run)")
         requests, slots, where = self._last_wanted
         if logits.shape[0] != len(requests):
             raise ValueError("the logits are not those of the last step")
@@ -205,7 +227,7 @@ class ModelRunner:
         entry[1].record()
         return PickedTokens(entry[0].numpy(), entry[1], requests, slots)
 
-    _FIXED = 10   # arrays of the metadata before the cache groups'
+    _FIXED = 9   # arrays of the metadata before the cache groups'
 
     def _width(self, context):
         """Block-table entries a step carries per request: what its longest context needs, in steps of 16 entries,
@@ -213,12 +235,13 @@ class ModelRunner:
         need = -(-int(context) // self.page_size)
         return min(self.table_width, -(-need // 16) * 16)
 
-    def _layout(self, T, S, R, W):
+    def _layout(self, T, S, R, W, carried):
         """Offsets of the packed int32 metadata: tokens, positions, seg_of_row, seg_start, seg_first_pos,
-        state_slots, logit_rows, token_source, logit_slots, single_rows, then per group slots and tables, then one
-        attention task list per known tiling (its length is the most tiles that T rows in S segments can make)."""
+        state_slots, logit_rows, token_source, logit_slots, then per group slots and tables, then the step arrays
+        that parts asked for."""
         G = len(self.cache.groups)
-        sizes = [T, T, T, S + 1, S, S, R, T, R, S] + [T, S * W] * G + [4 * (-(-T // r) + S) for r in self.task_tilings]
+        sizes = [T, T, T, S + 1, S, S, R, T, R] + [T, S * W] * G + [int(array.words(T, S)) for array in carried]
+        self.counters["layouts"] += 1
         return np.concatenate(([0], np.cumsum(sizes))).astype(np.int64)
 
     def _table_rows(self, g, done, W):
@@ -236,18 +259,19 @@ class ModelRunner:
                 stamps[d.state_slot] = stamp
         return mirror[[d.state_slot for d in done], :W]
 
-    def _single_segments(self, done):
-        """How many one-token segments of a mixed step get an attention launch of their own: all of them, if
-        one of them has a long context; none in a step of one-token segments only, or of short contexts."""
-        singles = [d.start + 1 for d in done if d.count == 1]
-        if not singles or len(singles) == len(done) or max(singles) < self.split_single_from:
-            return 0
-        return len(singles)
+    def _launch_values(self, done):
+        """What the parts' launches depend on beside rows, segments and contexts: the launch value of every carried
+        step array that has one (context.StepArray), for this batch."""
+        batch = Batch([d.count for d in done], [d.start for d in done], None, all(d.count == 1 for d in done), {})
+        for array in self.carried:
+            batch.launch_values[array] = array.launch_value(batch)
+        return batch.launch_values
 
-    def _context(self, entries, done, pad=None, device_buffer=None, n_single=None, context=None):
+    def _context(self, entries, done, pad=None, device_buffer=None, launch_values=None, context=None):
         """Build the step's metadata on the host, upload it in one copy and wrap it.
         `pad` = (T, S, R) pads the batch with inert rows (for captured programs):
-        token 0 at position 0, no segment, no cache slot."""
+        token 0 at position 0, no segment, no cache slot.  `launch_values`: those of the captured program
+        (rounded up), instead of the batch's own."""
         counts = [d.count for d in done]
         starts = [d.start for d in done]
         n_rows, n_seg = sum(counts), len(entries)
@@ -256,17 +280,16 @@ class ModelRunner:
         # the longest context of the step (a captured program brings the bound of its bucket) sizes the block tables
         longest = max(s + c for s, c in zip(starts, counts))
         W, G, F = self._width(longest if context is None else context), len(self.cache.groups), self._FIXED
-        layout = (T, S, R, W, tuple(self.task_tilings))
+        carried = tuple(self.carried)
+        layout = (T, S, R, W, carried)
         offsets = self._layouts.get(layout)
         if offsets is None:
-            offsets = self._layouts[layout] = [int(x) for x in self._layout(T, S, R, W)]
+            offsets = self._layouts[layout] = [int(x) for x in self._layout(T, S, R, W, carried)]
         total = offsets[-1]
         host = self._stage(total)
         arr = host.numpy()
-        tokens, positions, seg_of_row, seg_start, seg_first, state_slots, logit_rows, token_source, logit_slots, single_rows = (
-            arr[offsets[i]:offsets[i + 1]] for i in range(10))
-        if n_single is None:      # (a captured program brings its padded number)
-            n_single = self._single_segments(done)
+        tokens, positions, seg_of_row, seg_start, seg_first, state_slots, logit_rows, token_source, logit_slots = (
+            arr[offsets[i]:offsets[i + 1]] for i in range(F))
         decode_only = n_rows == n_seg
         slot_of = [d.state_slot for d in done]
         wanted_seg = [s for s, e in enumerate(entries) for _ in e.want]
@@ -316,21 +339,13 @@ class ModelRunner:
             if pad is not None:
                 slots[n_rows:] = -1
                 tables[n_seg:] = -1
-        single_rows[:] = -1
-        if n_single:
-            own = [int(first_row[s]) for s, c in enumerate(counts) if c == 1]
-            single_rows[:len(own)] = own
-        tilings = list(self.task_tilings)
-        for i, rows_per_tile in enumerate(tilings):
-            tasks = arr[offsets[F + 2 * G + i]:offsets[F + 1 + 2 * G + i]].reshape(-1, 4)
-            if decode_only:      # one tile of one row a segment
-                n = n_seg
-                tasks[:n, 0] = tasks[:n, 1] = first_row
-                tasks[:n, 2] = 1
-                tasks[:n, 3] = 0
-            else:
-                n = fill_tasks(tasks, counts, rows_per_tile, starts, skip_single=n_single > 0)
-            tasks[n:] = (-1, 0, 0, 0)   # tiles of no segment do nothing
+        # what the parts asked for: first every launch value, then the arrays (one may read another's value)
+        batch = Batch(counts, starts, first_row, decode_only, {})
+        for array in carried:
+            own = array.launch_value(batch)
+            batch.launch_values[array] = own if launch_values is None or own is None else launch_values.get(array, 0)
+        for i, array in enumerate(carried):
+            array.fill(arr[offsets[F + 2 * G + i]:offsets[F + 1 + 2 * G + i]], batch, batch.launch_values[array])
         dev = self._upload(host, total, device_buffer)
 
         def view(i, shape=None):
@@ -342,9 +357,9 @@ class ModelRunner:
         ctx.tokens, ctx.positions, ctx.seg_of_row = view(0), view(1), view(2)
         ctx.seg_start, ctx.seg_first_pos, ctx.state_slots, ctx.logit_rows = view(3), view(4), view(5), view(6)
         ctx.token_source = view(7)
-        ctx.single_rows, ctx.n_single = view(9), n_single
         ctx.kv = [GroupView(view(F + 2 * g), view(F + 1 + 2 * g, (S, W)), self.page_size, W) for g in range(G)]
-        ctx.tasks = {r: view(F + 2 * G + i, (-1, 4)) for i, r in enumerate(tilings)}
+        ctx.batch = batch
+        ctx.arrays = {array: (view(F + 2 * G + i), batch.launch_values[array]) for i, array in enumerate(carried)}
         self._last_wanted = ([entries[s].request for s in wanted_seg], wanted_slots, view(8)[:n_want])
         ctx.segments = [(d.request, d.start, d.count) for d in done]
         ctx.max_context = ctx.span_hint = longest
@@ -379,39 +394,44 @@ class ModelRunner:
     # -- captured programs ------------------------------------------------------------
     def _program_key(self, entries, done):
         """What the launches of a step depend on: the padded numbers of rows, segments and
-        wanted rows, whether every segment brings one token, and the context length rounded up
-        to a power of two (it decides how attention splits the keys).  Steps with the same key
+        wanted rows, whether every segment brings one token, the context length rounded up
+        to a power of two (parts size their launches by it), whether tokens are taken from the device, and the
+        launch values of the step arrays that parts carry (rounded up; those that are zero are left out, so that
+        an array which joins later changes no key of a step it has nothing to say about).  Steps with the same key
         replay one captured graph; only the metadata they read differs."""
         rows = sum(d.count for d in done)
         wanted = sum(len(e.want) for e in entries)
         decode_only = all(d.count == 1 for d in done)
         context = 1 << (max(d.start + d.count for d in done) - 1).bit_length()
+        values = tuple((array, _bucket(value)) for array, value in self._launch_values(done).items() if value)
         return (_bucket(rows), _bucket(len(entries)), _bucket(wanted), decode_only, max(context, 256),
-                any(e.pending for e in entries), _bucket(self._single_segments(done)))
+                any(e.pending for e in entries), values)
 
     def _run_program(self, key, entries, done):
-        T, S, R, decode_only, context, take, n_single = key
+        T, S, R, decode_only, context, take, values = key
         program = self.programs.get(key)
         if program is None:
-            program = {"meta": None, "graph": None, "runs": 0, "tilings": None}
+            program = {"meta": None, "graph": None, "runs": 0, "carried": None}
             self.programs[key] = program
             while len(self.programs) > self.program_capacity:
                 oldest = next(iter(self.programs))
                 torch.cuda.synchronize()
                 del self.programs[oldest]
                 self.workspace.release(oldest)
+                self.counters["evictions"] += 1
         else:
             self.programs[key] = self.programs.pop(key)  # most recently used last
-        if program["tilings"] != self.task_tilings:
-            # a mixer asked for a task list that the metadata did not hold yet: lay it out again
+        if program["carried"] != self.carried:
+            # a part asked for a step array that the metadata did not hold yet: lay it out again
             torch.cuda.synchronize()
-            program.update(meta=torch.zeros(int(self._layout(T, S, R, self._width(context))[-1]), dtype=torch.int32, device=self.device),
-                           graph=None, runs=0, tilings=list(self.task_tilings))
-        ctx = self._context(entries, done, pad=(T, S, R), device_buffer=program["meta"], n_single=n_single, context=context)
+            words = int(self._layout(T, S, R, self._width(context), tuple(self.carried))[-1])
+            program.update(meta=torch.zeros(words, dtype=torch.int32, device=self.device),
+                           graph=None, runs=0, carried=list(self.carried))
+        ctx = self._context(entries, done, pad=(T, S, R), device_buffer=program["meta"], launch_values=dict(values), context=context)
         ctx.owner = key
         ctx.span_hint = context   # launch shapes inside a captured program depend on the key only
         ctx.decode_only = decode_only
-        if program["graph"] is None and program["runs"] >= 1 and program["tilings"] == self.task_tilings:
+        if program["graph"] is None and program["runs"] >= 1 and program["carried"] == self.carried:
             # the first run was eager and allocated every buffer; capture launches nothing
             # nothing but kernel launches may happen while the stream records: keep the garbage
             # collector from freeing device objects (other graphs, events) in the middle of it
@@ -426,178 +446,35 @@ class ModelRunner:
                 if collecting:
                     gc.enable()
             program["graph"] = graph
+            self.counters["captures"] += 1
         if program["graph"] is not None:
             program["graph"].replay()
             logits = program["logits"]
+            self.counters["replays"] += 1
         else:
             logits = self._forward(ctx, take)
+            self.counters["eager_steps"] += 1
         program["runs"] += 1
         wanted = sum(len(e.want) for e in entries)
         if logits is None:
             return torch.empty((0, self.model.vocab_size), dtype=torch.float32, device=self.device)
         return logits[:wanted]
 
-    # -- attention dispatch -------------------------------------------------------
-    def attention(self, ctx, q, q_row_stride, kcache, vcache, view, out, heads, kv_heads, head_dim, window, scale,
-                  defer_merge=None):
-        """bfloat16 with a head size in steps of 8 and pages of a power of two >= 4 run
-        on the matrix cores (one block per row for decode steps, tiles of rows from a
-        task list otherwise); everything else runs the exact row-wise kernel.
-
-        `defer_merge(splits) -> bool`: the caller's next product can merge the partial results of a decode step whose
-        keys are split over `splits` blocks itself (ops.gemm_merged).  Where that is so, no merge kernel runs, `out`
-        is left alone and (partial outputs bf16, statistics float, splits) is returned; otherwise None."""
-        rows = out.shape[0]
-        span = ctx.span_hint if not window else min(ctx.span_hint, window + 31)
-        if ops.mfma_attention_supported(out.dtype, head_dim, view.page_size):
-            group = heads // kv_heads
-            heads_per_chunk = min(group, 16)
-            if ctx.decode_only:
-                blocks = rows * kv_heads * -(-group // heads_per_chunk)
-                waves, splits = self._rows_launch(blocks, span, heads_per_chunk, head_dim)
-                if splits > 1 and defer_merge is not None:
-                    # the product that follows merges 2, 4 or 8 partial results of a row while it prepares its operand:
-                    # one kernel fewer than merging here.  Every block of that product reads them all, so more than 8
-                    # rows bring at most 4 each.  (135M sizes, 8 rows at 2k: a step of 0.808 ms with the merge kernel,
-                    # 0.808 with 4 splits merged there, whose attention blocks are half as many, 0.784 with 8.)
-                    fused = next((n for n in (8, 4, 2) if n <= splits and (n <= 4 or rows <= 8) and defer_merge(n)), None)
-                    if fused is not None:
-                        workspace = (ctx.buffer("attn.part_o16", (rows * heads * fused * head_dim,), torch.bfloat16),
-                                     ctx.buffer("attn.part_ml", (rows * heads * fused * 2,), torch.float32))
-                        ops.attention_mfma(q, q_row_stride, kcache, vcache, view.tables, ctx.seg_of_row, ctx.positions, out,
-                                           heads, kv_heads, head_dim, view.page_size, window, scale, None, fused, workspace, waves,
-                                           merge=False)
-                        return workspace[0], workspace[1], fused
-                workspace = None
-                if splits > 1:
-                    workspace = (ctx.buffer("attn.part_o", (rows * heads * splits * head_dim,), torch.float32),
-                                 ctx.buffer("attn.part_ml", (rows * heads * splits * 2,), torch.float32))
-                ops.attention_mfma(q, q_row_stride, kcache, vcache, view.tables, ctx.seg_of_row, ctx.positions, out,
-                                   heads, kv_heads, head_dim, view.page_size, window, scale, None, splits, workspace, waves)
-            else:
-                if ctx.n_single:
-                    # the decoded tokens of this mixed step: a launch of their own that splits their keys
-                    n = ctx.n_single
-                    waves, splits = self._rows_launch(n * kv_heads * -(-group // heads_per_chunk), span, heads_per_chunk, head_dim)
-                    workspace = None
-                    if splits > 1:
-                        workspace = (ctx.buffer("attn.part_o", (n * heads * splits * head_dim,), torch.float32),
-                                     ctx.buffer("attn.part_ml", (n * heads * splits * 2,), torch.float32))
-                    ops.attention_mfma(q, q_row_stride, kcache, vcache, view.tables, ctx.seg_of_row, ctx.positions, out,
-                                       heads, kv_heads, head_dim, view.page_size, window, scale, None, splits, workspace, waves,
-                                       row_ids=ctx.single_rows[:n])
-                kind, item_tiles, halves = self.prompt_attention_form(rows, ctx.n_segments, span, heads, kv_heads, head_dim, view.page_size)
-                tasks = ctx.attention_tasks((16 if kind == "tiles" else 64) * item_tiles // heads_per_chunk)
-                ops.attention_mfma(q, q_row_stride, kcache, vcache, view.tables, ctx.seg_of_row, ctx.positions, out,
-                                   heads, kv_heads, head_dim, view.page_size, window, scale, tasks, waves=self.tile_waves,
-                                   block_tiles={"tiles": False, "block": True, "square": 32}[kind], item_tiles=item_tiles,
-                                   key_groups=halves)
-            return
-        splits = self._splits(rows * heads, span)
-        workspace = None
-        if splits > 1:
-            workspace = (ctx.buffer("attn.part_o", (rows * heads * splits * head_dim,), torch.float32),
-                         ctx.buffer("attn.part_ml", (rows * heads * splits * 2,), torch.float32))
-        ops.attention_rowwise(q, q_row_stride, kcache, vcache, view.tables, ctx.seg_of_row, ctx.positions, out,
-                              heads, kv_heads, head_dim, view.page_size, window, scale, splits, workspace)
-
-    def prompt_attention_form(self, rows, n_segments, span, heads, kv_heads, head_dim, page_size):
-        """Which form of the matrix-core kernel the prompt rows of a step take, (kind, n, halves): ("tiles", n, 1): a block
-        is one tile of 16 n items (a token row and a query head) whose waves split its keys; ("block", n, 1): 64 n items,
-        four waves that own different rows and share keys and values through LDS; ("square", n, halves): 64 n items on
-        the 32 x 32 instruction with waves of their own for the copies, as one half or as two that take the even and the
-        odd steps.  `span`: the longest context of the step."""
-        group = heads // kv_heads
-        heads_per_chunk = min(group, 16)
-        long_portions = rows >= 16 * n_segments
-        if long_portions and head_dim <= 128:
-            # enough long portions to fill the GPU with blocks of 64 items (or more): the waves of a block own different
-            # rows and share each step's keys and values through LDS.  Otherwise (few heads, short portions) the waves
-            # of a block share one tile of 16 items (32 with small heads) and split its keys, which is what hides
-            # the latency of a step when blocks are scarce.
-            blocks = -(-rows // (64 // heads_per_chunk)) * kv_heads * -(-group // heads_per_chunk)
-            # Long contexts: the 32 x 32 form, with three steps in flight a wave.  It costs about 3 us more to start
-            # than the others, so it is for tiles that walk a thousand keys and more; larger blocks share the copies
-            # among more waves but need more blocks to fill the GPU (MI355X, 2,048 rows: 1.7B sizes 61 us -> 46,
-            # 8B sizes 115 -> 71, 135M sizes 32 -> 30; 4,096 rows at the 1.7B sizes: 147 with 128 items, 125 with 256).
-            if page_size >= 8 and self.square_tiles != 0:
-                n = 0
-                if self.square_tiles is not None:
-                    n = self.square_tiles
-                elif span >= 1024 and blocks >= 512:
-                    # from 2,048 blocks of 64 items on: 192 items, six computing waves beside the two that copy (eight waves:
-                    # a compute unit holds two such blocks with small heads, one with large, and no wave slot stays empty).
-                    # 32 heads of 64 at 16k rows: 1.42 ms against 1.46 with 256 items and 1.54 with 128; 9 heads over 3 at
-                    # 32k: 1.49 against 1.58 and 1.61; 32 heads of 128 over 8 at 8k: 0.60 against 0.63 with 128 items
-                    # (heads of more than 64 coordinates, one computing wave a SIMD: already from 1,100 blocks on; 32 heads
-                    # of 128 over 8 at 3,072 rows, 1,536 blocks: 106 us against 123; 24 heads of 96 over 8: 72 against 84)
-                    n = 3 if blocks >= (2048 if head_dim <= 64 else 1100) else 2
-                elif span >= 1024 and blocks >= 128:
-                    # (fewer blocks than compute units and a thousand keys: 64-item blocks, in two halves; 1,024 rows of
-                    # 12 heads of 128 take 25 us against 35 as LDS block tiles, of 16 heads of 64 over 4: 17 against 18)
-                    n = 1
-                if n:
-                    # about one block a compute unit: the time is the longest tile's chain of steps, which two halves a
-                    # block cut in two (2,048 rows at the 135M sizes 31.6 -> 28.4 us, 4,096 rows 64 -> 55; with more
-                    # blocks than that the halves only crowd the compute units: 46 -> 68 us at the 1.7B sizes)
-                    # (up to 511 blocks of 64 items when the chain is long: 3,072 rows at the 135M sizes, 441 blocks,
-                    # 35.6 us against 43.4; 16 heads over 4 at 1,536 rows 22.1 against 25.4; at 1,000 rows the halves lose)
-                    # and up to 512 blocks of 128 items from 3,072 keys on: 8 heads of 64 at 6,144 rows 71 against 89,
-                    # 9 over 3 at 6,144 rows 76 against 92, 16 over 4 at 3,072 rows 42 against 50
-                    few = (-(-blocks // n) <= 320 or (n == 1 and span >= 1536)
-                           or (n == 2 and -(-blocks // n) <= 512 and span >= 3072))
-                    fits = n == 1 or (n == 2 and head_dim <= 64)
-                    halves = 2 if (few and fits if self.square_halves is None else self.square_halves == 2 and fits) else 1
-                    return "square", n, halves
-            block_tiles = (2 if blocks >= 2048 else 1 if blocks >= 512 else 0) if self.block_tiles is None else self.block_tiles
-            if block_tiles:
-                return "block", block_tiles, 1
-        return "tiles", 2 if self.item_tiles == 2 and long_portions and head_dim <= 64 else 1, 1
-
-    @staticmethod
-    def _splits(waves, span):
-        """Row-wise kernel: how many ways a row's keys are split among wavefronts: enough to
-        fill the GPU when the batch alone does not, never finer than 256 keys a split."""
-        if waves >= 2048 or span <= 256:
-            return 1
-        return int(min(32, -(-span // 256), max(1, 4096 // waves)))
-
-    @staticmethod
-    def _rows_launch(blocks, span, heads_per_chunk, head_dim):
-        """Matrix-core decode kernel: (wavefronts a block, blocks along the keys).  Few rows:
-        eight waves share a row's keys inside one block; when that still leaves the GPU idle
-        and the context is long, the keys are also split over blocks (a merge kernel follows).
-        Many rows: four waves a block, one block a row and head group, or with small heads eight waves
-        when that gives every compute unit at most one block."""
-        steps = -(-span // 32)
-        few = blocks < 128
-        # eight waves a block with few rows and small heads (at 8k and 32k too, now that at most eight splits of few
-        # rows are merged by the product that follows: 4 rows at 8k 15.3 us against 16.3 with four waves, 8 rows at
-        # 32k 44.4 against 46.5)
-        waves = 8 if few and head_dim <= 64 else 4
-        if steps <= 2 * waves:
-            # two steps a wave: nothing to split (a second block along the keys and the merge cost 2 us of 8 to 10)
-            return waves, 1
-        if few:
-            # Few rows: split the keys until the blocks fill the GPU once: an eight-wave block fills a compute
-            # unit (256 blocks; more start a second round: 16 splits of 8 rows at 2k to 4k are 10 % slower than
-            # 8), four-wave blocks fit three a unit, of which two are worth having (512 blocks: a thousand are
-            # 12 % slower at 30k, where each then lives for three steps a wave only).  A wave keeps at least one
-            # 32-key step (with two, 8 rows at 2k have 4 splits and are 5 % slower).
-            # At most 32 splits: a single row of 8 key heads at 8k takes 23 us with 32 and 30 with 64.
-            room = 256 if waves == 8 else 512
-            splits = int(max(1, min(steps // waves, room // blocks, 32)))
-        elif head_dim <= 64 and 140 <= blocks <= 256:
-            # enough rows to give most compute units one block of eight waves, and no more than one each: the
-            # keys are not split and no merge follows (9-11 % faster than four waves and three or four splits at
-            # 144 to 256 blocks and 2k keys, 4-5 % at 8k)
-            waves, splits = 8, 1
-        else:
-            # Many rows split until every compute unit has the blocks of four waves that its registers hold (three
-            # with small heads, two otherwise: 3-5 % faster at 384 blocks of the 135M sizes than one block a unit;
-            # from 512 blocks on a split costs 3-8 %); a wave keeps at least four 32-key steps (with two, 128 rows at
-            # 512 keys take 19.4 us against 16.5 unsplit).
-            target = 768 if head_dim <= 64 else 512
-            per = target // blocks if head_dim <= 64 and blocks > 256 else -(-target // blocks)
-            splits = int(max(1, min(steps // (waves * 4), per, 64)))
-        return waves, splits
+    # -- what it holds ------------------------------------------------------------------
+    def report(self):
+        """Counters and bytes of the step function, as the reference's executor reports its own
+        (runtime/execution.py:156-165: captures, replays, workspace and staging bytes; runtime/device.py:81-112):
+        steps run, how many kernel by kernel, programs captured, replayed and evicted, metadata layouts made;
+        bytes of the intermediate buffers, of the products' scratch memory, of the pinned and device staging of the
+        metadata, of the captured programs' own metadata; the step arrays that parts asked for; the cache report."""
+        staging = sum(e[0].numel() * 4 for e in self._staging if e is not None)
+        return {
+            **self.counters,
+            "execution": self.execution,
+            "programs": len(self.programs), "program_capacity": self.program_capacity,
+            "workspace_bytes": self.workspace.bytes(), "scratch_bytes": self.scratch.bytes(),
+            "staging_host_bytes": staging, "staging_device_bytes": staging,
+            "program_metadata_bytes": sum(p["meta"].numel() * 4 for p in self.programs.values() if p["meta"] is not None),
+            "step_arrays": [repr(a) for a in self.carried],
+            "cache": self.cache.report(),
+        }

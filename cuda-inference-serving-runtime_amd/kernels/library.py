@@ -33,7 +33,8 @@ HIPCC_FLAGS = [
 _lock = threading.Lock()
 _libs = {}
 
-CORE = "kernels"                                   # everything but the matrix-core attention
+CORE = "kernels"                                   # everything but the matrix-core attention and the measurement kernels
+MEASURE = "measure"                                # kernels that only measure the machine; the engine never loads them
 ATTENTION_PADS = (32, 64, 96, 128, 160, 192, 224, 256)
 
 
@@ -52,12 +53,14 @@ def attention_unit(dpad):
 def units():
     """The shared objects the kernels are built into: the core, and one per padded head size of the
     matrix-core attention (a model needs only its own, so a first call compiles only that one)."""
-    return [CORE] + [attention_unit(d) for d in ATTENTION_PADS]
+    return [CORE, MEASURE] + [attention_unit(d) for d in ATTENTION_PADS]
 
 
 def sources(unit=CORE):
     if unit == CORE:
-        return sorted(p for p in CSRC.glob("*.hip") if not p.name.startswith("attention_mfma_d"))
+        return sorted(p for p in CSRC.glob("*.hip") if not p.name.startswith("attention_mfma_d") and p.stem != MEASURE)
+    if unit == MEASURE:
+        return [CSRC / "measure.hip"]
     path = CSRC / f"attention_mfma_{unit[len('attn_'):]}.hip"
     if not path.exists():
         raise KernelLibraryError(f"no source for kernel unit {unit}")

@@ -8,7 +8,6 @@ graph.  Nothing here computes on the CPU.  One kind of call leaves the kernels o
 products of more than 64 rows, which go to the vendor's library through torch.mm (see library_ok).
 """
 import ctypes as C
-import os
 
 import torch
 
@@ -47,10 +46,7 @@ def _declare(h):
         "cisr_rope_scatter": [p, p, p, p, p, p, p, i, i, i, i, i, i, i, i, i, i, p],
         "cisr_page_copy": [p, p, p, i, i, ll, ll, p],
         "cisr_f32_to_bf16": [p, p, ll, p],
-        "cisr_idle": [i, p],
         "cisr_bias_add": [p, p, ll, i, i, i, p],
-        "cisr_stream_read": [p, ll, p, i, p],
-        "cisr_grid_meet": [p, p, i, i, i, C.c_uint, p],
         "cisr_attn_rowwise": [p, i, p, p, p, p, p, p, p, p, i, i, i, i, i, i, i, f, i, i, p],
         "cisr_gemm_f32": [p, i, p, i, p, i, p, i, i, i, i, p],
         "cisr_gemm_bf16": [p, i, p, i, p, i, p, i, i, i, i, i, p],
@@ -93,13 +89,10 @@ def _attention_entry(dpad):
     return fn
 
 
-def prepare(head_dims=(), dtype=None):
-    """Build, side by side, whatever a model with these attention head sizes will load: the core, and for
-    bfloat16 the matrix-core attention of each head size that it supports."""
-    wanted = [library.CORE]
-    if dtype == torch.bfloat16:
-        wanted += [library.attention_unit(-(-d // 32) * 32) for d in head_dims if d % 8 == 0 and 0 < d <= 256]
-    library.ensure(wanted)
+def prepare(units=()):
+    """Build, side by side, the core and the further shared objects `units` (names of library.units(): what the
+    parts of a model say they need, `kernel_units`), and load the core."""
+    library.ensure([library.CORE] + [u for u in dict.fromkeys(units) if u != library.CORE])
     lib()
 
 
@@ -286,35 +279,6 @@ def f32_to_bf16(x, out):
     return out
 
 
-def idle(blocks=1):
-    """Launches a kernel of `blocks` blocks that does nothing (the cost of a launch, for measurement)."""
-    _check(lib().cisr_idle(int(blocks), _stream()), "idle")
-
-
-def stream_read(buffer, sink, blocks=512):
-    """Reads every byte of `buffer` once and keeps nothing (the read bandwidth of the memory, for measurement).
-    `sink`: a GPU tensor of at least 4 bytes."""
-    nbytes = buffer.numel() * buffer.element_size()
-    if not buffer.is_contiguous() or nbytes % 16 or buffer.data_ptr() % 16:
-        raise KernelError("stream_read: a contiguous buffer of a multiple of 16 bytes, 16-byte aligned")
-    _check(lib().cisr_stream_read(buffer.data_ptr(), nbytes, _dev(sink, "sink"), int(blocks), _stream()), "stream_read")
-
-
-def grid_meet(blocks, rounds, exchange=0, spin_limit=1 << 22):
-    """One kernel of `blocks` blocks (a multiple of 32, at most 512) that all meet `rounds` times, passing `exchange`
-    floats through memory at each meeting (what a barrier over the whole grid costs beside a launch, for measurement).
-    Returns the words it counted in: [0] the number of groups of 32 blocks that arrived, over all rounds, [-1] is set
-    when a block gave up waiting after `spin_limit` polls."""
-    if blocks <= 0 or blocks % 32 or blocks > 512 or rounds * blocks >= 1 << 31 or exchange < 0:
-        raise KernelError(f"grid_meet: {blocks} blocks must be a multiple of 32, at most 512, and {rounds} rounds few enough to count")
-    device = torch.device("cuda", torch.cuda.current_device())
-    words = torch.zeros(1024, dtype=torch.int32, device=device)
-    passed = torch.empty(max(2 * exchange, 1), dtype=torch.float32, device=device)
-    _check(lib().cisr_grid_meet(words.data_ptr(), passed.data_ptr(), int(exchange), int(blocks), int(rounds), int(spin_limit),
-                                _stream()), "grid_meet")
-    return words
-
-
 def attention_rowwise(q, q_row_stride, kcache, vcache, tables, seg_of_row, positions, out, heads, kv_heads, dim,
                       page_size, window, scale, splits=1, workspace=None):
     """Each row attends to its request's cached keys lo..position.  q is a view
@@ -359,10 +323,37 @@ def attention_rowwise(q, q_row_stride, kcache, vcache, tables, seg_of_row, posit
 # sizes), as are all products of small weights, and both save the kernel after the product.  The least weights are
 # those of the 1.7B sizes' output projection (8 MB: 10.7 against 13.9 us at 128 rows, 29 against 33 at 2,048, the
 # residual sum included; the products of the 135M sizes, 0.7 to 3.5 MB, are as fast or faster here).  0 rows: never.
-LIBRARY_MIN_ROWS = int(os.environ.get("CISR_LIBRARY_MIN_ROWS", "65"))
-LIBRARY_MIN_BYTES = int(float(os.environ.get("CISR_LIBRARY_MIN_MB", "8")) * (1 << 20))
+LIBRARY_MIN_ROWS = 65
+LIBRARY_MIN_BYTES = 8 << 20
 LIBRARY_GATED_MIN_ROWS, LIBRARY_GATED_MIN_BYTES = 33, 64 << 20
-_library_scratch = {}   # (device, elements) -> bf16 buffers, never freed: captured programs keep their addresses
+
+
+class ScratchPool:
+    """Device memory that some products need beyond their inputs and outputs: the library's bf16 product before its
+    sum into the residual, the wide kernel's partial sums, the slice winners of the argmax.  A buffer is handed out
+    again to every later call that it is large enough for, and none is freed before `clear`: captured programs keep
+    the addresses.  A step function owns one pool (calls on its stream are ordered, so they can share buffers);
+    calls that name no pool share DEFAULT_SCRATCH."""
+
+    def __init__(self):
+        self.buffers = {}   # (kind, device, dtype) -> [tensors]
+
+    def get(self, kind, elements, dtype, device):
+        pool = self.buffers.setdefault((kind, device, dtype), [])
+        for buf in pool:
+            if buf.numel() >= elements:
+                return buf
+        pool.append(torch.empty(1 << max(int(elements) - 1, 0).bit_length(), dtype=dtype, device=device))
+        return pool[-1]
+
+    def bytes(self):
+        return sum(t.numel() * t.element_size() for pool in self.buffers.values() for t in pool)
+
+    def clear(self):
+        self.buffers.clear()
+
+
+DEFAULT_SCRATCH = ScratchPool()
 
 
 def library_ok(m, w, gated=False):
@@ -377,20 +368,15 @@ def library_ok(m, w, gated=False):
             and w.numel() * 2 >= LIBRARY_MIN_BYTES)
 
 
-def _scratch_bf16(device, rows, cols):
-    pool = _library_scratch.setdefault(device, [])
-    for buf in pool:
-        if buf.numel() >= rows * cols:
-            return buf[:rows * cols].view(rows, cols)
-    pool.append(torch.empty(1 << (rows * cols - 1).bit_length(), dtype=torch.bfloat16, device=device))
-    return pool[-1][:rows * cols].view(rows, cols)
+def _scratch_bf16(scratch, device, rows, cols):
+    return (scratch or DEFAULT_SCRATCH).get("library", rows * cols, torch.bfloat16, device)[:rows * cols].view(rows, cols)
 
 
-def gemm(a, w, out, residual=None, after_norm=False):
+def gemm(a, w, out, residual=None, after_norm=False, scratch=None):
     """out[M, N] = a[M, K] . w[N, K]^T (+ residual).  float operands run the true
     32-bit kernel; bf16 operands run on the matrix cores with float accumulation.
     out may be float or (bf16 operands only) bf16; residual is float and may be `out`.
-    `after_norm`: a hint for the choice of kernel, see wide_ok."""
+    `after_norm`: a hint for the choice of kernel, see wide_ok.  `scratch`: the ScratchPool of the caller's steps."""
     m, k = a.shape
     n, k2 = w.shape
     if k != k2:
@@ -416,11 +402,11 @@ def gemm(a, w, out, residual=None, after_norm=False):
         if residual is None:
             torch.mm(a, w.t(), out=out)
             return out
-        product = _scratch_bf16(a.device, m, n)
+        product = _scratch_bf16(scratch, a.device, m, n)
         torch.mm(a, w.t(), out=product)
         return residual_add(out, product)
     elif a.dtype == torch.bfloat16 and m <= SKINNY_ROWS and _skinny_ok(a, w) and wide_ok(m, w, after_norm=after_norm):
-        return _gemm_wide(a, w, out, residual, False, "gemm")
+        return _gemm_wide(a, w, out, residual, False, "gemm", scratch)
     elif a.dtype == torch.bfloat16 and m <= SKINNY_ROWS and _skinny_ok(a, w):
         code = lib().cisr_gemm_skinny_bf16(a.data_ptr(), a.stride(0), w.data_ptr(), w.stride(0), out.data_ptr(),
                                            out.stride(0), rp, ldr, m, n, k, _storage(out, "out"), 0, None, 0.0, None,
@@ -440,10 +426,9 @@ def gemm(a, w, out, residual=None, after_norm=False):
 # with at most 16 rows the activations are a small part of the traffic and the fused kernels hold out up to
 # about 64 MB; with 17 to 32 rows the wide kernel wins from about 12 MB on, with more from about 30 MB on
 # (a block then holds so much of the activations that it needs many rows of W to spread their cost over).
-WIDE_MIN_BYTES_FEW_ROWS = int(float(os.environ.get("CISR_WIDE_MIN_MB_FEW_ROWS", "64")) * (1 << 20))
-WIDE_MIN_BYTES = int(float(os.environ.get("CISR_WIDE_MIN_MB", "12")) * (1 << 20))
-WIDE_MIN_BYTES_MANY_ROWS = int(float(os.environ.get("CISR_WIDE_MIN_MB_MANY_ROWS", "30")) * (1 << 20))
-_wide_workspaces = {}    # device -> buffers, never freed: captured programs keep their addresses
+WIDE_MIN_BYTES_FEW_ROWS = 64 << 20
+WIDE_MIN_BYTES = 12 << 20
+WIDE_MIN_BYTES_MANY_ROWS = 30 << 20
 _wide_plans = {}
 
 
@@ -482,24 +467,19 @@ def _wide_plan(m, n, k, swiglu):
     return need
 
 
-def _wide_workspace(device, floats):
+def _wide_workspace(scratch, device, floats):
     if floats <= 0:
         return None
-    pool = _wide_workspaces.setdefault(device, [])
-    for buf in pool:
-        if buf.numel() >= floats:
-            return buf
-    pool.append(torch.empty(1 << (floats - 1).bit_length(), dtype=torch.float32, device=device))
-    return pool[-1]
+    return (scratch or DEFAULT_SCRATCH).get("wide", floats, torch.float32, device)
 
 
-def _gemm_wide(a, w, out, residual, swiglu, what):
+def _gemm_wide(a, w, out, residual, swiglu, what, scratch=None):
     m, k = a.shape
     n = w.shape[0] // 2 if swiglu else w.shape[0]
     need = _wide_plan(m, n, k, swiglu)
     if need < 0 or a.stride(0) % 8 or a.data_ptr() % 16:
         raise KernelError(f"{what}: shape not supported by the wide kernel")
-    work = _wide_workspace(a.device, need)
+    work = _wide_workspace(scratch, a.device, need)
     rp, ldr = (residual.data_ptr(), residual.stride(0)) if residual is not None else (None, 0)
     _check(lib().cisr_gemm_wide_bf16(a.data_ptr(), a.stride(0), w.data_ptr(), w.stride(0), out.data_ptr(), out.stride(0),
                                      rp, ldr, m, n, k, _storage(out, "out"), n if swiglu else 0,
@@ -508,7 +488,7 @@ def _gemm_wide(a, w, out, residual, swiglu, what):
     return out
 
 
-def gemm_unfinished(a, w, residual):
+def gemm_unfinished(a, w, residual, scratch=None):
     """The product a . w^T that is to be added to the float rows `residual`, left unfinished where adding it takes a
     kernel of its own: the wide kernel's partial sums of a product cut into slices, (partial sums [slices, M, N],
     slices), or the library's bf16 product, (product [M, N], 0); rmsnorm_partials or add_partials then are that
@@ -521,7 +501,7 @@ def gemm_unfinished(a, w, residual):
     if library_ok(m, w):
         if not a.is_contiguous():
             return None
-        product = _scratch_bf16(a.device, m, n)
+        product = _scratch_bf16(scratch, a.device, m, n)
         torch.mm(a, w.t(), out=product)
         return product, 0
     if not 0 < m <= SKINNY_ROWS or not _skinny_ok(a, w) or not wide_ok(m, w):
@@ -529,7 +509,7 @@ def gemm_unfinished(a, w, residual):
     need = _wide_plan(m, n, k, False)
     if need <= 0:
         return None
-    work = _wide_workspace(a.device, need)
+    work = _wide_workspace(scratch, a.device, need)
     _check(lib().cisr_gemm_wide_partials_bf16(a.data_ptr(), a.stride(0), w.data_ptr(), w.stride(0), m, n, k,
                                               work.data_ptr(), work.numel(), _stream()), "gemm_unfinished")
     return work, need // (m * n)
@@ -577,11 +557,11 @@ def gemm_normed(x, norm, w, out):
     return out
 
 
-def gemm_swiglu(a, w_gate_up, out, scratch=None, norm=None):
+def gemm_swiglu(a, w_gate_up, out, gate_up=None, norm=None, scratch=None):
     """out[M, I] = silu(a . Wg^T) * (a . Wu^T) with w_gate_up = [Wg; Wu] ([2I, K]).
     Few rows of bf16 run one fused weight-streaming kernel (with `norm` = (weight, eps, None), `a` is the float
-    residual and RMSNorm is fused too); otherwise the product goes to `scratch` [M, 2I] and the activation is
-    a second kernel."""
+    residual and RMSNorm is fused too); otherwise the product goes to `gate_up` [M, 2I] and the activation is
+    a second kernel.  `scratch`: the ScratchPool of the caller's steps."""
     m, k = a.shape
     two_i, k2 = w_gate_up.shape
     inter = two_i // 2
@@ -598,12 +578,12 @@ def gemm_swiglu(a, w_gate_up, out, scratch=None, norm=None):
     if out.dtype != a.dtype or a.dtype != w_gate_up.dtype:
         raise KernelError("gemm_swiglu: dtypes differ")
     if a.dtype == torch.bfloat16 and library_ok(m, w_gate_up, gated=True) and a.is_contiguous():
-        product = _scratch_bf16(a.device, m, two_i)
+        product = _scratch_bf16(scratch, a.device, m, two_i)
         torch.mm(a, w_gate_up.t(), out=product)
         return swiglu(product, out)
     if swiglu_fused_ok(a, w_gate_up):
         if m <= SKINNY_ROWS and wide_ok(m, w_gate_up, True, after_norm=True):
-            return _gemm_wide(a, w_gate_up, out, None, True, "gemm_swiglu")
+            return _gemm_wide(a, w_gate_up, out, None, True, "gemm_swiglu", scratch)
         if m <= SKINNY_ROWS:
             _check(lib().cisr_gemm_skinny_bf16(a.data_ptr(), a.stride(0), w_gate_up.data_ptr(), w_gate_up.stride(0),
                                                out.data_ptr(), out.stride(0), None, 0, m, inter, k, BF16, inter, None, 0.0,
@@ -612,10 +592,10 @@ def gemm_swiglu(a, w_gate_up, out, scratch=None, norm=None):
             _check(lib().cisr_gemm_bf16_swiglu(a.data_ptr(), a.stride(0), w_gate_up.data_ptr(), w_gate_up.stride(0),
                                                out.data_ptr(), out.stride(0), m, inter, k, inter, _stream()), "gemm_swiglu")
         return out
-    if scratch is None:
-        raise KernelError("gemm_swiglu: this shape needs a scratch buffer [M, 2I]")
-    gemm(a, w_gate_up, scratch)
-    return swiglu(scratch, out)
+    if gate_up is None:
+        raise KernelError("gemm_swiglu: this shape needs a buffer [M, 2I] for the product of gate and up")
+    gemm(a, w_gate_up, gate_up, scratch=scratch)
+    return swiglu(gate_up, out)
 
 
 def qkv_rope_fused_ok(a, w, head_dim, cos, normed):
@@ -629,7 +609,7 @@ def qkv_rope_fused_ok(a, w, head_dim, cos, normed):
             and a.dtype == (torch.float32 if normed else torch.bfloat16))
 
 
-def qkv_rope(a, w, q_out, positions, slots, cos, sin, kcache, vcache, heads, kv_heads, dim, page_size, norm=None):
+def qkv_rope(a, w, q_out, positions, slots, cos, sin, kcache, vcache, heads, kv_heads, dim, page_size, norm=None, scratch=None):
     """One kernel for a decode step's projections: (RMSNorm of the float residual `a` if `norm` = (weight, eps),
     else `a` is bf16 and normed), product with w = [Wq; Wk; Wv], rotary embedding of q and k, q into
     q_out [M, heads*dim], k and v into the cache at `slots`.  kcache None: w = Wq only (a layer reading
@@ -651,7 +631,7 @@ def qkv_rope(a, w, q_out, positions, slots, cos, sin, kcache, vcache, heads, kv_
     max_pos = cos.shape[0]
     if norm is None and wide_ok(m, w, after_norm=True):
         need = _wide_plan(m, w.shape[0], k, False)
-        work = _wide_workspace(a.device, need)
+        work = _wide_workspace(scratch, a.device, need)
         _check(lib().cisr_qkv_rope_wide(a.data_ptr(), a.stride(0), w.data_ptr(), w.stride(0),
                                         _dev(q_out, "q_out", torch.bfloat16, (m, heads * dim)), heads * dim, m, k,
                                         _dev(positions, "positions", torch.int32, (m,)), sp,
@@ -770,8 +750,6 @@ def mfma_attention_supported(dtype, dim, page_size):
             and page_size & (page_size - 1) == 0)
 
 
-_argmax_scratch = {}
-
 
 def _scatter(out, index, rows):
     """(pointer of index or None, length of out) for a token choice that writes out[index[r]]."""
@@ -782,15 +760,13 @@ def _scatter(out, index, rows):
     return _dev(index, "index", torch.int32, (rows,)), out.numel()
 
 
-def argmax(logits, out, index=None):
+def argmax(logits, out, index=None, scratch=None):
     """out[r] = index of the largest logit of row r (the lowest index wins a tie).  With `index`
     (int32 [R]) the result of row r goes to out[index[r]] instead, or nowhere if that is no place of out."""
     rows, vocab = logits.shape
-    key = (logits.device, rows)
-    if key not in _argmax_scratch:
-        _argmax_scratch[key] = (torch.empty(rows * 32, dtype=torch.float32, device=logits.device),
-                                torch.empty(rows * 32, dtype=torch.int32, device=logits.device))
-    val, idx = _argmax_scratch[key]
+    pool = scratch or DEFAULT_SCRATCH
+    val = pool.get("argmax", rows * 32, torch.float32, logits.device)
+    idx = pool.get("argmax", rows * 32, torch.int32, logits.device)
     where, out_n = _scatter(out, index, rows)
     _check(lib().cisr_argmax(_dev(logits, "logits", torch.float32), out.data_ptr(), where, out_n,
                              val.data_ptr(), idx.data_ptr(), rows, vocab, _stream()), "argmax")

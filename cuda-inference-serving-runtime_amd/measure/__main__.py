@@ -1,0 +1,259 @@
+"""python -m runtime.measure <workload>: what single kernels and the machine cost, one JSON line each.
+
+  floor                    a captured chain of kernels that do nothing (what a launch costs), and a meeting of all
+                           blocks inside one kernel (what a barrier over the grid costs instead)
+  attention                the prompt attention kernel alone at the family's head shapes, in the form the rule picks
+  attention_forms          every form of that kernel at a grid of head shapes, beside the form the rule picks
+  decode_attention_shapes  every launch shape of the decode attention kernel at a grid of requests and contexts,
+                           beside the one the rule picks
+"""
+import argparse
+import json
+import sys
+import time
+
+PEAK_TFLOPS = {"bf16": 2500.0, "fp32": 157.3}
+
+
+def launch_floor(args):
+    """Microseconds a kernel of a captured chain costs when it computes nothing: 1,000 launches of an empty kernel
+    (one block, and one block a compute unit) in one graph, replayed; the median of 20 replays.  A decode step of
+    L layers is 5 L + 4 kernels, so this times that count is the part of a step that no kernel work can remove.
+    Beside it, what the other way to order a step's parts costs: a meeting of all blocks inside one kernel (counters
+    in memory, 200 meetings, the median of 5 runs), alone and with 8 x 576 floats passed from all blocks to all."""
+    import statistics
+    import torch
+    from runtime.config import preset
+    from runtime import measure
+    chain = 1000
+    out = {}
+    for name, blocks in (("one_block", 1), ("block_per_cu", torch.cuda.get_device_properties(0).multi_processor_count)):
+        stream = torch.cuda.Stream()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(stream):
+            measure.idle(blocks)
+            stream.synchronize()
+            with torch.cuda.graph(graph, stream=stream):
+                for _ in range(chain):
+                    measure.idle(blocks)
+        times = []
+        for _ in range(20 + 3):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            graph.replay()
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t0)
+        out[name] = round(statistics.median(times[3:]) / chain * 1e6, 3)
+    # a meeting of all blocks inside one kernel, which a step fused into fewer kernels would need instead of a launch
+    meeting = {}
+    for name, blocks, exchange in (("128_blocks", 128, 0), ("256_blocks", 256, 0), ("256_blocks_passing_18_kb", 256, 8 * 576)):
+        rounds, times = 200, []
+        for _ in range(5 + 1):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            words = measure.grid_meet(blocks, rounds, exchange)
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t0)
+            if int(words[-1]) or int(words[0]) != rounds * (blocks // 32):
+                raise SystemExit(f"grid_meet: {blocks} blocks did not all meet ({int(words[0])} arrivals, flag {int(words[-1])})")
+        meeting[name] = round(statistics.median(times[1:]) / rounds * 1e6, 2)
+    out["meeting_inside_a_kernel"] = meeting
+    layers = preset(args.model)["num_hidden_layers"]
+    kernels = 5 * layers + 4
+    print(json.dumps({"metric": "microseconds a kernel that does nothing costs in a captured chain", "value": out["one_block"],
+                      "unit": "us", "higher_is_better": False, "n_gpus": 1, "chain": chain, "replays": 20, "us_per_kernel": out,
+                      "kernels_of_a_decode_step": kernels, "model": args.model,
+                      "floor_ms_of_a_decode_step": round(kernels * out["one_block"] / 1e3, 4)}))
+    return 0
+
+
+def _time_attention(heads, kv_heads, D, T, P, form, calls=20):
+    """Microseconds of one call of the prompt attention kernel in `form` (kind, n, halves): causal attention of T rows
+    over their own T keys in a paged cache; `calls` calls in one captured graph, the median of five replays."""
+    import statistics
+    import numpy as np
+    import torch
+    from runtime.kernels.attention import fill_tasks
+    from runtime.kernels import ops
+    dev = torch.device("cuda:0")
+    kind, n, halves = form
+    pages = -(-T // P)
+    q = torch.randn(T, heads * D, device=dev).bfloat16()
+    K = torch.randn(pages, kv_heads, P, D, device=dev).bfloat16()
+    V = torch.randn(pages, kv_heads, D, P, device=dev).bfloat16()
+    tables = torch.arange(pages, dtype=torch.int32, device=dev).reshape(1, pages)
+    seg = torch.zeros(T, dtype=torch.int32, device=dev)
+    pos = torch.arange(T, dtype=torch.int32, device=dev)
+    o = torch.empty(T, heads * D, device=dev, dtype=torch.bfloat16)
+    rows_per_tile = (16 if kind == "tiles" else 64) * n // min(heads // kv_heads, 16)
+    host = np.full((-(-T // rows_per_tile), 4), -1, dtype=np.int32)
+    fill_tasks(host, [T], rows_per_tile, [0])
+    tasks = torch.from_numpy(host).to(dev)
+
+    def run():
+        ops.attention_mfma(q, heads * D, K, V, tables, seg, pos, o, heads, kv_heads, D, P, None, D ** -0.5, tasks,
+                           block_tiles={"tiles": False, "block": True, "square": 32}[kind], item_tiles=n, key_groups=halves)
+    stream, graph = torch.cuda.Stream(), torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        run(); stream.synchronize()
+        with torch.cuda.graph(graph, stream=stream):
+            for _ in range(calls):
+                run()
+    times = []
+    for _ in range(6):
+        torch.cuda.synchronize(); t0 = time.perf_counter()
+        graph.replay()
+        torch.cuda.synchronize(); times.append((time.perf_counter() - t0) / calls)
+    return statistics.median(times[1:]) * 1e6
+
+
+def _form_name(form):
+    kind, n, halves = form
+    return f"{kind} x{n}" + (", two halves" if halves == 2 else "")
+
+
+def prompt_attention(args):
+    """The attention kernel alone on whole prompts: causal attention of T rows over their own T keys in a paged cache, at
+    the head shapes of the three family members, in the form the engine chooses for that size.  Twenty calls in one
+    captured graph, the median of five replays; flops are those of the causal half, 4 T (T + 1) / 2 x head size x heads."""
+    from runtime.config import preset
+    P = args.page_size
+    out = {}
+    from runtime.kernels.attention import prompt_form
+    for name in ("smollm2-135m", "smollm2-1.7b", "llama-3-8b"):
+        raw = preset(name)
+        heads, kv_heads = raw["num_attention_heads"], raw["num_key_value_heads"]
+        D = raw.get("head_dim") or raw["hidden_size"] // heads
+        for T in [int(t) for t in args.attention_rows.split(",") if t]:
+            form = prompt_form(T, 1, T, heads, kv_heads, D, P)
+            us = _time_attention(heads, kv_heads, D, T, P, form)
+            flops = 4 * T * (T + 1) / 2 * D * heads
+            out[f"{name}_{T}"] = {"heads": heads, "kv_heads": kv_heads, "head_dim": D, "rows": T, "form": _form_name(form),
+                                  "us": round(us, 1), "pflops": round(flops / us / 1e9, 3),
+                                  "frac_of_bf16_peak": round(flops / us / 1e6 / PEAK_TFLOPS["bf16"], 4)}
+    print(json.dumps({"metric": "prompt attention alone, PFLOP/s of the causal half (bf16, paged cache, page size %d)" % P,
+                      "unit": "PFLOP/s", "n_gpus": 1, "value": out["smollm2-1.7b_%s" % args.attention_rows.split(",")[0]]["pflops"],
+                      "higher_is_better": True, "shapes": out}))
+    return 0
+
+
+def attention_forms(args):
+    """Every form of the prompt attention kernel at a grid of head shapes (heads/key heads x head size, the family's and
+    others) and prompt lengths, beside the form the engine's rule picks: one line a point on stderr, then one JSON line
+    with the worst and the mean loss of the rule against the best form of each point."""
+    P = args.page_size
+    from runtime.kernels.attention import prompt_form
+    forms = [("tiles", 1, 1), ("tiles", 2, 1), ("block", 1, 1), ("block", 2, 1), ("square", 1, 1), ("square", 2, 1),
+             ("square", 3, 1), ("square", 4, 1), ("square", 1, 2), ("square", 2, 2)]
+
+    def takes(form, D, T):
+        kind, n, halves = form
+        if kind == "tiles":
+            return T <= 4096 and (n == 1 or D <= 64)      # (far from the best beyond that, and slow to measure)
+        return kind == "block" or D <= 64 or not (n == 4 or (n == 2 and halves == 2))
+    shapes = [(9, 3, 64), (32, 32, 64), (32, 8, 128), (16, 4, 64), (12, 12, 128), (8, 8, 64), (24, 8, 96), (64, 8, 128)]
+    points, losses = {}, []
+    for heads, kv_heads, D in shapes:
+        for T in [int(t) for t in args.attention_rows.split(",") if t]:
+            us = {form: _time_attention(heads, kv_heads, D, T, P, form, calls=8) for form in forms if takes(form, D, T)}
+            pick = tuple(prompt_form(T, 1, T, heads, kv_heads, D, P))
+            best = min(us, key=us.get)
+            loss = us[pick] / us[best] - 1
+            losses.append(loss)
+            points[f"{heads}/{kv_heads}x{D}_{T}"] = {"pick": _form_name(pick), "pick_us": round(us[pick], 1), "best": _form_name(best),
+                                                    "best_us": round(us[best], 1), "loss": round(loss, 3)}
+            print(f"{heads:2d}/{kv_heads:2d} x {D:3d}  {T:5d} rows  pick {_form_name(pick):22s} {us[pick]:7.1f} us   best {_form_name(best):22s} "
+                  f"{us[best]:7.1f} us   " + "  ".join(f"{_form_name(f)}: {v:.0f}" for f, v in us.items()), file=sys.stderr, flush=True)
+    print(json.dumps({"metric": "loss of the rule that picks the prompt attention form against the best form of each point",
+                      "unit": "fraction", "n_gpus": 1, "value": round(max(losses), 3), "higher_is_better": False,
+                      "mean": round(sum(losses) / len(losses), 4), "points": points}))
+    return 0
+
+
+def decode_attention_shapes(args):
+    """The decode attention kernel alone (one row a request, bf16, paged cache with scattered pages) at the family's head
+    shapes over a grid of requests and contexts: every launch shape (wavefronts a block x blocks along the keys, with the
+    merge kernel when the keys are split) beside the one `kernels.attention.rows_launch` picks.  Keys and values of up to
+    eight layers take turns, so that nothing is read from a cache twice in a row.  One line a point on stderr, then one
+    JSON line with the worst and the mean loss of the rule."""
+    import math
+    import torch
+    from runtime.config import preset
+    from runtime.kernels import ops
+    from runtime.kernels.attention import rows_launch
+    dev, P = torch.device("cuda:0"), args.page_size
+    points, losses = {}, []
+    for name in ("smollm2-135m", "smollm2-1.7b", "llama-3-8b"):
+        raw = preset(name)
+        heads, kv = raw["num_attention_heads"], raw["num_key_value_heads"]
+        D = raw.get("head_dim") or raw["hidden_size"] // heads
+        group = heads // kv
+        per_chunk = min(group, 16)
+        for C in (512, 2048, 8192, 32768):
+            for B in (1, 4, 8, 16, 32, 64, 128):
+                if B * C * kv * D * 4 > 6 << 30:
+                    continue
+                pages_per = -(-C // P)
+                n_pages = B * pages_per
+                copies = int(max(1, min(8, (600 << 20) // (n_pages * kv * P * D * 4))))
+                ks = [torch.randn(n_pages, kv, P, D, device=dev).bfloat16() for _ in range(copies)]
+                vs = [torch.randn(n_pages, kv, D, P, device=dev).bfloat16() for _ in range(copies)]
+                tables = torch.randperm(n_pages, device=dev).int().view(B, pages_per)
+                q = torch.randn(B, heads * D, device=dev).bfloat16()
+                seg = torch.arange(B, device=dev, dtype=torch.int32)
+                pos = torch.full((B,), C - 1, device=dev, dtype=torch.int32)
+                out = torch.empty(B, heads * D, device=dev).bfloat16()
+                blocks = B * kv * -(-group // per_chunk)
+                pick = tuple(rows_launch(blocks, C, per_chunk, D))
+                shapes = {(w, n) for w in (4, 8) for n in (1, 2, 4, 8, 16, 32) if (n == 1 or n * 32 <= C) and blocks * n <= 16384} | {pick}
+                us = {}
+                for waves, splits in sorted(shapes):
+                    ws = (torch.empty(B * heads * splits * D, device=dev), torch.empty(B * heads * splits * 2, device=dev))
+
+                    def run(i):
+                        ops.attention_mfma(q, heads * D, ks[i], vs[i], tables, seg, pos, out, heads, kv, D, P, None, 1 / math.sqrt(D),
+                                           None, splits, ws, waves)
+                    calls = max(copies, 4)
+                    for i in range(copies):
+                        run(i)
+                    torch.cuda.synchronize()
+                    graph = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(graph):
+                        for i in range(calls):
+                            run(i % copies)
+                    graph.replay()
+                    torch.cuda.synchronize()
+                    times = []
+                    for _ in range(3):
+                        t0 = time.perf_counter()
+                        graph.replay()
+                        torch.cuda.synchronize()
+                        times.append((time.perf_counter() - t0) / calls * 1e6)
+                    us[(waves, splits)] = sorted(times)[1]
+                best = min(us, key=us.get)
+                loss = us[pick] / us[best] - 1
+                losses.append(loss)
+                label = lambda shape: f"{shape[0]} waves x {shape[1]}"
+                points[f"{name}_{B}x{C}"] = {"pick": label(pick), "pick_us": round(us[pick], 1), "best": label(best),
+                                             "best_us": round(us[best], 1), "loss": round(loss, 3)}
+                print(f"{name:13s} {B:3d} rows x {C:5d} keys  pick {label(pick):13s} {us[pick]:7.1f} us   best {label(best):13s} {us[best]:7.1f} us   "
+                      + "  ".join(f"{w}x{n}: {v:.1f}" for (w, n), v in sorted(us.items())), file=sys.stderr, flush=True)
+    print(json.dumps({"metric": "loss of the rule that picks the decode attention launch shape against the best shape of each point",
+                      "unit": "fraction", "n_gpus": 1, "value": round(max(losses), 3), "higher_is_better": False,
+                      "mean": round(sum(losses) / len(losses), 4), "points": points}))
+    return 0
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser(prog="python -m runtime.measure")
+    ap.add_argument("workload", choices=["floor", "attention", "attention_forms", "decode_attention_shapes"])
+    ap.add_argument("--model", default="smollm2-135m", help="floor: the preset whose decode step the floor is priced for")
+    ap.add_argument("--page-size", type=int, default=16)
+    ap.add_argument("--attention-rows", default="2048,7936", help="attention workloads: prompt lengths (comma separated)")
+    args = ap.parse_args(argv)
+    return {"floor": launch_floor, "attention": prompt_attention, "attention_forms": attention_forms,
+            "decode_attention_shapes": decode_attention_shapes}[args.workload](args)
+
+
+if __name__ == "__main__":
+    sys.exit(main())

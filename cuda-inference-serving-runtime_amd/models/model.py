@@ -35,10 +35,10 @@ class Model:
             if entry.reads is not None:
                 if not 0 <= entry.reads < index or self.schedule[entry.reads].reads is not None:
                     raise ValueError(f"schedule entry {index} must read an earlier entry that keeps a cache")
-                if self.layers[entry.layer].mixer.cache_need() is not None:
+                if self.layers[entry.layer].cache_need() is not None:
                     raise ValueError(f"schedule entry {index} reads another cache but its mixer keeps one")
-                kept = self.layers[self.schedule[entry.reads].layer].mixer.cache_need()
-                reader = self.layers[entry.layer].mixer
+                kept = self.layers[self.schedule[entry.reads].layer].cache_need()
+                reader = self.layers[entry.layer]
                 wanted = reader.cache_read() if hasattr(reader, "cache_read") else None
                 if kept is None:
                     raise ValueError(f"schedule entry {index} reads entry {entry.reads}, which keeps no cache")
@@ -86,7 +86,7 @@ class Model:
     def cache_needs(self):
         needs = {}
         for index, entry in enumerate(self.schedule):
-            need = self.layers[entry.layer].mixer.cache_need()
+            need = self.layers[entry.layer].cache_need()
             if need is not None and entry.reads is None:
                 needs[index] = need
         return needs
@@ -94,10 +94,18 @@ class Model:
     def state_needs(self):
         needs = {}
         for index, entry in enumerate(self.schedule):
-            need = self.layers[entry.layer].mixer.state_need()
+            need = self.layers[entry.layer].state_need()
             if need is not None:
                 needs[index] = need
         return needs
+
+    def kernel_units(self):
+        """Shared objects beside the core that the model's parts need for its compute dtype."""
+        return [u for part in self.parts() if hasattr(part, "kernel_units") for u in part.kernel_units(self.dtype)]
+
+    def step_arrays(self):
+        """Step arrays that the parts want every step's metadata to carry from the start."""
+        return [a for part in self.parts() if hasattr(part, "step_arrays") for a in part.step_arrays()]
 
     @property
     def max_positions(self):

@@ -18,13 +18,13 @@ import math
 import torch
 
 from ..cache.pages import KVNeed
-from ..kernels import ops
+from ..kernels import attention as kernel, ops
 from .base import Mixer, TensorSpec, matrix_operand, register_part
 
 
 class PagedAttention(Mixer):
     def __init__(self, name, hidden, heads, kv_heads, head_dim, position, window=None, scale=None, own_kv=True,
-                 bias=False, out_bias=False):
+                 bias=False, out_bias=False, tuning=None):
         if heads % kv_heads:
             raise ValueError(f"{heads} query heads are not a multiple of {kv_heads} key/value heads")
         if head_dim % 2 or head_dim > 256:
@@ -34,6 +34,13 @@ class PagedAttention(Mixer):
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)
         self.bias, self.out_bias = bool(bias), bool(out_bias)
         self.w_in = self.w_out = self.b_in = self.b_out = None
+        self.tuning = tuning if tuning is not None else kernel.DEFAULT_TUNING   # what the kernel's launch rules may be told
+
+    def kernel_units(self, dtype):
+        return kernel.kernel_units(self.head_dim, dtype)
+
+    def step_arrays(self):
+        return [kernel.SingleRows(self.tuning.split_single_from)]
 
     def cache_need(self):
         return KVNeed(self.kv_heads, self.head_dim, self.window) if self.own_kv else None
@@ -84,7 +91,7 @@ class PagedAttention(Mixer):
     def forward(self, h, residual, ctx, site, norm=None):
         T = residual.shape[0]
         D, nh, nkv = self.head_dim, self.heads, self.kv_heads
-        gid, kcache, vcache = ctx.cache.kv_of_site(site)
+        gid, kcache, vcache = ctx.cache.pages_of_site(site)
         view = ctx.kv[gid]
         cos, sin = self.position.tables()
         if not self.own_kv:
@@ -96,19 +103,20 @@ class PagedAttention(Mixer):
             q, q_stride = ctx.buffer("attn.q", (T, nh * D), ctx.dtype), nh * D
             ops.qkv_rope(residual if norm is not None else h, self.w_in, q, ctx.positions, slots, cos, sin,
                          kcache_w, vcache_w, nh, nkv, D, view.page_size,
-                         norm=(norm.weight, norm.eps) if norm is not None else None)
+                         norm=(norm.weight, norm.eps) if norm is not None else None, scratch=ctx.scratch)
         else:
             q_stride = (nh + (2 * nkv if self.own_kv else 0)) * D
             q = ctx.buffer("attn.qkv", (T, q_stride), ctx.dtype)
-            ops.gemm(h, self.w_in, q)
+            ops.gemm(h, self.w_in, q, scratch=ctx.scratch)
             if self.b_in is not None:
                 ops.bias_add(q, self.b_in)
             ops.rope_scatter(q, ctx.positions, slots, cos, sin, kcache_w, vcache_w, nh, nkv, D, view.page_size,
                              interleaved=self._interleaved)
         out = ctx.buffer("attn.out", (T, nh * D), ctx.dtype)
         # a decode step of few rows may leave the partial results of its split keys to the output projection
-        unmerged = ctx.attend(q, q_stride, kcache, vcache, view, out, nh, nkv, D, self.window, self.scale,
-                              defer_merge=lambda splits: ops.gemm_merged_ok(T, self.w_out, nh, D, splits))
+        unmerged = kernel.paged_attention(ctx, q, q_stride, kcache, vcache, view, out, nh, nkv, D, self.window, self.scale,
+                                          defer_merge=lambda splits: ops.gemm_merged_ok(T, self.w_out, nh, D, splits),
+                                          tuning=self.tuning)
         if unmerged is not None:
             residual = ops.gemm_merged(unmerged, nh, D, self.w_out, residual, residual)
         else:

@@ -22,6 +22,25 @@ class PreNormBlock(Part):
         for p in self.parts():
             p.prepare(device, dtype)
 
+    # What the block keeps between steps, asked of the block (not of a part inside it): one mixer here, so one need
+    # of each kind; an arrangement with more parts that keep something answers for all of them.
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    def cache_read(self):
+        return self.mixer.cache_read() if hasattr(self.mixer, "cache_read") else None
+
+    def state_need(self):
+        return self.mixer.state_need()
+
+    def kernel_units(self, dtype):
+        """Shared objects beside the core that the parts need (names of kernels.library.units())."""
+        return [u for p in self.parts() if hasattr(p, "kernel_units") for u in p.kernel_units(dtype)]
+
+    def step_arrays(self):
+        """Step arrays that the parts want every step's metadata to carry from the start (engine.context.StepArray)."""
+        return [a for p in self.parts() if hasattr(p, "step_arrays") for a in p.step_arrays()]
+
     def first_norm(self):
         """The norm that reads the residual stream first: the block before may leave its last product to it."""
         return self.mixer_norm

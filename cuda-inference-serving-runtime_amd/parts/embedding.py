@@ -46,4 +46,4 @@ class LMHead(Part):
         logits = ctx.buffer("logits", (n, self.vocab), torch.float32)
         if norm is not None:
             return ops.gemm_normed(residual, (norm.weight, norm.eps, ctx.logit_rows), self.weight, logits)
-        return ops.gemm(h, self.weight, logits, after_norm=True)
+        return ops.gemm(h, self.weight, logits, after_norm=True, scratch=ctx.scratch)

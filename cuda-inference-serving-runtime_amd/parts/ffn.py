@@ -40,15 +40,15 @@ class GatedMLP(FeedForward):
         T = residual.shape[0]
         act = ctx.buffer("ffn.act", (T, self.intermediate), ctx.dtype)
         if self.bias:
-            gate_up = ops.gemm(h, self.w_gate_up, ctx.buffer("ffn.gate_up", (T, 2 * self.intermediate), ctx.dtype))
+            gate_up = ops.gemm(h, self.w_gate_up, ctx.buffer("ffn.gate_up", (T, 2 * self.intermediate), ctx.dtype), scratch=ctx.scratch)
             ops.swiglu(ops.bias_add(gate_up, self.b_gate_up), act)
             return ops.bias_add(ctx.add_product(act, self.w_down, residual), self.b_down)
         if norm is not None:
-            ops.gemm_swiglu(residual, self.w_gate_up, act, norm=(norm.weight, norm.eps, None))
+            ops.gemm_swiglu(residual, self.w_gate_up, act, norm=(norm.weight, norm.eps, None), scratch=ctx.scratch)
         elif ops.swiglu_fused_ok(h, self.w_gate_up):
-            ops.gemm_swiglu(h, self.w_gate_up, act)   # one kernel: product and activation
+            ops.gemm_swiglu(h, self.w_gate_up, act, scratch=ctx.scratch)   # one kernel: product and activation
         else:
-            ops.gemm_swiglu(h, self.w_gate_up, act, scratch=ctx.buffer("ffn.gate_up", (T, 2 * self.intermediate), ctx.dtype))
+            ops.gemm_swiglu(h, self.w_gate_up, act, gate_up=ctx.buffer("ffn.gate_up", (T, 2 * self.intermediate), ctx.dtype), scratch=ctx.scratch)
         return ctx.add_product(act, self.w_down, residual)
 
 

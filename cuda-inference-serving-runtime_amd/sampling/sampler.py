@@ -40,6 +40,7 @@ class Sampler:
 
     def __init__(self):
         self._staging = {}    # device -> [pinned int64 host buffers, device buffer, events, next]
+        self._scratch = ops.ScratchPool()   # the argmax kernel's slice winners
 
     def _params(self, params, device):
         """(temperature, seeds, counters) on the device, through pinned memory so the host does not wait."""
@@ -77,7 +78,7 @@ class Sampler:
         if not keep:
             out = torch.empty(rows, dtype=torch.int32, device=logits.device)
         if all(not (p[0] > 0) for p in params):
-            ops.argmax(logits, out, index)
+            ops.argmax(logits, out, index, scratch=self._scratch)
         else:
             temperature, seeds, counters = self._params(params, logits.device)
             ops.sample(logits, temperature, seeds, counters, out, index)

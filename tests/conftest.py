@@ -61,18 +61,21 @@ def make_weights(c, seed, sharp=True):
     projections are scaled up so that attention scores have a spread of one to
     three units (as in a trained model) instead of near zero, and a wrong key,
     position or page changes the logits; the other matrices are scaled so that
-    the layers' contributions are as large as the embedding."""
+    the layers' contributions are as large as the embedding.  `sharp` may also be the two
+    factors themselves, (queries and keys, the other matrices)."""
     import torch
     rng = np.random.default_rng(seed)
+    qk, rest = (6.0, 4.0) if sharp is True else sharp if sharp else (1.0, 1.0)
+    sharp = bool(sharp)
     out = {}
     for name, shape in sorted(tensor_shapes(c).items()):
         w = rng.standard_normal(size=shape).astype(np.float32) * 0.02
         if name.endswith("norm.weight") or name.endswith("layernorm.weight"):
             w = 1.0 + w
         elif sharp and ("q_proj" in name or "k_proj" in name):
-            w = w * 6.0
+            w = w * qk
         elif sharp and ("v_proj" in name or "o_proj" in name or "mlp" in name):
-            w = w * 4.0
+            w = w * rest
         out[name] = torch.from_numpy(w).to(torch.bfloat16)
     return out
 
@@ -106,6 +109,16 @@ def plain_logits(folder, tokens):
     return _PLAIN[key]
 
 
+def tune_attention(model, **settings):
+    """Give every attention mixer of `model` launch rules that are told `settings` (kernels.attention.AttentionTuning)."""
+    from runtime.kernels.attention import AttentionTuning
+    tuning = AttentionTuning(**settings)
+    for layer in model.layers:
+        if hasattr(getattr(layer, "mixer", None), "tuning"):
+            layer.mixer.tuning = tuning
+    return tuning
+
+
 def random_tokens(seed, n, vocab):
     return np.random.default_rng(seed).integers(0, vocab, size=n).tolist()
 
@@ -119,6 +132,22 @@ F32_TOL = 2e-5
 BF16_RMSE = 0.04
 
 
+ACHIEVED = {}    # (test file, dtype) -> the largest error that a comparison of that file came to
+
+
+def _record(dtype, err):
+    name = os.environ.get("PYTEST_CURRENT_TEST", "?").split("::")[0]
+    ACHIEVED[(name, dtype)] = max(ACHIEVED.get((name, dtype), 0.0), float(err))
+
+
+def pytest_terminal_summary(terminalreporter):
+    """What the comparisons with the plain implementation came to, beside their bounds."""
+    if ACHIEVED:
+        terminalreporter.write_line(f"largest errors against the plain implementation (bounds: float32 {F32_TOL}, bfloat16 rmse {BF16_RMSE})")
+        for (name, dtype), err in sorted(ACHIEVED.items()):
+            terminalreporter.write_line(f"  {name:40s} {dtype:9s} {err:.2e}")
+
+
 def assert_close(got, ref, dtype, what=""):
     got = np.asarray(got, np.float64)
     ref = np.asarray(ref, np.float64)
@@ -126,9 +155,11 @@ def assert_close(got, ref, dtype, what=""):
     assert np.isfinite(got).all(), f"{what}: non-finite logits"
     if dtype == "float32":
         err = np.abs(got - ref).max() / np.abs(ref).max()
+        _record(dtype, err)
         assert err < F32_TOL, f"{what}: float32 differs by {err:.3e} (bound {F32_TOL})"
     else:
         err = np.linalg.norm(got - ref) / np.linalg.norm(ref)
+        _record(dtype, err)
         assert err < BF16_RMSE, f"{what}: bfloat16 relative rmse {err:.3e} (bound {BF16_RMSE})"
         rows = np.linalg.norm(got - ref, axis=-1) / np.linalg.norm(ref, axis=-1)
         assert rows.max() < 3 * BF16_RMSE, f"{what}: bfloat16 worst row {rows.max():.3e}"

@@ -115,7 +115,7 @@ def test_evicted_programs_are_built_again_and_stay_right(folders, name, dtype):
     from conftest import plain_logits, assert_close
     V = TINY[name]["vocab_size"]
     model = load_model(folders[name], dtype=dtype)
-    runner = ModelRunner(model, n_pages=80, page_size=8, max_requests=4, execution="graph")
+    runner = ModelRunner(model, n_pages=80, page_size=8, max_requests=4, execution="graph", program_capacity=16)
     seqs = {k: random_tokens(700 + i, 200, V) for i, k in enumerate("uvw")}
     refs = {k: plain_logits(folders[name], seqs[k]) for k in seqs}
     fed = {}
@@ -159,6 +159,9 @@ def test_evicted_programs_are_built_again_and_stay_right(folders, name, dtype):
                 seen.add(next(reversed(runner.programs)))
             assert len(runner.programs) <= runner.program_capacity
     assert len(seen) > runner.program_capacity, "not enough different shapes to push a program out"
+    report = runner.report()
+    assert report["evictions"] >= len(seen) - 16        # what the step function says of itself: every drop counted
+    assert report["captures"] >= len(seen) and report["replays"] > 0 and report["programs"] <= 16
     assert first_key not in runner.programs, "the first program was never dropped"
     restart()
     feed([("u", 3)]); feed([("v", 2)])
@@ -225,10 +228,9 @@ def test_decoded_tokens_of_mixed_steps_in_a_launch_of_their_own(folders, name, d
     from conftest import plain_logits, assert_close
     V = TINY[name]["vocab_size"]
     model = load_model(folders[name], dtype=dtype)
+    from conftest import tune_attention
+    tune_attention(model, split_single_from=1, rows_launch=launch)
     runner = ModelRunner(model, n_pages=32, page_size=8, max_requests=4, execution=execution)
-    runner.split_single_from = 1
-    if launch:
-        runner._rows_launch = lambda *a: launch
     seen = []
     attend = ops.attention_mfma
     def spy(*a, **kw):
@@ -284,7 +286,7 @@ def test_steps_through_the_wide_product_match_the_plain_model(folders, name, exe
     runner = ModelRunner(model, n_pages=24, page_size=8, max_requests=4, execution=execution)
     calls = []
     wide = ops._gemm_wide
-    monkeypatch.setattr(ops, "_gemm_wide", lambda *a: (calls.append(a[-1]), wide(*a))[1])
+    monkeypatch.setattr(ops, "_gemm_wide", lambda *a: (calls.append(a[5]), wide(*a))[1])   # a[5]: which entry point asked
     seqs = {k: random_tokens(500 + i, 60, V) for i, k in enumerate("xyz")}
     refs = {k: plain_logits(folders[name], seqs[k]) for k in seqs}
     for k in seqs:
@@ -337,7 +339,7 @@ def test_layers_of_real_sizes_match_the_plain_model(tmp_path_factory, sizes, exe
     from conftest import write_folder, plain_logits, assert_close
     left = []
     unfinished = ops.gemm_unfinished
-    monkeypatch.setattr(ops, "gemm_unfinished", lambda *a: (left.append(unfinished(*a)), left[-1])[1])
+    monkeypatch.setattr(ops, "gemm_unfinished", lambda *a, **kw: (left.append(unfinished(*a, **kw)), left[-1])[1])
     cfg = REAL_SIZES[sizes]
     folder = write_folder(tmp_path_factory.mktemp("real") / "m", cfg, 77, sharp=False)
     model = load_model(folder, dtype="bfloat16")
@@ -390,8 +392,9 @@ def test_long_portions_through_block_tiles_match_the_plain_model(folders, name, 
     from conftest import plain_logits, assert_close
     V = TINY[name]["vocab_size"]
     model = load_model(folders[name], dtype="bfloat16")
+    from conftest import tune_attention
+    tune_attention(model, block_tiles=item_tiles, square_tiles=0)
     runner = ModelRunner(model, n_pages=64, page_size=8, max_requests=4)
-    runner.block_tiles = item_tiles
     seqs = {k: random_tokens(500 + i, 230, V) for i, k in enumerate("pq")}
     refs = {k: plain_logits(folders[name], seqs[k]) for k in seqs}
     for k in seqs:
@@ -416,8 +419,9 @@ def test_long_portions_through_square_tiles_match_the_plain_model(folders, name,
     seqs = {k: random_tokens(600 + i, 230, V) for i, k in enumerate("pq")}
     refs = {k: plain_logits(folders[name], seqs[k]) for k in seqs}
     for execution in ("eager", "graph"):
+        from conftest import tune_attention
+        tune_attention(model, square_tiles=square, square_halves=halves)
         runner = ModelRunner(model, n_pages=64, page_size=8, max_requests=4, execution=execution)
-        runner.square_tiles, runner.square_halves = square, halves
         for k in seqs:
             runner.create(k)
         got = runner.step([StepEntry("p", seqs["p"][:150], list(range(150)))]).float().cpu().numpy()

@@ -86,7 +86,7 @@ def test_a_cut_across_the_library_threshold_changes_rounding_only(family_folders
 
 
 @pytest.mark.parametrize("execution", ["eager", "graph"])
-def test_decoding_at_a_context_whose_keys_are_split_over_blocks(family_folders, execution):
+def test_decoding_at_a_context_whose_keys_are_split_over_blocks(family_folders, execution, monkeypatch):
     """From a context of about 550 keys on (more than two 32-key steps a wave), a decode step of few rows splits every row's keys over blocks; at the
     135M sizes the output projection then merges the blocks' partial results itself (no merge kernel).  Three requests
     of very different lengths decode together (the short one's later splits see no key at all), then one alone."""
@@ -102,15 +102,15 @@ def test_decoding_at_a_context_whose_keys_are_split_over_blocks(family_folders, 
         runner.create(k)
         fed[k] = len(toks) - 12
         runner.step([StepEntry(k, toks[:fed[k]], [])])
+    from runtime.kernels import ops
     seen = []
-    real = runner.attention
+    real = ops.gemm_merged
 
-    def spy(*args, **kwargs):
-        out = real(*args, **kwargs)
-        seen.append(None if out is None else out[2])
-        return out
+    def spy(partials, *args, **kwargs):
+        seen.append(partials[2])
+        return real(partials, *args, **kwargs)
 
-    runner.attention = spy
+    monkeypatch.setattr(ops, "gemm_merged", spy)
     for step in range(12):
         live = [k for k in seqs if step < 8 or k == "long"]          # the last four steps: one row
         out = runner.step([StepEntry(k, [seqs[k][fed[k]]], [0]) for k in live]).float().cpu().numpy()

@@ -398,7 +398,26 @@ def run_mfma(ops, qt, kt, vt, tables, rows, page_size, mode, splits=1, window=No
     return f64(out).reshape(T, heads, dim)
 
 
-MFMA_TOL = dict(rtol=2e-2, atol=2e-2)
+MFMA_WORST, MFMA_RMS = 8e-3, 4e-3
+_mfma_seen = {"worst": 0.0, "rms": 0.0}
+
+
+def close_mfma(got, want, err_msg=""):
+    """Matrix-core attention against the float64 reference: the largest difference as a part of the largest output,
+    and the relative root-mean-square difference.  bfloat16 rounds the weights inside the kernel and the outputs
+    at 2^-9 each; what the kernels come to is printed at the end of the module (worst 3.5e-3, rms 2.2e-3 when the bounds were set).
+    One key dropped, doubled or taken from a wrong page among the tens to hundreds of a row moves that row by
+    several hundredths of the largest output."""
+    got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
+    assert got.shape == want.shape and np.isfinite(got).all(), err_msg
+    worst = np.abs(got - want).max() / np.abs(want).max()
+    rms = np.linalg.norm(got - want) / np.linalg.norm(want)
+    _mfma_seen["worst"], _mfma_seen["rms"] = max(_mfma_seen["worst"], worst), max(_mfma_seen["rms"], rms)
+    assert worst < MFMA_WORST and rms < MFMA_RMS, f"{err_msg}: worst {worst:.2e} (bound {MFMA_WORST}), rms {rms:.2e} (bound {MFMA_RMS})"
+
+
+def teardown_module(module):
+    print(f"\nmatrix-core attention against its reference: worst {_mfma_seen['worst']:.2e} of the largest output, rms {_mfma_seen['rms']:.2e}")
 
 
 def square_modes(dim):
@@ -415,17 +434,17 @@ def test_attention_mfma_rows(ops, heads, kv_heads, dim, page_size):
     for splits in (1, 2, 3, 16, 40):
         for waves in (4, 8):
             got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, "rows", splits, waves=waves)
-            np.testing.assert_allclose(got, want, **MFMA_TOL, err_msg=f"splits={splits} waves={waves}")
+            close_mfma(got, want, f"splits={splits} waves={waves}")
     rows2 = list(rows); rows2[0] = (-1, 0)            # a padding row gives zeros
     got = run_mfma(ops, qt, kt, vt, tables, rows2, page_size, "rows", 2)
     assert (got[0] == 0).all()
-    np.testing.assert_allclose(got[1:], want[1:], **MFMA_TOL)
+    close_mfma(got[1:], want[1:])
     again = [run_mfma(ops, qt, kt, vt, tables, rows, page_size, "rows", 16) for _ in range(3)]
     assert all((a == again[0]).all() for a in again)  # the merge order is fixed: repeated runs agree bit for bit
     # a list of rows (the decode rows of a mixed step): only those are computed and written, a negative entry is none
     for splits in (1, 5, 20):
         got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, "rows", splits, waves=8, row_ids=[3, -1, 0, -1])
-        np.testing.assert_allclose(got[[3, 0]], want[[3, 0]], **MFMA_TOL, err_msg=f"listed rows, splits={splits}")
+        close_mfma(got[[3, 0]], want[[3, 0]], f"listed rows, splits={splits}")
         assert (got[[1, 2, 4]] == 9.0).all()
 
 
@@ -440,7 +459,7 @@ def test_attention_mfma_rows_over_many_steps(ops, heads, kv_heads, dim, page_siz
     for splits in (1, 2, 5):
         for waves in (4, 8):
             got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, "rows", splits, waves=waves)
-            np.testing.assert_allclose(got, want, **MFMA_TOL, err_msg=f"splits={splits} waves={waves}")
+            close_mfma(got, want, f"splits={splits} waves={waves}")
     window = 300
     want_w = reference_attention(qt, kt, vt, tables, rows, page_size, window=window)
     t2 = tables.clone()
@@ -449,7 +468,7 @@ def test_attention_mfma_rows_over_many_steps(ops, heads, kv_heads, dim, page_siz
     only = [i for i, (s, p) in enumerate(rows) if not (s == 0 and p + 1 <= window)]       # (its row at 0 needs page 0)
     for splits, waves in ((1, 8), (1, 4), (3, 8)):
         got = run_mfma(ops, qt[only].contiguous(), kt, vt, t2, [rows[i] for i in only], page_size, "rows", splits, waves=waves, window=window)
-        np.testing.assert_allclose(got, want_w[only], **MFMA_TOL, err_msg=f"window, splits={splits} waves={waves}")
+        close_mfma(got, want_w[only], f"window, splits={splits} waves={waves}")
 
 
 def portion_case(heads, kv_heads, dim, page_size, plan, seed):
@@ -471,25 +490,25 @@ def test_attention_mfma_tiles(ops, heads, kv_heads, dim, page_size):
     qt, kt, vt, tables, rows = portion_case(heads, kv_heads, dim, page_size, plan, seed=dim * 3 + heads)
     want = reference_attention(qt, kt, vt, tables, rows, page_size)
     got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, "tiles")
-    np.testing.assert_allclose(got, want, **MFMA_TOL)
+    close_mfma(got, want)
     got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, "tiles", waves=8)
-    np.testing.assert_allclose(got, want, **MFMA_TOL)
+    close_mfma(got, want)
     got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, "tiles", rows_per_tile=1)   # tiles need not be full
-    np.testing.assert_allclose(got, want, **MFMA_TOL)
+    close_mfma(got, want)
     if dim <= 64:
         got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, "tiles2")               # two item tiles a wave
-        np.testing.assert_allclose(got, want, **MFMA_TOL)
+        close_mfma(got, want)
         got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, "tiles2", rows_per_tile=2)
-        np.testing.assert_allclose(got, want, **MFMA_TOL)
+        close_mfma(got, want)
     if dim > 128:                                                                        # block tiles: head sizes up to 128
         with pytest.raises(ops.KernelError):
             run_mfma(ops, qt, kt, vt, tables, rows, page_size, "block")
         return
     for mode in ("block", "block2"):                                                     # 64 / 128-item tiles through LDS
         got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, mode)
-        np.testing.assert_allclose(got, want, **MFMA_TOL, err_msg=mode)
+        close_mfma(got, want, mode)
         got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, mode, rows_per_tile=3)
-        np.testing.assert_allclose(got, want, **MFMA_TOL, err_msg=mode)
+        close_mfma(got, want, mode)
     if page_size < 8:                                                                    # 32 x 32 tiles: pages of at least 8 keys
         with pytest.raises(ops.KernelError):
             run_mfma(ops, qt, kt, vt, tables, rows, page_size, "square")
@@ -500,9 +519,9 @@ def test_attention_mfma_tiles(ops, heads, kv_heads, dim, page_size):
     for mode in square_modes(dim):                                                       # 64 / 128 / 192 / 256 items on the 32 x 32 instruction
         for given in (False, True):
             got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, mode, positions_given=given)
-            np.testing.assert_allclose(got, want, **MFMA_TOL, err_msg=f"{mode} positions given: {given}")
+            close_mfma(got, want, f"{mode} positions given: {given}")
         got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, mode, rows_per_tile=3, positions_given=True)
-        np.testing.assert_allclose(got, want, **MFMA_TOL, err_msg=mode)
+        close_mfma(got, want, mode)
 
 
 @pytest.mark.parametrize("heads, kv_heads, dim, page_size", [(4, 4, 64, 16), (6, 2, 128, 16), (5, 1, 96, 8), (2, 2, 32, 32)])
@@ -523,11 +542,11 @@ def test_attention_square_tiles_over_long_contexts(ops, heads, kv_heads, dim, pa
     for mode in square_modes(dim):
         for rpt in (None, 5):
             got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, mode, rows_per_tile=rpt, positions_given=True)
-            np.testing.assert_allclose(got, want, **MFMA_TOL, err_msg=f"{mode} rows a tile: {rpt}")
+            close_mfma(got, want, f"{mode} rows a tile: {rpt}")
     for window in (40, 257):
         want_w = reference_attention(qt, kt, vt, tables, rows, page_size, window=window)
         got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, "square2", window=window, positions_given=True)
-        np.testing.assert_allclose(got, want_w, **MFMA_TOL, err_msg=f"window {window}")
+        close_mfma(got, want_w, f"window {window}")
 
 
 @pytest.mark.parametrize("dim, page_size", [(64, 16), (128, 16), (32, 8)])
@@ -557,40 +576,40 @@ def test_attention_survives_scores_beyond_the_exponent_range(ops, dim, page_size
     for mode in modes:
         got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, mode, positions_given=mode.startswith("square"))
         assert np.isfinite(got).all(), mode
-        np.testing.assert_allclose(got, want, **MFMA_TOL, err_msg=mode)
+        close_mfma(got, want, mode)
     for splits in (1, 3):
         got = run_mfma(ops, qt, kt, vt, tables, rows, page_size, "rows", splits)
         assert np.isfinite(got).all()
-        np.testing.assert_allclose(got, want, **MFMA_TOL, err_msg=f"rows, splits={splits}")
+        close_mfma(got, want, f"rows, splits={splits}")
 
 
 def test_attention_mfma_window_and_far_key(ops):
     qt, kt, vt, tables, rows = portion_case(4, 2, 32, 8, [(40, 30), (0, 9)], seed=21)
     for window in (1, 8, 9, 33, 64):
         want = reference_attention(qt, kt, vt, tables, rows, 8, window=window)
-        np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables, rows, 8, "tiles", window=window), want, **MFMA_TOL)
-        np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables, rows, 8, "block", window=window), want, **MFMA_TOL)
-        np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables, rows, 8, "block2", window=window), want, **MFMA_TOL)
-        np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables, rows, 8, "tiles2", window=window), want, **MFMA_TOL)
+        close_mfma(run_mfma(ops, qt, kt, vt, tables, rows, 8, "tiles", window=window), want)
+        close_mfma(run_mfma(ops, qt, kt, vt, tables, rows, 8, "block", window=window), want)
+        close_mfma(run_mfma(ops, qt, kt, vt, tables, rows, 8, "block2", window=window), want)
+        close_mfma(run_mfma(ops, qt, kt, vt, tables, rows, 8, "tiles2", window=window), want)
         for mode in square_modes(32):
-            np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables, rows, 8, mode, window=window), want, **MFMA_TOL, err_msg=mode)
-        np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables, rows, 8, "rows", 2, window=window), want, **MFMA_TOL)
+            close_mfma(run_mfma(ops, qt, kt, vt, tables, rows, 8, mode, window=window), want, mode)
+        close_mfma(run_mfma(ops, qt, kt, vt, tables, rows, 8, "rows", 2, window=window), want)
     want = reference_attention(qt, kt, vt, tables, rows, 8, scale=0.3)
-    np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables, rows, 8, "tiles", scale=0.3), want, **MFMA_TOL)
+    close_mfma(run_mfma(ops, qt, kt, vt, tables, rows, 8, "tiles", scale=0.3), want)
     # pages the window has passed are marked -1 in the table and must never be needed
     tables2 = tables.clone(); tables2[0, :4] = -1          # keys 0..31 of request 0; window 8 from position 40 starts at 33
     want = reference_attention(qt, kt, vt, tables, rows, 8, window=8)
-    np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables2, rows, 8, "tiles", window=8), want, **MFMA_TOL)
-    np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables2, rows, 8, "block", window=8), want, **MFMA_TOL)
-    np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables2, rows, 8, "block2", window=8), want, **MFMA_TOL)
-    np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables2, rows, 8, "square", window=8), want, **MFMA_TOL)
-    np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables2, rows, 8, "square2", window=8, positions_given=True), want, **MFMA_TOL)
-    np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables2, rows, 8, "rows", 3, window=8), want, **MFMA_TOL)
+    close_mfma(run_mfma(ops, qt, kt, vt, tables2, rows, 8, "tiles", window=8), want)
+    close_mfma(run_mfma(ops, qt, kt, vt, tables2, rows, 8, "block", window=8), want)
+    close_mfma(run_mfma(ops, qt, kt, vt, tables2, rows, 8, "block2", window=8), want)
+    close_mfma(run_mfma(ops, qt, kt, vt, tables2, rows, 8, "square", window=8), want)
+    close_mfma(run_mfma(ops, qt, kt, vt, tables2, rows, 8, "square2", window=8, positions_given=True), want)
+    close_mfma(run_mfma(ops, qt, kt, vt, tables2, rows, 8, "rows", 3, window=8), want)
     # one far key among hundreds stands out
     qt, kt, vt, tables, rows = paged_case(4, 2, 64, 16, [700, 40], torch.bfloat16, seed=5, sharpen=(0, 3))
     want = reference_attention(qt, kt, vt, tables, rows, 16)
     for mode, splits in (("rows", 1), ("rows", 8), ("tiles", 1), ("block", 1), ("block2", 1), ("square", 1), ("square2", 1)):
-        np.testing.assert_allclose(run_mfma(ops, qt, kt, vt, tables, rows, 16, mode, splits), want, **MFMA_TOL)
+        close_mfma(run_mfma(ops, qt, kt, vt, tables, rows, 16, mode, splits), want)
 
 
 def test_attention_mfma_ignores_what_unseen_slots_hold(ops):
@@ -622,7 +641,7 @@ def test_attention_mfma_ignores_what_unseen_slots_hold(ops):
                              ("square_halves", 1), ("square2_halves", 1), ("rows", 1), ("rows", 3)):
             got = run_mfma(ops, qt, kt, vt, t2, rows, P_, mode, splits, window=window)
             assert np.isfinite(got).all(), f"{mode} window={window}: poison reached the output"
-            np.testing.assert_allclose(got, want[window], **MFMA_TOL, err_msg=f"{mode} window={window}")
+            close_mfma(got, want[window], f"{mode} window={window}")
     # page 0 itself poisoned, with a table whose passed pages read it
     if 0 not in {int(tab[2, j]) for j in range(3, 5)}:
         k0, v0 = kt[0].clone(), vt[0].clone()
@@ -632,21 +651,22 @@ def test_attention_mfma_ignores_what_unseen_slots_hold(ops):
         sub_rows = [rows[i] for i in only]
         got = run_mfma(ops, qt[only].contiguous(), kt, vt, t2, sub_rows, P_, "rows", 2, window=16)
         assert np.isfinite(got).all()
-        np.testing.assert_allclose(got, want[16][only], **MFMA_TOL)
+        close_mfma(got, want[16][only])
         kt[0], vt[0] = k0, v0
 
 
 def test_stream_read_reads_and_writes_nothing(ops):
     """The read-bandwidth probe of the benchmark: any size that is a multiple of 16 bytes, any number of blocks; it
     leaves its sink alone (the folded word never has the value that would be written)."""
+    from runtime import measure
     sink = torch.zeros(4, dtype=torch.int32, device=DEV)
     for nbytes, blocks in ((16, 1), (4096, 3), (1 << 20, 512), (16 * 100003, 7), (48, 256)):
         buf = torch.arange(nbytes, dtype=torch.int64, device=DEV).to(torch.uint8)
-        ops.stream_read(buf, sink, blocks)
+        measure.stream_read(buf, sink, blocks)
     torch.cuda.synchronize()
     assert (sink == 0).all()
     with pytest.raises(ops.KernelError):
-        ops.stream_read(torch.zeros(24, dtype=torch.uint8, device=DEV), sink)
+        measure.stream_read(torch.zeros(24, dtype=torch.uint8, device=DEV), sink)
 
 
 def test_gemm_skinny_and_fused_swiglu(ops):
@@ -678,7 +698,7 @@ def test_gemm_skinny_and_fused_swiglu(ops):
     with pytest.raises(ops.KernelError):
         ops.gemm_swiglu(a, w, torch.empty(70, 90, dtype=torch.bfloat16, device=DEV))
     gq = torch.from_numpy(f64(a) @ f64(w).T).to(torch.bfloat16).double().numpy()
-    two = ops.gemm_swiglu(a, w, torch.empty(70, 90, dtype=torch.bfloat16, device=DEV), scratch=torch.empty(70, 180, dtype=torch.bfloat16, device=DEV))
+    two = ops.gemm_swiglu(a, w, torch.empty(70, 90, dtype=torch.bfloat16, device=DEV), gate_up=torch.empty(70, 180, dtype=torch.bfloat16, device=DEV))
     np.testing.assert_allclose(f64(two), P.swiglu(gq[:, :90], gq[:, 90:]), rtol=2e-2, atol=2e-2)
     # a row's result does not depend on how many rows are beside it: bit for bit among the batches that one kernel
     # takes (up to 16 rows of a narrow output: four columns a block; more: sixteen), to rounding between the two
@@ -1216,9 +1236,10 @@ def test_kernels_refuse_what_they_cannot_take(ops):
 @pytest.mark.gpu
 @pytest.mark.parametrize("blocks,exchange", [(32, 0), (256, 0), (96, 500)])
 def test_grid_meet_counts_every_group_every_round(ops, blocks, exchange):
+    from runtime import measure
     from runtime.kernels.ops import KernelError
     rounds = 50
-    words = ops.grid_meet(blocks, rounds, exchange)
+    words = measure.grid_meet(blocks, rounds, exchange)
     torch.cuda.synchronize()
     assert int(words[-1]) == 0                              # no block gave up waiting
     assert int(words[0]) == rounds * (blocks // 32)         # every group arrived in every round
@@ -1226,7 +1247,7 @@ def test_grid_meet_counts_every_group_every_round(ops, blocks, exchange):
     for g in range(groups):
         assert int(words[16 * (1 + g)]) == rounds * 32
     with pytest.raises(KernelError, match="multiple of 32"):
-        ops.grid_meet(48, 1)
+        measure.grid_meet(48, 1)
 
 
 @pytest.mark.gpu

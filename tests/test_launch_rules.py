@@ -3,14 +3,7 @@ measurements settled them (profiles/prompt_attention_forms_and_the_rule_that_pic
 profiles/decode_attention_launch_shapes_and_the_rule_that_picks.txt), so that a change of a rule shows."""
 import pytest
 
-from runtime.engine.runner import ModelRunner
-
-
-def chooser():
-    runner = ModelRunner.__new__(ModelRunner)          # only the rule is used
-    runner.square_tiles = runner.block_tiles = runner.square_halves = None
-    runner.item_tiles = 2
-    return runner
+from runtime.kernels.attention import fused_merge_splits, prompt_form, rows_launch
 
 
 @pytest.mark.parametrize("heads, kv_heads, dim, rows, form", [
@@ -26,14 +19,13 @@ def chooser():
     (16, 4, 64, 6144, ("square", 2, 1)),      # 768 blocks of 128 items: the halves would crowd the compute units
 ])
 def test_prompt_attention_form_at_measured_points(heads, kv_heads, dim, rows, form):
-    assert tuple(chooser().prompt_attention_form(rows, 1, rows, heads, kv_heads, dim, 16)) == form
+    assert tuple(prompt_form(rows, 1, rows, heads, kv_heads, dim, 16)) == form
 
 
 def test_prompt_attention_form_needs_long_portions_and_pages_of_eight_keys():
-    rule = chooser()
-    assert rule.prompt_attention_form(40, 8, 3000, 9, 3, 64, 16)[0] == "tiles"        # many short portions
-    assert rule.prompt_attention_form(2048, 1, 2048, 9, 3, 64, 4)[0] != "square"      # the copying waves take 8 keys of a page
-    assert rule.prompt_attention_form(2048, 1, 2048, 2, 2, 256, 16)[0] == "tiles"     # heads of more than 128 coordinates
+    assert prompt_form(40, 8, 3000, 9, 3, 64, 16)[0] == "tiles"        # many short portions
+    assert prompt_form(2048, 1, 2048, 9, 3, 64, 4)[0] != "square"      # the copying waves take 8 keys of a page
+    assert prompt_form(2048, 1, 2048, 2, 2, 256, 16)[0] == "tiles"     # heads of more than 128 coordinates
 
 
 @pytest.mark.parametrize("blocks, keys, group, dim, launch", [
@@ -48,4 +40,19 @@ def test_prompt_attention_form_needs_long_portions_and_pages_of_eight_keys():
     (512, 2048, 4, 128, (4, 1)),
 ])
 def test_decode_attention_launch_at_measured_points(blocks, keys, group, dim, launch):
-    assert tuple(ModelRunner._rows_launch(blocks, keys, group, dim)) == launch
+    assert tuple(rows_launch(blocks, keys, group, dim)) == launch
+
+
+@pytest.mark.parametrize("splits, rows, fused", [
+    (8, 8, 8),         # eight requests of the 135M sizes at 2k: the output projection merges all eight
+    (10, 8, 8),        # at 8k the rule asks for ten: eight merged there still beat ten and a merge kernel
+    (8, 16, 4),        # more than 8 rows bring at most four each
+    (4, 16, 4),
+    (32, 1, None),     # one row at 8k to 32k keeps its 32 splits: a quarter of the blocks would cost more than the merge kernel
+    (24, 1, None),
+    (3, 4, 2),
+    (1, 8, None),
+])
+def test_splits_that_the_output_projection_merges_itself(splits, rows, fused):
+    assert fused_merge_splits(splits, rows, lambda n: True) == fused
+    assert fused_merge_splits(splits, rows, lambda n: False) is None

@@ -55,6 +55,22 @@ def test_rope_is_a_complex_rotation_with_split_half_pairing():
     np.testing.assert_allclose(y[..., d // 2:], zr.imag, atol=1e-12)
 
 
+def test_rope_of_one_head_worked_by_hand_from_the_references_kernel():
+    """The reference states the rotation twice, independently: as NumPy (runtime/reference.py:9-15) and as a CUDA
+    kernel that its own tests hold against the former (kernels/ops.cu:21-33, tests/test_cuda.py:28-39).  This is the
+    kernel's arithmetic walked through by hand for one head of four coordinates at position 3 with theta 100:
+    thread d of `half = 2` reads a = x[d], b = x[d + half], turns them by 3 * 100^(-2 d / 4), so the pairs are
+    (0, 2) and (1, 3) and the angles 3 and 0.3.  Neighbouring pairs (0, 1), (2, 3), the angle schedule
+    theta^(-d / dim), or the sine's sign the other way round each change these four numbers.  (The installed
+    `transformers` package is no source for this repository, so its Llama is not imported here; the pairing is that
+    of the reference's two texts.)"""
+    from math import cos, sin
+    x = np.array([[[1.0, 2.0, 3.0, 4.0]]])
+    want = [1 * cos(3.0) - 3 * sin(3.0), 2 * cos(0.3) - 4 * sin(0.3), 3 * cos(3.0) + 1 * sin(3.0), 4 * cos(0.3) + 2 * sin(0.3)]
+    np.testing.assert_allclose(P.rope(x, [3], 100.0)[0, 0], want, rtol=1e-14)
+    np.testing.assert_allclose(want, [-1.4133525208, 0.7285921516, -2.8288574817, 4.4123863698], rtol=1e-9)
+
+
 def test_rope_scores_depend_on_distance_only():
     rng = np.random.default_rng(3)
     q, k = rng.normal(size=(1, 1, 16)), rng.normal(size=(1, 1, 16))

@@ -131,6 +131,68 @@ def test_mixed_requests_reuse_pages(folders, tmp_path, name, dtype, execution):
 
 @pytest.mark.parametrize("execution", EXECUTIONS)
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name, page_size", [("a", 16), ("b", 8), ("c", 16)])
+def test_fork_in_the_middle_of_a_page_then_both_go_on(folders, tmp_path, name, page_size, dtype, execution):
+    """A request is forked where its last page is partly filled (37 tokens); source and copy go on with different
+    tokens, in portions and token by token, beside a third request, in a pool so small that the pages the first
+    fork gave back are taken again; then the copy is forked once more, right after a decoded token.  Whoever
+    writes into the shared page first gets a copy of it; the other must still read what was there."""
+    V = TINY[name]["vocab_size"]
+    stem = random_tokens(21, 37, V)
+    seqs = {"a": stem + random_tokens(22, 60, V), "b": stem + random_tokens(23, 45, V), "c": random_tokens(24, 50, V)}
+    seqs["d"] = seqs["b"][:37 + 20] + random_tokens(25, 30, V)
+    trace = Trace()
+    trace.add([("a", stem, [36])])
+    # the copy writes first (a portion that crosses the page's edge), the source sits this step out
+    trace.add([("b", seqs["b"][37:37 + 13], list(range(13))), ("c", seqs["c"][:9], [8])], fork=[("a", "b")])
+    trace.add([("a", seqs["a"][37:39], [0, 1]), ("b", seqs["b"][50:51], [0]), ("c", seqs["c"][9:30], [20])])
+    at = {"a": 39, "b": 51, "c": 30}
+    for _ in range(6):
+        trace.add([(k, seqs[k][at[k]:at[k] + 1], [0]) for k in "abc"])
+        for k in at:
+            at[k] += 1
+    assert at["b"] == 57
+    # a second fork, from the copy, right after a decoded token; its source ends in the same step
+    trace.add([("d", seqs["d"][57:57 + 11], list(range(11))), ("a", seqs["a"][at["a"]:at["a"] + 17], [16])], fork=[("b", "d")])
+    at["a"] += 17
+    trace.add([("b", seqs["b"][57:], list(range(len(seqs["b"]) - 57))), ("d", seqs["d"][68:70], [1])], end=["b"])
+    trace.add([("a", seqs["a"][at["a"]:], [len(seqs["a"]) - at["a"] - 1]), ("c", seqs["c"][at["c"]:], [len(seqs["c"]) - at["c"] - 1]),
+               ("d", seqs["d"][70:], list(range(len(seqs["d"]) - 70)))], end=["a", "c", "d"])
+    assert all(trace.fed[k] == seqs[k] for k in seqs)
+    runner = run(folders[name], dtype, trace, tmp_path, page_size=page_size, execution=execution)
+    pool = runner.cache.groups[0].pool
+    assert pool.peak < sum(-(-len(s) // page_size) for s in seqs.values()), "the forks shared no page"
+    assert all(free == g.pool.n_pages for free, g in zip(runner.cache.free_pages(), runner.cache.groups))
+    trace.check(folders[name], tmp_path, dtype, V, seqs)
+
+
+@pytest.mark.parametrize("execution", EXECUTIONS)
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_tiny_b_with_pages_of_eight_tokens(folders, tmp_path, dtype, execution):
+    """The second tiny configuration as it is specified: pages of 8 tokens.  Prompts of 1, 9, 33 and 64 tokens cut
+    into portions of 7 beside decoded tokens of the others, then 12 more tokens each."""
+    name = "b"
+    V = TINY[name]["vocab_size"]
+    seqs = {f"r{i}": random_tokens(40 + i, n + 12, V) for i, n in enumerate([1, 9, 33, 64])}
+    prompt = {k: len(v) - 12 for k, v in seqs.items()}
+    trace, at = Trace(), {k: 0 for k in seqs}
+    while any(at[k] < len(seqs[k]) for k in seqs):
+        entries, ending = [], []
+        for k in seqs:
+            if at[k] >= len(seqs[k]):
+                continue
+            n = min(7, prompt[k] - at[k]) if at[k] < prompt[k] else 1
+            entries.append((k, seqs[k][at[k]:at[k] + n], [n - 1]))
+            at[k] += n
+            if at[k] == len(seqs[k]):
+                ending.append(k)
+        trace.add(entries, end=ending)
+    run(folders[name], dtype, trace, tmp_path, page_size=8, execution=execution)
+    trace.check(folders[name], tmp_path, dtype, V, seqs)
+
+
+@pytest.mark.parametrize("execution", EXECUTIONS)
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_long_decoding_and_first_tokens(folders, tmp_path, dtype, execution):
     name = "a"
     V = TINY[name]["vocab_size"]

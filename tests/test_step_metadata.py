@@ -1,7 +1,8 @@
 """Host-side metadata of a step: the attention task lists and the sizes that captured programs pad to."""
 import numpy as np
 
-from runtime.engine.context import fill_tasks
+from runtime.kernels.attention import SingleRows, TileTasks, fill_tasks
+from runtime.engine.context import Batch
 from runtime.engine.runner import _bucket
 
 
@@ -60,3 +61,30 @@ def test_workspace_buffers_are_stable_for_programs_and_bounded_for_other_steps()
     assert bigger.shape == (11, 3) and ws.bytes() == 15 * 3 * 4      # grown by half, the old one dropped
     assert ws.get("y", (2, 5), torch.float32).shape == (2, 5)       # another trailing shape: another buffer
     assert ws.get("z", (7,), torch.int32, zeroed=True).sum() == 0
+
+
+def test_step_arrays_of_the_attention_kernels():
+    """The two lists that the attention kernels ask every step to carry, filled from a batch as the step function does:
+    the rows of the one-token segments of a mixed step (when one of them has a long context), and the tiles of the
+    other segments (which then leave the one-token segments out)."""
+    singles = SingleRows(split_from=100)
+    tiles = TileTasks(4, singles)
+    counts, starts = [1, 6, 1, 3], [150, 0, 20, 7]
+    first_row = np.array([0, 1, 7, 8], dtype=np.int32)
+    batch = Batch(counts, starts, first_row, False, {})
+    assert singles.launch_value(batch) == 2 and tiles.launch_value(batch) is None
+    assert singles.launch_value(Batch([1, 1], [150, 3], None, True, {})) == 0          # a step of single tokens only
+    assert singles.launch_value(Batch([1, 6], [50, 0], None, False, {})) == 0          # short contexts: they stay tiles
+    batch.launch_values[singles] = 4                                                    # (rounded up, as a captured program does)
+    rows = np.full(singles.words(16, 8), 99, dtype=np.int32)
+    singles.fill(rows, batch, 4)
+    assert rows.tolist() == [0, 7, -1, -1, -1, -1, -1, -1]
+    tasks = np.full(tiles.words(16, 8), 99, dtype=np.int32)
+    tiles.fill(tasks, batch, None)
+    tasks = tasks.reshape(-1, 4)
+    real = tasks[tasks[:, 0] >= 0]
+    assert sorted(map(tuple, real[:, :3])) == [(1, 1, 4), (1, 5, 2), (3, 8, 3)]          # no tile for segments 0 and 2
+    assert (tasks[len(real):] == (-1, 0, 0, 0)).all()
+    batch.launch_values[singles] = 0
+    tiles.fill(tasks.reshape(-1), batch, None)
+    assert sorted(tasks[tasks[:, 0] >= 0][:, 0].tolist()) == [0, 1, 1, 2, 3]

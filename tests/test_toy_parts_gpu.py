@@ -152,6 +152,59 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path):
         cleanup()
 
 
+def test_a_step_that_fails_after_a_state_was_written_cannot_be_tried_again(tmp_path):
+    """The toy model updates a per-request state in its first layer; here the last layer of the order raises in the
+    middle of a step.  Lengths and pages go back (the cache manager's part of the promise), but the first layer's
+    state already holds the step's tokens and nothing keeps the old one: the requests of that step are refused from
+    then on instead of being stepped twice over the same tokens, other requests go on, and a released and recreated
+    request starts from a zeroed state and gives the right logits."""
+    import plain_llama as P
+    from runtime.engine import load_model, ModelRunner, StepEntry
+    cleanup = build_toy()
+    try:
+        raw = {"model_type": "toy-decay-lm", "vocab_size": 61, "hidden_size": 24, "decay": 0.7,
+               "max_position_embeddings": 96, "rms_norm_eps": 1e-5}
+        from runtime.engine.loading import build_from_config_dict
+        from runtime.weights import write_model_folder
+        _, _, blueprint = build_from_config_dict(raw)
+        write_model_folder(tmp_path, raw, blueprint.tensor_specs(), seed=3, dtype=torch.float32)
+        cfg, w = P.read_folder(tmp_path)
+        model = load_model(tmp_path, dtype="float32")
+        runner = ModelRunner(model, n_pages=12, page_size=8, max_requests=3)
+        tokens = np.random.default_rng(0).integers(0, 61, 20).tolist()
+        want = plain_toy(raw, w, tokens)
+        runner.create("x"); runner.create("bystander")
+        runner.step([StepEntry("x", tokens[:6], []), StepEntry("bystander", tokens[:3], [])])
+        mixer, calls = model.layers[1].mixer, []
+        real = mixer.forward
+
+        def fails_at_its_second_place(h, residual, ctx, site, **kw):
+            calls.append(site)
+            if len(calls) == 2:
+                raise RuntimeError("injected")
+            return real(h, residual, ctx, site, **kw)
+
+        mixer.forward = fails_at_its_second_place
+        free = runner.cache.free_pages()
+        with pytest.raises(RuntimeError, match="injected"):
+            runner.step([StepEntry("x", tokens[6:15], [8])])
+        mixer.forward = real
+        assert runner.length("x") == 6 and runner.cache.free_pages() == free      # lengths and pages stand where they stood
+        runner.cache.check()
+        with pytest.raises(RuntimeError, match="cannot be stepped again"):
+            runner.step([StepEntry("x", tokens[6:15], [8])])
+        with pytest.raises(ValueError, match="last step"):
+            runner.pick(None, torch.zeros(1, 61, device=DEV), [(0.0, 0, 0)])        # no logits of a step that never ran
+        out = runner.step([StepEntry("bystander", tokens[3:], list(range(17)))]).cpu().numpy()   # others go on
+        np.testing.assert_allclose(out, want[3:], rtol=2e-4, atol=2e-5)
+        runner.release("x"); runner.create("x")
+        out = runner.step([StepEntry("x", tokens, list(range(20)))]).cpu().numpy()
+        np.testing.assert_allclose(out, want, rtol=2e-4, atol=2e-5)
+        runner.cache.check()
+    finally:
+        cleanup()
+
+
 def build_routed_toy():
     """A feed-forward with routing (two experts, the best one scaled by its softmax weight) and a position
     encoding of its own (rotary angles that grow linearly with the pair index), both defined here."""

@@ -18,10 +18,13 @@ class Trace:
     def __init__(self):
         self.steps, self.expect, self.fed, self.peak, self._live = [], {}, {}, 0, {}
 
-    def add(self, entries, end=()):
-        """entries: [(id, tokens, want)]"""
+    def add(self, entries, end=(), fork=()):
+        """entries: [(id, tokens, want)]; fork: [(source, target)], done before the entries run"""
         index = len(self.steps)
         rows = []
+        for source, target in fork:
+            self.fed[target] = list(self.fed[source])
+            self._live[target] = len(self.fed[target])
         for rid, tokens, want in entries:
             start = len(self.fed.setdefault(rid, []))
             self.fed[rid].extend(tokens)
@@ -31,7 +34,7 @@ class Trace:
         for rid in end:
             self._live.pop(rid)
         self.steps.append({"step": index, "entries": [{"id": r, "tokens": list(map(int, t)), "want": list(w)} for r, t, w in entries],
-                           "end": list(end)})
+                           "end": list(end), **({"fork": [list(f) for f in fork]} if fork else {})})
         if rows:
             self.expect[index] = rows
         return index

@@ -63,21 +63,25 @@ def main(argv=None):
         engine = Engine.from_preset(args.model, seed=args.seed, folder=folder, **common)
         raw = read_config_json(folder)
         prompt = [int(t) for t in args.tokens.split(",")]
-    inputs = json.loads(args.requests.read_text()) if args.requests else [
-        {"key": "request-0", "prompt": prompt, "max_new_tokens": args.max_new_tokens}]
-    eos = raw.get("eos_token_id")
-    for index, item in enumerate(inputs):
-        fields = {"eos_token_id": eos, "temperature": args.temperature, "seed": args.seed + index}
-        fields.update(item)
-        engine.submit(Request(**fields))
-    result = []
-    for r in engine.run():
-        result.append({"key": r.key, "status": r.status, "generated": r.generated,
-                       "text": tokenizer.decode(r.generated) if tokenizer else None,
-                       "ttft_ms": None if r.first_token_at is None else (r.first_token_at - r.submitted_at) * 1000})
-    print(json.dumps({"device": "hip", "dtype": args.dtype, "execution": execution,
-                      "weights": "pretrained-local" if args.checkpoint else "random-" + args.model,
-                      "requests": result}, indent=2))
+    if args.requests:
+        workload = json.loads(args.requests.read_text())
+    else:
+        workload = [dict(key="request-0", prompt=prompt, max_new_tokens=args.max_new_tokens)]
+    for index, item in enumerate(workload):
+        # what the file says wins over the defaults: the checkpoint's end-of-sequence id, the command line's sampling
+        engine.submit(Request(**{"eos_token_id": raw.get("eos_token_id"), "temperature": args.temperature,
+                                 "seed": args.seed + index, **item}))
+
+    def outcome(r):
+        waited = None if r.first_token_at is None else 1e3 * (r.first_token_at - r.submitted_at)
+        return dict(key=r.key, status=r.status, generated=r.generated,
+                    text=None if tokenizer is None else tokenizer.decode(r.generated), ttft_ms=waited)
+
+    # the reference's report (runtime/__main__.py:43-50): one object, the requests in the order they were submitted
+    report = dict(device="hip", dtype=args.dtype, execution=execution,
+                  weights=f"random-{args.model}" if not args.checkpoint else "pretrained-local",
+                  requests=[outcome(r) for r in engine.run()])
+    print(json.dumps(report, indent=2))
     return 0
 
 

@@ -209,20 +209,25 @@ class Engine:
 
     # -- one tick = one step --------------------------------------------------------
     def plan(self):
-        """[(request, n_tokens)] for the next step under the budget; advances the rotation."""
-        order = self.active[self.rotation:] + self.active[:self.rotation]
-        self.rotation = (self.rotation + 1) % max(1, len(self.active))
+        """[(request, n_tokens)] for the next step under the budget; advances the rotation.  The request that is
+        served first moves on by one place every tick, so that a budget smaller than the batch starves nobody
+        (the reference's rotating priority, runtime/engine.py:82-85); `decode_first` then lets every decoding
+        request, in that order, stand before every prompt."""
+        live = [r for r in self.active if r.status is not Phase.DRAINING]
+        first = self.rotation % len(self.active) if self.active else 0
+        turn = {id(r): (i - first) % len(self.active) for i, r in enumerate(self.active)}
+        self.rotation = first + 1
         if self.policy == "decode_first":
-            order.sort(key=lambda r: r.status is not Phase.DECODE)
-        remaining, plan = self.token_budget, []
-        for r in order:
-            if remaining == 0:
+            live.sort(key=lambda r: (r.status is not Phase.DECODE, turn[id(r)]))
+        else:
+            live.sort(key=lambda r: turn[id(r)])
+        plan, left = [], self.token_budget
+        for r in live:
+            if left <= 0:
                 break
-            if r.status is Phase.DRAINING:
-                continue
-            n = 1 if r.status is Phase.DECODE else min(self.prefill_chunk, len(r.prompt) - r.cursor, remaining)
+            n = 1 if r.status is Phase.DECODE else min(self.prefill_chunk, len(r.prompt) - r.cursor, left)
             plan.append((r, n))
-            remaining -= n
+            left -= n
         return plan
 
     def _entries(self, plan):
@@ -306,13 +311,15 @@ class Engine:
                 self._close(r)
 
     def run(self):
-        """Tick until every request is over; sleeps (at most 10 ms at a time) while only future arrivals wait."""
-        while self.tick():
-            if not self.active and self.waiting:
-                pause = min(r.submitted_at for r in self.waiting) - time.perf_counter()
-                if pause > 0:
-                    time.sleep(min(pause, 0.01))
-        return list(self.requests.values())
+        """Tick until every request is over.  While nothing is live and the next arrival lies in the future the
+        loop sleeps, never longer than 10 ms at a time (the reference's idle wait, runtime/engine.py:117-122)."""
+        busy = True
+        while busy:
+            busy = self.tick()
+            if busy and not self.active and self.waiting:
+                until_next = min(r.submitted_at for r in self.waiting) - time.perf_counter()
+                time.sleep(max(0.0, min(until_next, 0.01)))
+        return [self.requests[key] for key in self.requests]
 
     # -- conveniences ---------------------------------------------------------------
     @classmethod

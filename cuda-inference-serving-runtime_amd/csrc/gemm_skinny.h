@@ -40,3 +40,9 @@ int cisr_narrow_launch_t4(const SkinnyArgs& a, int units, bool norm, int epi, in
 int cisr_narrow_merge_launch_t1(const SkinnyArgs& a, int units, int splits, hipStream_t stream);
 int cisr_narrow_merge_launch_t2(const SkinnyArgs& a, int units, int splits, hipStream_t stream);
 int cisr_narrow_merge_launch_t4(const SkinnyArgs& a, int units, int splits, hipStream_t stream);
+
+// The matrix-vector kernel (gemv.hip): at most GEMV_MAX_ROWS rows of A, whole rows of W a wave.  `units`: N, or with
+// EPI_ROPE the rotary pairs (heads + 2 kv_heads) head_dim / 2; `splits` > 0 selects the merge prologue (2, 4, 8).
+#define GEMV_MAX_ROWS 8
+bool cisr_gemv_takes(int M, int K);
+int cisr_gemv_launch(const SkinnyArgs& a, int units, bool norm, int epi, int out_dtype, int splits, hipStream_t stream);

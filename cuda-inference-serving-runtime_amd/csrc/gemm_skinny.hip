@@ -1,7 +1,6 @@
 // Entry points of the skinny (M <= 64) bf16 matrix products; the kernels live in gemm_skinny.inc,
 // compiled once per number of 16-row tiles (gemm_skinny_m1..m4.hip).
 #include "gemm_skinny.h"
-#include <stdlib.h>
 
 // More than 16 rows of A: the kernels take up to 64 rows a block (MT tiles of 16), but a narrow output then has few
 // blocks, each with all rows' partial tiles to add up.  Such a product runs as groups of 16 MT rows instead (a block
@@ -21,16 +20,20 @@ static int launch_rows(const SkinnyArgs& a, int blocks, bool norm, int epi, int 
 
 static bool aligned16(const void* p) { return ((uintptr_t)p) % 16 == 0; }
 
+// Very few rows: the matrix-vector kernel (gemv.hip), whatever the size of the weights.  The most rows it is given
+// can be set (cisr_gemv_set_rows: 0 switches it off), for measurements of one kernel against the other.
+static int gemv_rows = GEMV_MAX_ROWS;
+extern "C" void cisr_gemv_set_rows(int rows) { gemv_rows = rows < 0 ? 0 : rows > GEMV_MAX_ROWS ? GEMV_MAX_ROWS : rows; }
+extern "C" int cisr_gemv_ok(int M, int K) { return M <= gemv_rows && cisr_gemv_takes(M, K); }
+
 // Few rows against small weights with a narrow output: a block for every 16 columns would leave most compute
 // units idle, so the narrow kernels take over (a block for every 4 columns).  Measured on an MI355X in captured
 // chains: the down projection of the 135M sizes (8 rows, 576 x 1536) 4.3 us with 36 blocks of 16 columns.
-// CISR_NARROW=0 switches them off.
 static bool narrow_wanted(int M, int N, int K, bool norm) {
-    static const int enabled = getenv("CISR_NARROW") ? atoi(getenv("CISR_NARROW")) : 1;
     const int rows = M <= 4 ? 4 : M <= 8 ? 8 : 16;
     // with the norm fused, a block's rows must fit LDS and be one batch of loads: inner sizes up to 1024, 640, 576
     if (norm && ((size_t)rows * (K + 8) * 2 > 40 * 1024 || K > (rows == 4 ? 1024 : rows == 8 ? 640 : 576))) return false;
-    return enabled && M <= 16 && (N + 15) / 16 < 256 && (long long)N * K * 2 <= (4LL << 20);
+    return M <= 16 && (N + 15) / 16 < 256 && (long long)N * K * 2 <= (4LL << 20);
 }
 
 static int launch_narrow(const SkinnyArgs& a, int units, bool norm, int epi, int out_dtype, hipStream_t stream) {
@@ -52,6 +55,7 @@ extern "C" int cisr_gemm_skinny_bf16(const void* A, int lda, const void* W, int 
     a.A = A; a.lda = lda; a.W = (const bf16_t*)W; a.ldw = ldw; a.C = C; a.ldc = ldc; a.R = R; a.ldr = ldr;
     a.M = M; a.N = N; a.K = K; a.dual_off = dual_off; a.norm_w = norm_w; a.eps = eps; a.rows = rows;
     const int epi = dual_off > 0 ? EPI_SWIGLU : EPI_STORE;
+    if (cisr_gemv_ok(M, K)) return cisr_gemv_launch(a, N, norm_w != nullptr, epi, out_dtype, 0, stream);
     if (narrow_wanted(M, dual_off > 0 ? 2 * N : N, K, norm_w != nullptr)) return launch_narrow(a, (N + 3) / 4, norm_w != nullptr, epi, out_dtype, stream);
     const int blocks = (N + 15) / 16;
     return launch_rows(a, blocks, norm_w != nullptr, epi, out_dtype, stream);
@@ -74,6 +78,7 @@ extern "C" int cisr_qkv_rope_skinny(const void* A, int lda, const void* W, int l
     a.positions = positions; a.slots = slots; a.cos_tab = cos_tab; a.sin_tab = sin_tab;
     a.kcache = (bf16_t*)kcache; a.vcache = (bf16_t*)vcache; a.heads = heads; a.kv_heads = kv_heads;
     a.head_dim = head_dim; a.page_size = page_size; a.max_pos = max_pos;
+    if (cisr_gemv_ok(M, K)) return cisr_gemv_launch(a, a.N / 2, norm_w != nullptr, EPI_ROPE, DT_BF16, 0, stream);
     if (narrow_wanted(M, a.N, K, norm_w != nullptr)) return launch_narrow(a, a.N / 4, norm_w != nullptr, EPI_ROPE, DT_BF16, stream);
     const int blocks = (heads + 2 * kv_heads) * (head_dim / 16);
     return launch_rows(a, blocks, norm_w != nullptr, EPI_ROPE, DT_BF16, stream);
@@ -85,6 +90,7 @@ extern "C" int cisr_qkv_rope_skinny(const void* A, int lda, const void* W, int l
 extern "C" int cisr_gemm_merged_ok(int M, int N, int heads, int head_dim, int splits) {
     const int K = heads * head_dim, rows = M <= 4 ? 4 : M <= 8 ? 8 : 16;
     const int batches = rows == 4 ? 2 : rows == 8 ? 3 : 5;
+    if (M >= 1 && head_dim % 8 == 0 && (splits == 2 || splits == 4 || splits == 8) && cisr_gemv_ok(M, K)) return 1;
     return M >= 1 && M <= 16 && head_dim % 8 == 0 && (splits == 2 || splits == 4 || splits == 8) &&
            narrow_wanted(M, N, K, false) && (size_t)rows * (K + 8) * 2 <= 40 * 1024 && M * (K / 8) <= batches * 256;
 }
@@ -99,6 +105,7 @@ extern "C" int cisr_gemm_merged_bf16(const void* part_o, const float* part_ml, i
     SkinnyArgs a = {};
     a.W = (const bf16_t*)W; a.ldw = ldw; a.C = C; a.ldc = ldc; a.R = R; a.ldr = ldr; a.M = M; a.N = N; a.K = K;
     a.part_o = (const bf16_t*)part_o; a.part_ml = part_ml; a.merge_heads = heads; a.merge_dim = head_dim;
+    if (cisr_gemv_ok(M, K)) return cisr_gemv_launch(a, N, false, EPI_STORE, DT_F32, splits, stream);
     const int units = (N + 3) / 4;
     if (M <= 4) return cisr_narrow_merge_launch_t1(a, units, splits, stream);
     if (M <= 8) return cisr_narrow_merge_launch_t2(a, units, splits, stream);

@@ -1,0 +1,330 @@
+// Products of very few rows (M <= 8):  C[M,N] = A[M,K] . W[N,K]^T  as a matrix-vector kernel.
+//
+// With one to eight rows of A a product is a stream of W and nothing else: every byte of W is used M times and the
+// matrix cores have nothing to win.  What counts is how soon the first byte of W is asked for and how many are in
+// flight.  So: a wave owns whole rows of W (one or two at a time: a unit), its lanes take the 16-byte chunks of a row
+// in turn (chunk c to lane c mod 64), the products are packed-bf16 dot instructions with float sums (v_dot2_f32_bf16),
+// the lanes' sums meet in a butterfly of lane exchanges, and a lane finishes each activation row.  No partial tiles
+// in LDS, no barrier after the prologue, no second kernel; the first loads of W are issued before the prologue's
+// barrier, because they do not depend on the activations.
+//
+// Prologue, once a block (256 threads), into LDS as packed bf16 rows [M][K]:
+//   plain   A is bf16: copied;
+//   NORM    A is the float residual: bf16(x[m,k] * w_norm[k]), and the row's sum of squares; rsqrt(mean + eps) is
+//           applied to the finished sums (a per-row factor commutes with the product); `rows` picks input rows;
+//   MSPL    A is the output of decode attention whose keys were split over MSPL blocks, merged here
+//           (out = sum_s w_s o_s / sum_s w_s, w_s = 2^(m_s - max m) l_s), as in gemm_narrow.inc.
+// Epilogues as in gemm_skinny.inc: store / residual; SwiGLU (a unit is the gate row and the up row of one output);
+// rotary embedding and cache write of the fused q/k/v projection (a unit is the rotary pair (i, i + D/2) of a head).
+//
+// A row's result does not depend on the other rows of the step: a lane's chunks, the order of its sums and the
+// butterfly's order are fixed by K alone.
+// Requires K % 8 == 0 and 16-byte aligned rows; M * K * 2 bytes of LDS.
+#include "gemm_skinny.h"
+
+typedef __attribute__((ext_vector_type(2))) __bf16 gv_bf16x2;
+typedef __attribute__((ext_vector_type(4))) float gv_f32x4;
+typedef __attribute__((ext_vector_type(4))) uint32_t gv_u32x4;
+
+#define GEMV_THREADS 256
+#define GEMV_WAVES 4
+#define GEMV_CB 4                 // chunks of a row that a lane has in flight per batch (and as many of the batch after)
+#define GEMV_MAX_LDS (144 * 1024)
+
+__device__ __forceinline__ float gv_dot2(uint32_t w, uint32_t a, float acc) {
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(gv_bf16x2, w), __builtin_bit_cast(gv_bf16x2, a), acc, false);
+}
+// (the words are taken out of the vectors first: a bit cast of a vector's component reads its first component)
+__device__ __forceinline__ float gv_dot8(gv_u32x4 w, gv_u32x4 a, float acc) {
+    const uint32_t w0 = w[0], w1 = w[1], w2 = w[2], w3 = w[3], a0 = a[0], a1 = a[1], a2 = a[2], a3 = a[3];
+    return gv_dot2(w3, a3, gv_dot2(w2, a2, gv_dot2(w1, a1, gv_dot2(w0, a0, acc))));
+}
+
+// M: rows of A the kernel has room for (1, 2, 4, 8); R rows of W a unit (1: store, 2: SwiGLU and rotary pairs)
+template <int M, bool NORM, int EPI, typename TC, int MSPL>
+__global__ void __launch_bounds__(GEMV_THREADS)
+gemv_kernel(SkinnyArgs p, int units, int per_wave) {
+    static_assert(MSPL == 0 || (!NORM && EPI == EPI_STORE), "the merge prologue feeds the output projection");
+    constexpr int R = EPI == EPI_STORE ? 1 : 2;
+    constexpr int CB = GEMV_CB;
+    extern __shared__ __attribute__((aligned(16))) uint32_t a_lds[];      // [M][K / 2]: packed bf16 pairs
+    __shared__ float ssq_s[M][GEMV_WAVES];
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / WAVE), lane = tid % WAVE;
+    const int K = p.K, nchunks = K / 8, words = K / 2;
+    const int iters = (nchunks + WAVE - 1) / WAVE;                         // chunks a lane takes of one row
+    const int total_waves = gridDim.x * GEMV_WAVES, wave_global = blockIdx.x * GEMV_WAVES + wave;
+
+    // the rows of W of unit u
+    auto rows_of = [&](int u, int& r0, int& r1) {
+        if (EPI == EPI_ROPE) {
+            const int half = p.head_dim / 2, sh = u / half, i = u % half;
+            r0 = sh * p.head_dim + i; r1 = r0 + half;
+        } else {
+            r0 = u; r1 = u + p.dual_off;
+        }
+    };
+    // the wave's j-th unit (units are dealt to the waves in turn) and its batch b of chunks, all loads at once; a chunk past
+    // the row reads the row's first again (no branch around a load) and counts as zero
+    auto unit_of = [&](int j) { return wave_global + j * total_waves; };
+    auto load_batch = [&](int u, int b, gv_u32x4 (&w)[R][CB]) {
+        int r0, r1;
+        rows_of(u < units ? u : 0, r0, r1);
+        const bf16_t* w0 = p.W + (size_t)r0 * p.ldw;
+        const bf16_t* w1 = p.W + (size_t)r1 * p.ldw;
+#pragma unroll
+        for (int c = 0; c < CB; ++c) {
+            const int chunk = lane + WAVE * (b * CB + c), at = chunk < nchunks ? chunk * 8 : 0;
+            w[0][c] = *(const gv_u32x4*)(w0 + at);
+            if (R == 2) w[1][c] = *(const gv_u32x4*)(w1 + at);
+        }
+    };
+    gv_u32x4 wcur[R][CB];
+    load_batch(unit_of(0), 0, wcur);                  // on its way while the activations are prepared
+
+    // ---- prologue: the activation rows as packed bf16 in LDS
+    if constexpr (NORM) {
+        const int words4 = K / 4;
+#pragma unroll
+        for (int m = 0; m < M; ++m) {
+            float sq = 0.f;
+            if (m < p.M) {
+                const int src = p.rows ? p.rows[m] : m;
+                const float* x = (const float*)p.A + (size_t)src * p.lda;
+#pragma unroll 4
+                for (int k4 = tid; k4 < words4; k4 += GEMV_THREADS) {
+                    const gv_f32x4 xv = *(const gv_f32x4*)(x + k4 * 4), nv = *(const gv_f32x4*)(p.norm_w + k4 * 4);
+                    sq += xv.x * xv.x + xv.y * xv.y + xv.z * xv.z + xv.w * xv.w;
+                    a_lds[m * words + k4 * 2] = pack_bf16x2(xv.x * nv.x, xv.y * nv.y);
+                    a_lds[m * words + k4 * 2 + 1] = pack_bf16x2(xv.z * nv.z, xv.w * nv.w);
+                }
+            } else {
+                for (int k4 = tid; k4 < words4; k4 += GEMV_THREADS) { a_lds[m * words + k4 * 2] = 0u; a_lds[m * words + k4 * 2 + 1] = 0u; }
+            }
+            sq = wave_sum(sq);
+            if (lane == 0) ssq_s[m][wave] = sq;
+        }
+    } else if constexpr (MSPL > 0) {
+        const int per_row = K / 8, n_items = M * per_row;
+        const int D = p.merge_dim, nh = p.merge_heads;
+        for (int item = tid; item < n_items; item += GEMV_THREADS) {
+            const int row = item / per_row, k = (item % per_row) * 8;
+            gv_u32x4 out = {0u, 0u, 0u, 0u};
+            if (row < p.M) {
+                const size_t base = ((size_t)row * nh + k / D) * MSPL;
+                gv_u32x4 po[MSPL];
+                float ms[MSPL], ls[MSPL];
+#pragma unroll
+                for (int sp = 0; sp < MSPL; ++sp) {
+                    po[sp] = *(const gv_u32x4*)(p.part_o + (base + sp) * D + k % D);
+                    ms[sp] = p.part_ml[(base + sp) * 2]; ls[sp] = p.part_ml[(base + sp) * 2 + 1];
+                }
+                float mx = -INFINITY;
+#pragma unroll
+                for (int sp = 0; sp < MSPL; ++sp) mx = fmaxf(mx, ms[sp]);
+                float den = 0.f, num[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) num[j] = 0.f;
+#pragma unroll
+                for (int sp = 0; sp < MSPL; ++sp) {       // in the order of the splits
+                    const float w = ls[sp] > 0.f ? __builtin_amdgcn_exp2f(ms[sp] - mx) * ls[sp] : 0.f;
+                    den += w;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        num[2 * j] += w * __uint_as_float(po[sp][j] << 16);
+                        num[2 * j + 1] += w * __uint_as_float(po[sp][j] & 0xffff0000u);
+                    }
+                }
+                const float inv = den > 0.f ? 1.0f / den : 0.f;
+                out = (gv_u32x4){pack_bf16x2(num[0] * inv, num[1] * inv), pack_bf16x2(num[2] * inv, num[3] * inv),
+                                 pack_bf16x2(num[4] * inv, num[5] * inv), pack_bf16x2(num[6] * inv, num[7] * inv)};
+            }
+            *(gv_u32x4*)(a_lds + row * words + k / 2) = out;
+        }
+    } else {
+        const int n_items = M * nchunks;
+        for (int item = tid; item < n_items; item += GEMV_THREADS) {
+            const int row = item / nchunks, c = item % nchunks;
+            gv_u32x4 v = {0u, 0u, 0u, 0u};
+            if (row < p.M) v = *(const gv_u32x4*)((const bf16_t*)p.A + (size_t)row * p.lda + c * 8);
+            *(gv_u32x4*)(a_lds + row * words + c * 4) = v;
+        }
+    }
+    __syncthreads();
+
+    // the lane that finishes activation row `my_m` of every unit (see the butterfly below), and what it needs from
+    // memory that does not depend on the unit
+    constexpr int NV = M * R;                         // sums a lane holds for one unit: [m][r]
+    int my_m = 0;
+    {
+        int nv = NV, off = 32;
+        while (nv > R) { nv /= 2; if (lane & off) my_m += nv / R; off >>= 1; }
+    }
+    const bool finisher = (lane & ((64 / M) - 1)) == 0 && my_m < p.M;      // one lane for every activation row
+    float scale = 1.f;
+    if (NORM) scale = 1.0f / sqrtf((((ssq_s[my_m][0] + ssq_s[my_m][1]) + ssq_s[my_m][2]) + ssq_s[my_m][3]) / (float)K + p.eps);
+    int pos = 0, slot = -1;
+    if (EPI == EPI_ROPE && finisher) {
+        pos = p.positions[my_m];
+        pos = pos < 0 ? 0 : (pos >= p.max_pos ? p.max_pos - 1 : pos);
+        if (p.slots) slot = p.slots[my_m];
+    }
+
+    for (int j = 0; j < per_wave; ++j) {
+        const int u = unit_of(j);
+        if (u >= units) break;                        // (uniform over the wave)
+        int r0, r1;
+        rows_of(u, r0, r1);
+        // what the finishing lanes need of this unit, asked for before the products
+        float resid = 0.f, rot_cos = 1.f, rot_sin = 0.f;
+        if (EPI == EPI_STORE && p.R && finisher) resid = p.R[(size_t)my_m * p.ldr + u];
+        if (EPI == EPI_ROPE && finisher) {
+            const int half = p.head_dim / 2;
+            rot_cos = p.cos_tab[(size_t)pos * half + u % half];
+            rot_sin = p.sin_tab[(size_t)pos * half + u % half];
+        }
+        float acc[M][R];
+#pragma unroll
+        for (int m = 0; m < M; ++m)
+#pragma unroll
+            for (int r = 0; r < R; ++r) acc[m][r] = 0.f;
+        const int batches = (iters + CB - 1) / CB;
+        for (int b = 0; b < batches; ++b) {
+            // the batch after this one (or the first of the wave's next unit) is asked for before this one is used
+            gv_u32x4 wnext[R][CB];
+            const bool more = b + 1 < batches;
+            load_batch(more ? u : unit_of(j + 1), more ? b + 1 : 0, wnext);
+#pragma unroll
+            for (int c = 0; c < CB; ++c) {
+                const int chunk = lane + WAVE * (b * CB + c);
+                const bool ok = chunk < nchunks;
+                const int at = ok ? chunk * 4 : 0;
+                const uint32_t keep = ok ? 0xffffffffu : 0u;
+                gv_u32x4 w0 = wcur[0][c], w1 = wcur[R - 1][c];
+                w0.x &= keep; w0.y &= keep; w0.z &= keep; w0.w &= keep;
+                if (R == 2) { w1.x &= keep; w1.y &= keep; w1.z &= keep; w1.w &= keep; }
+#pragma unroll
+                for (int m = 0; m < M; ++m) {
+                    const gv_u32x4 a = *(const gv_u32x4*)(a_lds + m * words + at);
+                    acc[m][0] = gv_dot8(w0, a, acc[m][0]);
+                    if (R == 2) acc[m][R - 1] = gv_dot8(w1, a, acc[m][R - 1]);
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+#pragma unroll
+                for (int c = 0; c < CB; ++c) wcur[r][c] = wnext[r][c];
+        }
+        // The lanes' sums meet: offsets 32, 16, 8, ... in this order whatever M is.  While a lane holds the sums of more
+        // than one activation row, the two lanes of a pair share them out (the upper lane keeps the upper half and
+        // sends the lower), so that a row's sums end in the lanes that finish it; then plain exchanges.
+        float v[NV];
+#pragma unroll
+        for (int m = 0; m < M; ++m)
+#pragma unroll
+            for (int r = 0; r < R; ++r) v[m * R + r] = acc[m][r];
+        {
+            int off = 32;
+#pragma unroll
+            for (int nv = NV; nv > R; nv /= 2) {
+                const bool upper = (lane & off) != 0;
+#pragma unroll
+                for (int i = 0; i < nv / 2; ++i) {
+                    const float send = upper ? v[i] : v[i + nv / 2], keepv = upper ? v[i + nv / 2] : v[i];
+                    v[i] = keepv + __shfl_xor(send, off, WAVE);
+                }
+                off >>= 1;
+            }
+#pragma unroll
+            for (; off > 0; off >>= 1)
+#pragma unroll
+                for (int r = 0; r < R; ++r) v[r] += __shfl_xor(v[r], off, WAVE);
+        }
+        if (!finisher) continue;
+        const int m = my_m;
+        float v0 = v[0] * scale;
+        if (EPI == EPI_STORE) {
+            if (p.R) v0 += resid;
+            store_f32((TC*)p.C + (size_t)m * p.ldc + u, v0);
+        } else if (EPI == EPI_SWIGLU) {
+            const float v1 = v[R - 1] * scale;
+            // the two-kernel path rounds gate and up to bf16 before the activation; do the same
+            const float gq = bf16_to_f32(f32_to_bf16(v0)), uq = bf16_to_f32(f32_to_bf16(v1));
+            ((bf16_t*)p.C)[(size_t)m * p.ldc + u] = f32_to_bf16(gq / (1.0f + expf(-gq)) * uq);
+        } else {
+            float v1 = v[R - 1] * scale;
+            const int D = p.head_dim, half = D / 2, sh = u / half, i = u % half;
+            if (sh < p.heads + p.kv_heads) {          // q or k head: turn the pair
+                const float a = v0, b = v1;
+                v0 = a * rot_cos - b * rot_sin; v1 = b * rot_cos + a * rot_sin;
+            }
+            if (sh < p.heads) {
+                bf16_t* q = (bf16_t*)p.C + (size_t)m * p.ldc + sh * D;
+                q[i] = f32_to_bf16(v0); q[half + i] = f32_to_bf16(v1);
+            } else if (slot >= 0) {
+                const int page = slot / p.page_size, off = slot % p.page_size;
+                if (sh < p.heads + p.kv_heads) {
+                    bf16_t* k = p.kcache + (((size_t)page * p.kv_heads + (sh - p.heads)) * p.page_size + off) * D;
+                    k[i] = f32_to_bf16(v0); k[half + i] = f32_to_bf16(v1);
+                } else {
+                    bf16_t* vv = p.vcache + ((size_t)page * p.kv_heads + (sh - p.heads - p.kv_heads)) * D * p.page_size + off;
+                    vv[(size_t)i * p.page_size] = f32_to_bf16(v0); vv[(size_t)(half + i) * p.page_size] = f32_to_bf16(v1);
+                }
+            }
+        }
+    }
+}
+
+static int gemv_compute_units() {
+    static int units = 0;
+    if (units == 0) {
+        int device = 0;
+        if (hipGetDevice(&device) != hipSuccess || hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || units <= 0)
+            units = 256;
+    }
+    return units;
+}
+
+template <int M, bool NORM, int EPI, typename TC, int MSPL>
+static int gemv_launch_one(const SkinnyArgs& a, int units, hipStream_t stream) {
+    const size_t lds = (size_t)M * a.K * 2;
+    if (lds > GEMV_MAX_LDS) return (int)hipErrorInvalidValue;
+    if (lds > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute((const void*)gemv_kernel<M, NORM, EPI, TC, MSPL>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return (int)e;
+    }
+    // units a wave: as few as give every compute unit eight waves (two blocks) of work, so that a short product is one round
+    const int waves = gemv_compute_units() * 8;
+    const int per_wave = (units + waves - 1) / waves;
+    const int blocks = (units + GEMV_WAVES * per_wave - 1) / (GEMV_WAVES * per_wave);
+    gemv_kernel<M, NORM, EPI, TC, MSPL><<<blocks, GEMV_THREADS, lds, stream>>>(a, units, per_wave);
+    return CISR_LAUNCH_CHECK();
+}
+
+template <int M>
+static int gemv_launch_rows(const SkinnyArgs& a, int units, bool norm, int epi, int out_dtype, int splits, hipStream_t stream) {
+    if (splits == 2) return gemv_launch_one<M, false, EPI_STORE, float, 2>(a, units, stream);
+    if (splits == 4) return gemv_launch_one<M, false, EPI_STORE, float, 4>(a, units, stream);
+    if (splits == 8) return gemv_launch_one<M, false, EPI_STORE, float, 8>(a, units, stream);
+    if (splits != 0) return (int)hipErrorInvalidValue;
+    if (epi == EPI_SWIGLU) return norm ? gemv_launch_one<M, true, EPI_SWIGLU, bf16_t, 0>(a, units, stream) : gemv_launch_one<M, false, EPI_SWIGLU, bf16_t, 0>(a, units, stream);
+    if (epi == EPI_ROPE) return norm ? gemv_launch_one<M, true, EPI_ROPE, bf16_t, 0>(a, units, stream) : gemv_launch_one<M, false, EPI_ROPE, bf16_t, 0>(a, units, stream);
+    if (out_dtype == DT_F32) return norm ? gemv_launch_one<M, true, EPI_STORE, float, 0>(a, units, stream) : gemv_launch_one<M, false, EPI_STORE, float, 0>(a, units, stream);
+    return norm ? gemv_launch_one<M, true, EPI_STORE, bf16_t, 0>(a, units, stream) : gemv_launch_one<M, false, EPI_STORE, bf16_t, 0>(a, units, stream);
+}
+
+// Whether the matrix-vector kernel takes M rows against an inner size of K: the rows must fit LDS.
+bool cisr_gemv_takes(int M, int K) {
+    if (M < 1 || M > GEMV_MAX_ROWS || K <= 0 || K % 8) return false;
+    const int room = M <= 1 ? 1 : M <= 2 ? 2 : M <= 4 ? 4 : 8;
+    return (size_t)room * K * 2 <= GEMV_MAX_LDS;
+}
+
+// `units`: N for the plain and SwiGLU forms (N outputs), (heads + 2 kv_heads) head_dim / 2 rotary pairs for EPI_ROPE.
+// `splits` > 0: the merge prologue.
+int cisr_gemv_launch(const SkinnyArgs& a, int units, bool norm, int epi, int out_dtype, int splits, hipStream_t stream) {
+    if (!cisr_gemv_takes(a.M, a.K)) return (int)hipErrorInvalidValue;
+    if (a.M <= 1) return gemv_launch_rows<1>(a, units, norm, epi, out_dtype, splits, stream);
+    if (a.M <= 2) return gemv_launch_rows<2>(a, units, norm, epi, out_dtype, splits, stream);
+    if (a.M <= 4) return gemv_launch_rows<4>(a, units, norm, epi, out_dtype, splits, stream);
+    return gemv_launch_rows<8>(a, units, norm, epi, out_dtype, splits, stream);
+}

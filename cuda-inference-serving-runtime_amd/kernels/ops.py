@@ -71,6 +71,10 @@ def _declare(h):
         fn.restype = C.c_int
     h.cisr_gemm_wide_workspace.argtypes = [i, i, i, i]
     h.cisr_gemm_wide_workspace.restype = C.c_longlong
+    h.cisr_gemv_ok.argtypes = [i, i]
+    h.cisr_gemv_ok.restype = C.c_int
+    h.cisr_gemv_set_rows.argtypes = [i]
+    h.cisr_gemv_set_rows.restype = None
 
 
 _attention_entries = {}
@@ -437,6 +441,8 @@ def wide_ok(m, w, swiglu=False, after_norm=False):
     `after_norm`: the rows are the output of an RMSNorm, which the other kernel would fuse (it then reads the
     float residual and the norm's weights for every 16 rows of W, which costs it more than bf16 rows do)."""
     n, k = w.shape
+    if gemv_ok(m, k):      # very few rows: the matrix-vector kernel takes them, whatever the size of the weights
+        return False
     least = WIDE_MIN_BYTES_FEW_ROWS if m <= 16 else WIDE_MIN_BYTES if m <= 32 else WIDE_MIN_BYTES_MANY_ROWS
     if m <= 16 and n < 16 * _compute_units(w.device) and k >= 4096:
         # a narrow output with a long inner size: the fused kernels have a block for every 16 columns and
@@ -448,6 +454,18 @@ def wide_ok(m, w, swiglu=False, after_norm=False):
             or w.data_ptr() % 16 or w.stride(1) != 1):
         return False
     return _wide_plan(m, n // 2 if swiglu else n, k, swiglu) >= 0
+
+
+def gemv_ok(m, k):
+    """Whether a product of m rows with an inner size of k runs the matrix-vector kernel (few rows: a wave owns whole
+    rows of the weights; see csrc/gemv.hip).  The weight-streaming entry points choose it themselves; callers ask
+    only to know that the wide kernel and its separate norm are not wanted."""
+    return bool(lib().cisr_gemv_ok(int(m), int(k)))
+
+
+def set_gemv_rows(rows):
+    """The most rows that the matrix-vector kernel is given (0 to 8; 0 switches it off): for measurements and tests."""
+    lib().cisr_gemv_set_rows(int(rows))
 
 
 _units = {}

@@ -109,6 +109,16 @@ def plain_logits(folder, tokens):
     return _PLAIN[key]
 
 
+@pytest.fixture
+def no_gemv():
+    """Products of up to 8 rows run the matrix-vector kernel; a test about the kernels that took such products before
+    it (and still take 9 rows and more) switches it off for its duration."""
+    from runtime.kernels import ops
+    ops.set_gemv_rows(0)
+    yield
+    ops.set_gemv_rows(8)
+
+
 def tune_attention(model, **settings):
     """Give every attention mixer of `model` launch rules that are told `settings` (kernels.attention.AttentionTuning)."""
     from runtime.kernels.attention import AttentionTuning

@@ -272,7 +272,7 @@ def test_decoded_tokens_of_mixed_steps_in_a_launch_of_their_own(folders, name, d
 
 @pytest.mark.parametrize("name", ["a", "b"])
 @pytest.mark.parametrize("execution", ["eager", "graph"])
-def test_steps_through_the_wide_product_match_the_plain_model(folders, name, execution, monkeypatch):
+def test_steps_through_the_wide_product_match_the_plain_model(folders, name, execution, monkeypatch, no_gemv):
     """With large weights the products of steps of up to 64 rows run the kernel that keeps the activations in
     registers, with norm, rotary embedding and cache write as kernels of their own; forced here on the tiny
     models: decode steps, short portions, mixed steps, again and again (its workspace is shared by the steps)."""
@@ -328,7 +328,7 @@ REAL_SIZES = {
 
 @pytest.mark.parametrize("execution", ["eager", "graph"])
 @pytest.mark.parametrize("sizes", ["1.7b", "8b"])
-def test_layers_of_real_sizes_match_the_plain_model(tmp_path_factory, sizes, execution, monkeypatch):
+def test_layers_of_real_sizes_match_the_plain_model(tmp_path_factory, sizes, execution, monkeypatch, no_gemv):
     """Layers of real sizes: the sizes at which products choose other kernels by themselves (the wide
     weight-streaming product for decode steps, with the fused projection finishing in it; the vendor's library
     for portions of more than 64 rows).  Whole prompts, portions, decode steps of several requests and mixed

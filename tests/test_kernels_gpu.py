@@ -20,6 +20,12 @@ def ops():
     return o
 
 
+@pytest.fixture(autouse=True)
+def other_kernels_take_few_rows(no_gemv):
+    """This module is about the kernels that take products of 9 rows and more, which its tests also run with fewer
+    rows; the matrix-vector kernel, which would take those, has a module of its own (test_gemv_gpu.py)."""
+
+
 def tol(dtype):
     return dict(rtol=2e-5, atol=2e-6) if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
 

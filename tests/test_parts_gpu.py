@@ -109,7 +109,7 @@ def test_block_part(setup):
     runner.cache.check()
 
 
-def test_product_left_to_the_next_norm_only_if_that_norm_adds_it(folders, monkeypatch):
+def test_product_left_to_the_next_norm_only_if_that_norm_adds_it(folders, monkeypatch, no_gemv):
     """ctx.add_product leaves a product that the wide kernel cuts into slices to the norm named in ctx.next_norm, if
     that norm says it adds partial sums; RMSNorm.forward then gives the norm of the finished rows and finishes them;
     any other reader (no norm named, a norm of another kind, ctx.settle) gets finished rows."""

@@ -140,25 +140,27 @@ __global__ void attn_merge_kernel(const float* __restrict__ part_o, const float*
         }
         return;
     }
-    // more splits: sixteen at a time, all their loads issued before the first is used, merged into running sums
-    // (maximum, denominator, numerator) in the order of the splits
+    // more splits: thirty-two at a time, all their loads issued before the first is used (one trip to memory for up
+    // to 32 splits: a second batch would wait for the first), merged into running sums (maximum, denominator,
+    // numerator) in the order of the splits
+    constexpr int SB = 32;
     for (int d = threadIdx.x; d < dim; d += blockDim.x) {
         float m = -INFINITY, den = 0.f, num = 0.f;
-        for (int s0 = 0; s0 < splits; s0 += 16) {
-            float ms[16], ls[16], os[16];
+        for (int s0 = 0; s0 < splits; s0 += SB) {
+            float ms[SB], ls[SB], os[SB];
 #pragma unroll
-            for (int s = 0; s < 16; ++s) {
+            for (int s = 0; s < SB; ++s) {
                 const size_t at = base + min(s0 + s, splits - 1);
                 ms[s] = part_ml[at * 2]; ls[s] = part_ml[at * 2 + 1]; os[s] = part_o[at * dim + d];
             }
             float m_new = m;
 #pragma unroll
-            for (int s = 0; s < 16; ++s) if (s0 + s < splits) m_new = fmaxf(m_new, ms[s]);
+            for (int s = 0; s < SB; ++s) if (s0 + s < splits) m_new = fmaxf(m_new, ms[s]);
             if (m_new == -INFINITY) continue;             // nothing visible so far
             const float keep = LOG2 ? exp2f(m - m_new) : expf(m - m_new);   // m = -inf gives 0
             den *= keep; num *= keep; m = m_new;
 #pragma unroll
-            for (int s = 0; s < 16; ++s) {
+            for (int s = 0; s < SB; ++s) {
                 if (s0 + s >= splits) continue;
                 const float dm = ms[s] - m;
                 const float w = ls[s] > 0.f ? (LOG2 ? exp2f(dm) : expf(dm)) * ls[s] : 0.f;
@@ -170,13 +172,17 @@ __global__ void attn_merge_kernel(const float* __restrict__ part_o, const float*
     }
 }
 
+// A thread a coordinate of the head (a second coordinate a thread is a second trip to memory): 64 to 256 threads.
+static int merge_threads(int dim) { return dim <= 64 ? 64 : dim <= 128 ? 128 : 256; }
+
 // merge of the matrix-core kernel's partials (bf16 output, maxima in log2 units)
 extern "C" int cisr_attn_merge(const float* part_o, const float* part_ml, void* out, int rows, int heads, int dim,
                                int splits, const int* row_ids, hipStream_t stream) {
     if (rows <= 0) return 0;
     if (heads > 65535 || splits < 1) return (int)hipErrorInvalidValue;
-    if (splits <= 16) attn_merge_kernel<bf16_t, true, false><<<dim3(rows, heads), 64, 0, stream>>>(part_o, part_ml, (bf16_t*)out, heads, dim, splits, row_ids);
-    else attn_merge_kernel<bf16_t, true, true><<<dim3(rows, heads), 64, 0, stream>>>(part_o, part_ml, (bf16_t*)out, heads, dim, splits, row_ids);
+    const int threads = merge_threads(dim);
+    if (splits <= 16) attn_merge_kernel<bf16_t, true, false><<<dim3(rows, heads), threads, 0, stream>>>(part_o, part_ml, (bf16_t*)out, heads, dim, splits, row_ids);
+    else attn_merge_kernel<bf16_t, true, true><<<dim3(rows, heads), threads, 0, stream>>>(part_o, part_ml, (bf16_t*)out, heads, dim, splits, row_ids);
     return CISR_LAUNCH_CHECK();
 }
 
@@ -199,12 +205,13 @@ extern "C" int cisr_attn_rowwise(const void* q, int q_row_stride, const void* kc
             dim, page_size, width, window, scale, splits);
     int err = CISR_LAUNCH_CHECK();
     if (err || splits == 1) return err;
+    const int threads = merge_threads(dim);
     if (dtype == DT_F32) {
-        if (splits <= 16) attn_merge_kernel<float, false, false><<<dim3(rows, heads), 64, 0, stream>>>(part_o, part_ml, (float*)out, heads, dim, splits);
-        else attn_merge_kernel<float, false, true><<<dim3(rows, heads), 64, 0, stream>>>(part_o, part_ml, (float*)out, heads, dim, splits);
+        if (splits <= 16) attn_merge_kernel<float, false, false><<<dim3(rows, heads), threads, 0, stream>>>(part_o, part_ml, (float*)out, heads, dim, splits);
+        else attn_merge_kernel<float, false, true><<<dim3(rows, heads), threads, 0, stream>>>(part_o, part_ml, (float*)out, heads, dim, splits);
     } else {
-        if (splits <= 16) attn_merge_kernel<bf16_t, false, false><<<dim3(rows, heads), 64, 0, stream>>>(part_o, part_ml, (bf16_t*)out, heads, dim, splits);
-        else attn_merge_kernel<bf16_t, false, true><<<dim3(rows, heads), 64, 0, stream>>>(part_o, part_ml, (bf16_t*)out, heads, dim, splits);
+        if (splits <= 16) attn_merge_kernel<bf16_t, false, false><<<dim3(rows, heads), threads, 0, stream>>>(part_o, part_ml, (bf16_t*)out, heads, dim, splits);
+        else attn_merge_kernel<bf16_t, false, true><<<dim3(rows, heads), threads, 0, stream>>>(part_o, part_ml, (bf16_t*)out, heads, dim, splits);
     }
     return CISR_LAUNCH_CHECK();
 }

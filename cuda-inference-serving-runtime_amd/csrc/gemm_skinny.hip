@@ -20,11 +20,23 @@ static int launch_rows(const SkinnyArgs& a, int blocks, bool norm, int epi, int 
 
 static bool aligned16(const void* p) { return ((uintptr_t)p) % 16 == 0; }
 
-// Very few rows: the matrix-vector kernel (gemv.hip), whatever the size of the weights.  The most rows it is given
-// can be set (cisr_gemv_set_rows: 0 switches it off), for measurements of one kernel against the other.
-static int gemv_rows = GEMV_MAX_ROWS;
-extern "C" void cisr_gemv_set_rows(int rows) { gemv_rows = rows < 0 ? 0 : rows > GEMV_MAX_ROWS ? GEMV_MAX_ROWS : rows; }
-extern "C" int cisr_gemv_ok(int M, int K) { return M <= gemv_rows && cisr_gemv_takes(M, K); }
+// One or two rows against weights of 4 MB and more: the matrix-vector kernel (gemv.hip).  Measured on an MI355X, decode
+// steps in captured programs (ms a step without it -> with it): 1.7B sizes, 8 layers, one request 0.537 -> 0.441, two
+// 0.571 -> 0.506; 8B sizes, 8 layers, 1.239 -> 1.066 and 1.254 -> 1.130.  Four rows lose (0.608 -> 0.636, 1.325 ->
+// 1.448: every row more is another read of LDS and another set of dot instructions for every 16 bytes of W), and so do
+// the small weights of the 135M sizes at any number of rows (one request 0.670 -> 0.751: there a product is its
+// prologue and epilogue, and the narrow kernel's are shorter; a form of this kernel for such weights that is a single
+// trip to memory, a unit a wave, no LDS and no barrier, came to the narrow kernel's times within 3 %, one request 0.668
+// -> 0.684, and lost with two, 0.682 -> 0.799: not kept).  The most rows it is given and the least bytes can be
+// set (cisr_gemv_set: rows 0 switches it off), for measurements of one kernel against the other and for tests.
+static int gemv_rows = 2;
+static long long gemv_bytes = 4ll << 20;
+extern "C" void cisr_gemv_set(int rows, long long least_bytes) {
+    gemv_rows = rows < 0 ? 0 : rows > GEMV_MAX_ROWS ? GEMV_MAX_ROWS : rows;
+    gemv_bytes = least_bytes < 0 ? 0 : least_bytes;
+}
+// `N`: rows of W that the product reads (both blocks of a gated product)
+extern "C" int cisr_gemv_ok(int M, int N, int K) { return M <= gemv_rows && (long long)N * K * 2 >= gemv_bytes && cisr_gemv_takes(M, K); }
 
 // Few rows against small weights with a narrow output: a block for every 16 columns would leave most compute
 // units idle, so the narrow kernels take over (a block for every 4 columns).  Measured on an MI355X in captured
@@ -55,7 +67,7 @@ extern "C" int cisr_gemm_skinny_bf16(const void* A, int lda, const void* W, int 
     a.A = A; a.lda = lda; a.W = (const bf16_t*)W; a.ldw = ldw; a.C = C; a.ldc = ldc; a.R = R; a.ldr = ldr;
     a.M = M; a.N = N; a.K = K; a.dual_off = dual_off; a.norm_w = norm_w; a.eps = eps; a.rows = rows;
     const int epi = dual_off > 0 ? EPI_SWIGLU : EPI_STORE;
-    if (cisr_gemv_ok(M, K)) return cisr_gemv_launch(a, N, norm_w != nullptr, epi, out_dtype, 0, stream);
+    if (cisr_gemv_ok(M, dual_off > 0 ? 2 * N : N, K)) return cisr_gemv_launch(a, N, norm_w != nullptr, epi, out_dtype, 0, stream);
     if (narrow_wanted(M, dual_off > 0 ? 2 * N : N, K, norm_w != nullptr)) return launch_narrow(a, (N + 3) / 4, norm_w != nullptr, epi, out_dtype, stream);
     const int blocks = (N + 15) / 16;
     return launch_rows(a, blocks, norm_w != nullptr, epi, out_dtype, stream);
@@ -78,7 +90,7 @@ extern "C" int cisr_qkv_rope_skinny(const void* A, int lda, const void* W, int l
     a.positions = positions; a.slots = slots; a.cos_tab = cos_tab; a.sin_tab = sin_tab;
     a.kcache = (bf16_t*)kcache; a.vcache = (bf16_t*)vcache; a.heads = heads; a.kv_heads = kv_heads;
     a.head_dim = head_dim; a.page_size = page_size; a.max_pos = max_pos;
-    if (cisr_gemv_ok(M, K)) return cisr_gemv_launch(a, a.N / 2, norm_w != nullptr, EPI_ROPE, DT_BF16, 0, stream);
+    if (cisr_gemv_ok(M, a.N, K)) return cisr_gemv_launch(a, a.N / 2, norm_w != nullptr, EPI_ROPE, DT_BF16, 0, stream);
     if (narrow_wanted(M, a.N, K, norm_w != nullptr)) return launch_narrow(a, a.N / 4, norm_w != nullptr, EPI_ROPE, DT_BF16, stream);
     const int blocks = (heads + 2 * kv_heads) * (head_dim / 16);
     return launch_rows(a, blocks, norm_w != nullptr, EPI_ROPE, DT_BF16, stream);
@@ -90,7 +102,7 @@ extern "C" int cisr_qkv_rope_skinny(const void* A, int lda, const void* W, int l
 extern "C" int cisr_gemm_merged_ok(int M, int N, int heads, int head_dim, int splits) {
     const int K = heads * head_dim, rows = M <= 4 ? 4 : M <= 8 ? 8 : 16;
     const int batches = rows == 4 ? 2 : rows == 8 ? 3 : 5;
-    if (M >= 1 && head_dim % 8 == 0 && (splits == 2 || splits == 4 || splits == 8) && cisr_gemv_ok(M, K)) return 1;
+    if (M >= 1 && head_dim % 8 == 0 && (splits == 2 || splits == 4 || splits == 8) && cisr_gemv_ok(M, N, K)) return 1;
     return M >= 1 && M <= 16 && head_dim % 8 == 0 && (splits == 2 || splits == 4 || splits == 8) &&
            narrow_wanted(M, N, K, false) && (size_t)rows * (K + 8) * 2 <= 40 * 1024 && M * (K / 8) <= batches * 256;
 }
@@ -105,7 +117,7 @@ extern "C" int cisr_gemm_merged_bf16(const void* part_o, const float* part_ml, i
     SkinnyArgs a = {};
     a.W = (const bf16_t*)W; a.ldw = ldw; a.C = C; a.ldc = ldc; a.R = R; a.ldr = ldr; a.M = M; a.N = N; a.K = K;
     a.part_o = (const bf16_t*)part_o; a.part_ml = part_ml; a.merge_heads = heads; a.merge_dim = head_dim;
-    if (cisr_gemv_ok(M, K)) return cisr_gemv_launch(a, N, false, EPI_STORE, DT_F32, splits, stream);
+    if (cisr_gemv_ok(M, N, K)) return cisr_gemv_launch(a, N, false, EPI_STORE, DT_F32, splits, stream);
     const int units = (N + 3) / 4;
     if (M <= 4) return cisr_narrow_merge_launch_t1(a, units, splits, stream);
     if (M <= 8) return cisr_narrow_merge_launch_t2(a, units, splits, stream);

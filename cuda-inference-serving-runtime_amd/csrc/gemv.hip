@@ -81,72 +81,114 @@ gemv_kernel(SkinnyArgs p, int units, int per_wave) {
     gv_u32x4 wcur[R][CB];
     load_batch(unit_of(0), 0, wcur);                  // on its way while the activations are prepared
 
-    // ---- prologue: the activation rows as packed bf16 in LDS
+    // ---- prologue: the activation rows as packed bf16 in LDS.  Every batch of loads is issued before the first of
+    // them is used, for all rows at once, with clamped addresses instead of branches (a branch around a load makes it a
+    // trip to memory of its own: eight rows one after the other took 6 us)
     if constexpr (NORM) {
         const int words4 = K / 4;
+        const float* xrow[M];
+        {
+            int src[M];
+#pragma unroll
+            for (int m = 0; m < M; ++m) { const int mm = m < p.M ? m : p.M - 1; src[m] = p.rows ? p.rows[mm] : mm; }
+#pragma unroll
+            for (int m = 0; m < M; ++m) xrow[m] = (const float*)p.A + (size_t)src[m] * p.lda;
+        }
+        float sq[M];
+#pragma unroll
+        for (int m = 0; m < M; ++m) sq[m] = 0.f;
+        constexpr int G = M <= 2 ? 4 : 2;                // 16-byte words of a row a thread takes per batch
+        for (int k0 = 0; k0 < words4; k0 += GEMV_THREADS * G) {
+            gv_f32x4 nv[G], xv[M][G];
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                const int k4 = k0 + g * GEMV_THREADS + tid, kk = k4 < words4 ? k4 : 0;
+                nv[g] = *(const gv_f32x4*)(p.norm_w + kk * 4);
+#pragma unroll
+                for (int m = 0; m < M; ++m) xv[m][g] = *(const gv_f32x4*)(xrow[m] + kk * 4);
+            }
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                const int k4 = k0 + g * GEMV_THREADS + tid;
+                if (k4 < words4) {
+#pragma unroll
+                    for (int m = 0; m < M; ++m) {
+                        const gv_f32x4 x = xv[m][g];
+                        const bool live = m < p.M;
+                        sq[m] += x.x * x.x + x.y * x.y + x.z * x.z + x.w * x.w;
+                        a_lds[m * words + k4 * 2] = live ? pack_bf16x2(x.x * nv[g].x, x.y * nv[g].y) : 0u;
+                        a_lds[m * words + k4 * 2 + 1] = live ? pack_bf16x2(x.z * nv[g].z, x.w * nv[g].w) : 0u;
+                    }
+                }
+            }
+        }
 #pragma unroll
         for (int m = 0; m < M; ++m) {
-            float sq = 0.f;
-            if (m < p.M) {
-                const int src = p.rows ? p.rows[m] : m;
-                const float* x = (const float*)p.A + (size_t)src * p.lda;
-#pragma unroll 4
-                for (int k4 = tid; k4 < words4; k4 += GEMV_THREADS) {
-                    const gv_f32x4 xv = *(const gv_f32x4*)(x + k4 * 4), nv = *(const gv_f32x4*)(p.norm_w + k4 * 4);
-                    sq += xv.x * xv.x + xv.y * xv.y + xv.z * xv.z + xv.w * xv.w;
-                    a_lds[m * words + k4 * 2] = pack_bf16x2(xv.x * nv.x, xv.y * nv.y);
-                    a_lds[m * words + k4 * 2 + 1] = pack_bf16x2(xv.z * nv.z, xv.w * nv.w);
-                }
-            } else {
-                for (int k4 = tid; k4 < words4; k4 += GEMV_THREADS) { a_lds[m * words + k4 * 2] = 0u; a_lds[m * words + k4 * 2 + 1] = 0u; }
-            }
-            sq = wave_sum(sq);
-            if (lane == 0) ssq_s[m][wave] = sq;
+            const float total = wave_sum(sq[m]);
+            if (lane == 0) ssq_s[m][wave] = total;
         }
     } else if constexpr (MSPL > 0) {
         const int per_row = K / 8, n_items = M * per_row;
         const int D = p.merge_dim, nh = p.merge_heads;
-        for (int item = tid; item < n_items; item += GEMV_THREADS) {
-            const int row = item / per_row, k = (item % per_row) * 8;
-            gv_u32x4 out = {0u, 0u, 0u, 0u};
-            if (row < p.M) {
+        constexpr int G = MSPL <= 4 ? 2 : 1;             // items a thread merges per batch
+        for (int i0 = 0; i0 < n_items; i0 += GEMV_THREADS * G) {
+            gv_u32x4 po[G][MSPL];
+            float ms[G][MSPL], ls[G][MSPL];
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                const int item = i0 + g * GEMV_THREADS + tid, it = item < n_items ? item : 0;
+                const int row = min(it / per_row, p.M - 1), k = (it % per_row) * 8;
                 const size_t base = ((size_t)row * nh + k / D) * MSPL;
-                gv_u32x4 po[MSPL];
-                float ms[MSPL], ls[MSPL];
 #pragma unroll
                 for (int sp = 0; sp < MSPL; ++sp) {
-                    po[sp] = *(const gv_u32x4*)(p.part_o + (base + sp) * D + k % D);
-                    ms[sp] = p.part_ml[(base + sp) * 2]; ls[sp] = p.part_ml[(base + sp) * 2 + 1];
+                    po[g][sp] = *(const gv_u32x4*)(p.part_o + (base + sp) * D + k % D);
+                    ms[g][sp] = p.part_ml[(base + sp) * 2]; ls[g][sp] = p.part_ml[(base + sp) * 2 + 1];
                 }
+            }
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                const int item = i0 + g * GEMV_THREADS + tid;
+                if (item >= n_items) continue;
+                const int row = item / per_row, k = (item % per_row) * 8;
                 float mx = -INFINITY;
 #pragma unroll
-                for (int sp = 0; sp < MSPL; ++sp) mx = fmaxf(mx, ms[sp]);
+                for (int sp = 0; sp < MSPL; ++sp) mx = fmaxf(mx, ms[g][sp]);
                 float den = 0.f, num[8];
 #pragma unroll
                 for (int j = 0; j < 8; ++j) num[j] = 0.f;
 #pragma unroll
                 for (int sp = 0; sp < MSPL; ++sp) {       // in the order of the splits
-                    const float w = ls[sp] > 0.f ? __builtin_amdgcn_exp2f(ms[sp] - mx) * ls[sp] : 0.f;
+                    const float w = ls[g][sp] > 0.f ? __builtin_amdgcn_exp2f(ms[g][sp] - mx) * ls[g][sp] : 0.f;
                     den += w;
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
-                        num[2 * j] += w * __uint_as_float(po[sp][j] << 16);
-                        num[2 * j + 1] += w * __uint_as_float(po[sp][j] & 0xffff0000u);
+                        num[2 * j] += w * __uint_as_float(po[g][sp][j] << 16);
+                        num[2 * j + 1] += w * __uint_as_float(po[g][sp][j] & 0xffff0000u);
                     }
                 }
-                const float inv = den > 0.f ? 1.0f / den : 0.f;
-                out = (gv_u32x4){pack_bf16x2(num[0] * inv, num[1] * inv), pack_bf16x2(num[2] * inv, num[3] * inv),
-                                 pack_bf16x2(num[4] * inv, num[5] * inv), pack_bf16x2(num[6] * inv, num[7] * inv)};
+                const float inv = (den > 0.f && row < p.M) ? 1.0f / den : 0.f;   // (a row without keys, or no row: zeros)
+                *(gv_u32x4*)(a_lds + row * words + k / 2) =
+                    (gv_u32x4){pack_bf16x2(num[0] * inv, num[1] * inv), pack_bf16x2(num[2] * inv, num[3] * inv),
+                               pack_bf16x2(num[4] * inv, num[5] * inv), pack_bf16x2(num[6] * inv, num[7] * inv)};
             }
-            *(gv_u32x4*)(a_lds + row * words + k / 2) = out;
         }
     } else {
         const int n_items = M * nchunks;
-        for (int item = tid; item < n_items; item += GEMV_THREADS) {
-            const int row = item / nchunks, c = item % nchunks;
-            gv_u32x4 v = {0u, 0u, 0u, 0u};
-            if (row < p.M) v = *(const gv_u32x4*)((const bf16_t*)p.A + (size_t)row * p.lda + c * 8);
-            *(gv_u32x4*)(a_lds + row * words + c * 4) = v;
+        constexpr int G = 4;
+        for (int i0 = 0; i0 < n_items; i0 += GEMV_THREADS * G) {
+            gv_u32x4 v[G];
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                const int item = i0 + g * GEMV_THREADS + tid, it = item < n_items ? item : 0;
+                v[g] = *(const gv_u32x4*)((const bf16_t*)p.A + (size_t)min(it / nchunks, p.M - 1) * p.lda + (it % nchunks) * 8);
+            }
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                const int item = i0 + g * GEMV_THREADS + tid;
+                if (item >= n_items) continue;
+                const int row = item / nchunks;
+                *(gv_u32x4*)(a_lds + row * words + (item % nchunks) * 4) = row < p.M ? v[g] : (gv_u32x4){0u, 0u, 0u, 0u};
+            }
         }
     }
     __syncthreads();
@@ -195,6 +237,7 @@ gemv_kernel(SkinnyArgs p, int units, int per_wave) {
             load_batch(more ? u : unit_of(j + 1), more ? b + 1 : 0, wnext);
 #pragma unroll
             for (int c = 0; c < CB; ++c) {
+                if (b * CB + c >= iters) break;        // (uniform: a slot that no lane has a chunk for)
                 const int chunk = lane + WAVE * (b * CB + c);
                 const bool ok = chunk < nchunks;
                 const int at = ok ? chunk * 4 : 0;
@@ -292,10 +335,12 @@ static int gemv_launch_one(const SkinnyArgs& a, int units, hipStream_t stream) {
         hipError_t e = hipFuncSetAttribute((const void*)gemv_kernel<M, NORM, EPI, TC, MSPL>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return (int)e;
     }
-    // units a wave: as few as give every compute unit eight waves (two blocks) of work, so that a short product is one round
+    // Blocks: with units enough, exactly two a compute unit (eight waves), so that every compute unit streams the same
+    // number of bytes (384 blocks on 256 units leave half of them with twice the work of the others); with fewer units
+    // than that many waves, one unit a wave.
     const int waves = gemv_compute_units() * 8;
     const int per_wave = (units + waves - 1) / waves;
-    const int blocks = (units + GEMV_WAVES * per_wave - 1) / (GEMV_WAVES * per_wave);
+    const int blocks = units >= waves ? waves / GEMV_WAVES : (units + GEMV_WAVES - 1) / GEMV_WAVES;
     gemv_kernel<M, NORM, EPI, TC, MSPL><<<blocks, GEMV_THREADS, lds, stream>>>(a, units, per_wave);
     return CISR_LAUNCH_CHECK();
 }

@@ -71,10 +71,10 @@ def _declare(h):
         fn.restype = C.c_int
     h.cisr_gemm_wide_workspace.argtypes = [i, i, i, i]
     h.cisr_gemm_wide_workspace.restype = C.c_longlong
-    h.cisr_gemv_ok.argtypes = [i, i]
+    h.cisr_gemv_ok.argtypes = [i, i, i]
     h.cisr_gemv_ok.restype = C.c_int
-    h.cisr_gemv_set_rows.argtypes = [i]
-    h.cisr_gemv_set_rows.restype = None
+    h.cisr_gemv_set.argtypes = [i, ll]
+    h.cisr_gemv_set.restype = None
 
 
 _attention_entries = {}
@@ -441,7 +441,7 @@ def wide_ok(m, w, swiglu=False, after_norm=False):
     `after_norm`: the rows are the output of an RMSNorm, which the other kernel would fuse (it then reads the
     float residual and the norm's weights for every 16 rows of W, which costs it more than bf16 rows do)."""
     n, k = w.shape
-    if gemv_ok(m, k):      # very few rows: the matrix-vector kernel takes them, whatever the size of the weights
+    if gemv_ok(m, n, k):   # one or two rows against large weights: the matrix-vector kernel takes them
         return False
     least = WIDE_MIN_BYTES_FEW_ROWS if m <= 16 else WIDE_MIN_BYTES if m <= 32 else WIDE_MIN_BYTES_MANY_ROWS
     if m <= 16 and n < 16 * _compute_units(w.device) and k >= 4096:
@@ -456,16 +456,21 @@ def wide_ok(m, w, swiglu=False, after_norm=False):
     return _wide_plan(m, n // 2 if swiglu else n, k, swiglu) >= 0
 
 
-def gemv_ok(m, k):
-    """Whether a product of m rows with an inner size of k runs the matrix-vector kernel (few rows: a wave owns whole
-    rows of the weights; see csrc/gemv.hip).  The weight-streaming entry points choose it themselves; callers ask
-    only to know that the wide kernel and its separate norm are not wanted."""
-    return bool(lib().cisr_gemv_ok(int(m), int(k)))
+GEMV_ROWS, GEMV_MIN_BYTES = 2, 4 << 20
 
 
-def set_gemv_rows(rows):
-    """The most rows that the matrix-vector kernel is given (0 to 8; 0 switches it off): for measurements and tests."""
-    lib().cisr_gemv_set_rows(int(rows))
+def gemv_ok(m, n, k):
+    """Whether a product of m rows with weights [n, k] runs the matrix-vector kernel (one or two rows against weights
+    of 4 MB and more: a wave owns whole rows of the weights; see csrc/gemv.hip and the measurements in
+    csrc/gemm_skinny.hip).  The weight-streaming entry points choose it themselves; callers ask only to know that
+    the wide kernel and its separate norm are not wanted."""
+    return bool(lib().cisr_gemv_ok(int(m), int(n), int(k)))
+
+
+def set_gemv(rows=GEMV_ROWS, least_bytes=GEMV_MIN_BYTES):
+    """The most rows (0 to 8; 0 switches it off) and the least bytes of weights that the matrix-vector kernel is given:
+    for measurements and tests.  Without arguments: the rule as it is."""
+    lib().cisr_gemv_set(int(rows), int(least_bytes))
 
 
 _units = {}

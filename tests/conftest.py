@@ -111,12 +111,12 @@ def plain_logits(folder, tokens):
 
 @pytest.fixture
 def no_gemv():
-    """Products of up to 8 rows run the matrix-vector kernel; a test about the kernels that took such products before
-    it (and still take 9 rows and more) switches it off for its duration."""
+    """Products of one or two rows against large weights run the matrix-vector kernel; a test about the kernels that
+    take every other product switches it off for its duration."""
     from runtime.kernels import ops
-    ops.set_gemv_rows(0)
+    ops.set_gemv(0)
     yield
-    ops.set_gemv_rows(8)
+    ops.set_gemv()
 
 
 def tune_attention(model, **settings):

@@ -1,4 +1,4 @@
-"""The matrix-vector kernel that takes products of one to eight rows: every prologue (plain rows, fused RMSNorm with
+"""The matrix-vector kernel (one or two rows against large weights in the engine; here given up to eight rows and weights of any size): every prologue (plain rows, fused RMSNorm with
 and without picked rows, the merge of split attention) and every epilogue (store, residual, SwiGLU, rotary embedding
 with the cache write) against float64, at the family's sizes and at sizes that fit nothing (inner sizes that leave
 lanes without a chunk, or give them several batches; outputs that do not fill the last wave).  A row's result is
@@ -19,8 +19,9 @@ DEV = "cuda:0"
 def ops():
     from runtime.kernels import ops as o
     o.lib()
-    o.set_gemv_rows(8)
-    return o
+    o.set_gemv(8, 0)          # every product of up to eight rows, whatever the size of the weights
+    yield o
+    o.set_gemv()
 
 
 def rnd(*shape, dtype=torch.float32, seed=0, scale=1.0):
@@ -43,7 +44,7 @@ SHAPES = [(1, 16, 32), (3, 100, 72), (8, 576, 576), (8, 576, 1536), (5, 1003, 20
 
 @pytest.mark.parametrize("M, N, K", SHAPES)
 def test_plain_and_residual(ops, M, N, K):
-    assert ops.gemv_ok(M, K) and not ops.gemv_ok(9, K)
+    assert ops.gemv_ok(M, N, K) and not ops.gemv_ok(9, N, K)
     a, w, r = rnd(M, K, dtype=torch.bfloat16, seed=1), rnd(N, K, dtype=torch.bfloat16, seed=2, scale=0.1), rnd(M, N, seed=3)
     want = f64(a) @ f64(w).T
     tol = dict(rtol=1e-4, atol=1e-5 * math.sqrt(K))
@@ -156,14 +157,17 @@ def test_output_projection_merges_split_attention_itself(ops, M, heads, dim, spl
     np.testing.assert_allclose(f64(got), want, rtol=1e-3, atol=2e-3)
 
 
-def test_few_rows_take_this_kernel_and_nine_do_not(ops):
+def test_which_products_take_this_kernel(ops):
     w = rnd(64, 128, dtype=torch.bfloat16)
-    assert ops.gemv_ok(8, 128) and not ops.gemv_ok(9, 128) and not ops.gemv_ok(4, 100)      # (an inner size that is no multiple of 8)
-    assert not ops.gemv_ok(8, 16384)                                                        # eight rows of it do not fit LDS
-    assert ops.gemv_ok(4, 16384)
+    assert ops.gemv_ok(8, 64, 128) and not ops.gemv_ok(9, 64, 128) and not ops.gemv_ok(4, 64, 100)      # (an inner size that is no multiple of 8)
+    assert not ops.gemv_ok(8, 64, 16384)                                                            # eight rows of it do not fit LDS
+    assert ops.gemv_ok(4, 64, 16384)
     assert not ops.wide_ok(8, w)
-    ops.set_gemv_rows(0)
+    ops.set_gemv()              # the engine's rule: one or two rows, weights of 4 MB and more
     try:
-        assert not ops.gemv_ok(1, 128)
+        assert ops.gemv_ok(1, 2048, 2048) and ops.gemv_ok(2, 6144, 4096) and ops.gemv_ok(1, 49152, 576)
+        assert not ops.gemv_ok(3, 6144, 4096) and not ops.gemv_ok(1, 3072, 576)
+        ops.set_gemv(0)
+        assert not ops.gemv_ok(1, 6144, 4096)
     finally:
-        ops.set_gemv_rows(8)
+        ops.set_gemv(8, 0)

@@ -35,8 +35,13 @@ extern "C" void cisr_gemv_set(int rows, long long least_bytes) {
     gemv_rows = rows < 0 ? 0 : rows > GEMV_MAX_ROWS ? GEMV_MAX_ROWS : rows;
     gemv_bytes = least_bytes < 0 ? 0 : least_bytes;
 }
-// `N`: rows of W that the product reads (both blocks of a gated product)
-extern "C" int cisr_gemv_ok(int M, int N, int K) { return M <= gemv_rows && (long long)N * K * 2 >= gemv_bytes && cisr_gemv_takes(M, K); }
+// The inner size must be at least `gemv_inner`: a row of W shorter than two rounds of a wave's lanes leaves most lanes
+// idle, and the kernel is then its per-row work (the head of the 135M sizes, 49,152 rows of 576: 36 us against 15.7).
+// A least size of 0 bytes lifts that too.  `N`: rows of W that the product reads (both blocks of a gated product).
+static int gemv_inner = 1024;
+extern "C" int cisr_gemv_ok(int M, int N, int K) {
+    return M <= gemv_rows && (long long)N * K * 2 >= gemv_bytes && (K >= gemv_inner || gemv_bytes == 0) && cisr_gemv_takes(M, K);
+}
 
 // Few rows against small weights with a narrow output: a block for every 16 columns would leave most compute
 // units idle, so the narrow kernels take over (a block for every 4 columns).  Measured on an MI355X in captured

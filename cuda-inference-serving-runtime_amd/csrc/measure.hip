@@ -104,3 +104,86 @@ extern "C" int cisr_stream_read(const void* src, long long bytes, void* sink, in
     stream_read_kernel<<<(unsigned)blocks, 256, 0, stream>>>((const read_word_t*)src, bytes / 16, (unsigned*)sink);
     return CISR_LAUNCH_CHECK();
 }
+
+// A chain of dependent matrix-vector products, the leanest kernel that a decode step of one request could be made of:
+// a wave owns one row of W (K = 512 KC bf16), its lanes read one 16-byte chunk of it per 512 inner positions and their
+// slices of the float vector x, the lanes' sums meet by lane exchanges, and lane 0 stores y[row] (squashed into
+// (-1, 1), so that a chain of any length keeps its values).  No LDS, no barrier, every load issued at the start.
+// What `python -m runtime.measure chain` times with it: how short a kernel of a captured chain can be (the floor under
+// the products of a decode step), and whether kernels on two streams that hand their results over through counters in
+// memory (WAIT: poll `cnt_in` until `expect` blocks have arrived; every block bumps `cnt_out` after its stores; x and
+// y then bypass the caches, which are not coherent between the eight dies) beat the order of one stream.
+// The wait is bounded (`spin_limit` polls, or as soon as another block has given up): then `err[0]` is set and the
+// kernel goes on with whatever it reads, so that every wave ends whatever happens.
+typedef float chain_f32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ float chain_bf(uint32_t v, int hi) { return __uint_as_float(hi ? (v & 0xffff0000u) : (v << 16)); }
+
+template <int KC, bool WAIT>
+__global__ void __launch_bounds__(256) chain_phase_kernel(const read_word_t* __restrict__ W, const float* x, float* y, unsigned* cnt_in,
+                                                          unsigned expect, unsigned* cnt_out, unsigned spin_limit, unsigned* err) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int row = blockIdx.x * 4 + wave;
+    read_word_t w[KC];
+#pragma unroll
+    for (int c = 0; c < KC; ++c) w[c] = __builtin_nontemporal_load(W + (size_t)row * (KC * 64) + c * 64 + lane);
+    if (WAIT) {
+        if (threadIdx.x == 0) {
+            unsigned spins = 0;
+            while (__hip_atomic_load(cnt_in, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < expect) {
+                if (++spins > spin_limit || ((spins & 1023u) == 0u && __hip_atomic_load(err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))) { *err = 1u; break; }
+            }
+        }
+        __syncthreads();
+    }
+    float xv[KC][8];
+#pragma unroll
+    for (int c = 0; c < KC; ++c) {
+        const float* p = x + (c * 64 + lane) * 8;
+        chain_f32x4 lo, hi;
+        if (WAIT) {     // straight from memory: another die's L2 may hold what a block there wrote
+            lo = (chain_f32x4){__hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT), __hip_atomic_load(p + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT),
+                               __hip_atomic_load(p + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT), __hip_atomic_load(p + 3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)};
+            hi = (chain_f32x4){__hip_atomic_load(p + 4, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT), __hip_atomic_load(p + 5, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT),
+                               __hip_atomic_load(p + 6, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT), __hip_atomic_load(p + 7, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)};
+        } else {
+            lo = *(const chain_f32x4*)p; hi = *(const chain_f32x4*)(p + 4);
+        }
+        xv[c][0] = lo.x; xv[c][1] = lo.y; xv[c][2] = lo.z; xv[c][3] = lo.w; xv[c][4] = hi.x; xv[c][5] = hi.y; xv[c][6] = hi.z; xv[c][7] = hi.w;
+    }
+    float a = 0.f;
+#pragma unroll
+    for (int c = 0; c < KC; ++c) {
+        const read_word_t v = w[c];
+        a += chain_bf(v.x, 0) * xv[c][0] + chain_bf(v.x, 1) * xv[c][1] + chain_bf(v.y, 0) * xv[c][2] + chain_bf(v.y, 1) * xv[c][3]
+           + chain_bf(v.z, 0) * xv[c][4] + chain_bf(v.z, 1) * xv[c][5] + chain_bf(v.w, 0) * xv[c][6] + chain_bf(v.w, 1) * xv[c][7];
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) a += __shfl_xor(a, off, 64);
+    a = a * 4.f;
+    a = a / (1.f + fabsf(a)) + 0.05f;
+    if (lane == 0) {
+        if (WAIT) __hip_atomic_store(y + row, a, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        else y[row] = a;
+    }
+    if (WAIT && cnt_out) {
+        __builtin_amdgcn_s_waitcnt(0);       // every wave's store is acknowledged before the block's arrival is counted
+        __syncthreads();
+        if (threadIdx.x == 0) __hip_atomic_fetch_add(cnt_out, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
+// y[N] = squash(W[N, K] . x[K]); N a multiple of 4, K 512 or 1536; `wait`: the hand-over through counters (see above).
+extern "C" int cisr_chain_phase(const void* W, const float* x, float* y, int N, int K, unsigned* cnt_in, unsigned expect,
+                                unsigned* cnt_out, unsigned* err, int wait, hipStream_t stream) {
+    if (N <= 0 || N % 4 || (K != 512 && K != 1536) || !W || !x || !y || (wait && (!cnt_in || !err)) || ((uintptr_t)W) % 16 || ((uintptr_t)x) % 16)
+        return (int)hipErrorInvalidValue;
+    const unsigned blocks = (unsigned)(N / 4), limit = 1u << 18;
+    if (K == 512) {
+        if (wait) chain_phase_kernel<1, true><<<blocks, 256, 0, stream>>>((const read_word_t*)W, x, y, cnt_in, expect, cnt_out, limit, err);
+        else chain_phase_kernel<1, false><<<blocks, 256, 0, stream>>>((const read_word_t*)W, x, y, cnt_in, expect, cnt_out, limit, err);
+    } else {
+        if (wait) chain_phase_kernel<3, true><<<blocks, 256, 0, stream>>>((const read_word_t*)W, x, y, cnt_in, expect, cnt_out, limit, err);
+        else chain_phase_kernel<3, false><<<blocks, 256, 0, stream>>>((const read_word_t*)W, x, y, cnt_in, expect, cnt_out, limit, err);
+    }
+    return CISR_LAUNCH_CHECK();
+}

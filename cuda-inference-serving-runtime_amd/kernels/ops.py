@@ -461,15 +461,16 @@ GEMV_ROWS, GEMV_MIN_BYTES = 2, 4 << 20
 
 def gemv_ok(m, n, k):
     """Whether a product of m rows with weights [n, k] runs the matrix-vector kernel (one or two rows against weights
-    of 4 MB and more: a wave owns whole rows of the weights; see csrc/gemv.hip and the measurements in
-    csrc/gemm_skinny.hip).  The weight-streaming entry points choose it themselves; callers ask only to know that
+    of 4 MB and more with an inner size of at least 1024: a wave owns whole rows of the weights; see csrc/gemv.hip
+    and the measurements in csrc/gemm_skinny.hip).  The weight-streaming entry points choose it themselves; callers ask only to know that
     the wide kernel and its separate norm are not wanted."""
     return bool(lib().cisr_gemv_ok(int(m), int(n), int(k)))
 
 
 def set_gemv(rows=GEMV_ROWS, least_bytes=GEMV_MIN_BYTES):
-    """The most rows (0 to 8; 0 switches it off) and the least bytes of weights that the matrix-vector kernel is given:
-    for measurements and tests.  Without arguments: the rule as it is."""
+    """The most rows (0 to 8; 0 switches it off) and the least bytes of weights that the matrix-vector kernel is given
+    (least_bytes 0 also lifts the rule's least inner size): for measurements and tests.  Without arguments: the rule
+    as it is."""
     lib().cisr_gemv_set(int(rows), int(least_bytes))
 
 

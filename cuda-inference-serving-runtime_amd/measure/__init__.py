@@ -17,7 +17,8 @@ def _lib():
         h = library.load(library.MEASURE)
         p, i, ll = C.c_void_p, C.c_int, C.c_longlong
         for name, args in {"cisr_idle": [i, p], "cisr_stream_read": [p, ll, p, i, p],
-                           "cisr_grid_meet": [p, p, i, i, i, C.c_uint, p]}.items():
+                           "cisr_grid_meet": [p, p, i, i, i, C.c_uint, p],
+                           "cisr_chain_phase": [p, p, p, i, i, p, C.c_uint, p, p, i, p]}.items():
             fn = getattr(h, name)
             fn.argtypes, fn.restype = args, C.c_int
         _handle = h
@@ -51,3 +52,18 @@ def grid_meet(blocks, rounds, exchange=0, spin_limit=1 << 22):
     _check(_lib().cisr_grid_meet(words.data_ptr(), passed.data_ptr(), int(exchange), int(blocks), int(rounds), int(spin_limit),
                                  _stream()), "grid_meet")
     return words
+
+
+def chain_phase(w, x, y, counters=None, wait=False):
+    """y = squash(w . x): one link of a chain of dependent matrix-vector products, the leanest kernel a decode step of
+    one request could be made of.  w bf16 [N, K] (N a multiple of 4, K 512 or 1536), x float [K], y float [N].
+    `wait`: the kernel polls counters[0] until counters[1] blocks have arrived before it reads x (straight from
+    memory), and every block bumps counters[2] after its store; counters = (int32 word in, expected, int32 word out or
+    None, int32 error word)."""
+    n, k = w.shape
+    if w.dtype != torch.bfloat16 or x.dtype != torch.float32 or y.dtype != torch.float32 or x.numel() < k or y.numel() < n:
+        raise KernelError("chain_phase: bf16 weights [N, K], float vectors of K and N elements")
+    cin, expect, cout, err = counters if counters is not None else (None, 0, None, None)
+    _check(_lib().cisr_chain_phase(_dev(w, "w"), x.data_ptr(), y.data_ptr(), n, k, None if cin is None else cin.data_ptr(), int(expect),
+                                   None if cout is None else cout.data_ptr(), None if err is None else err.data_ptr(), int(bool(wait)),
+                                   _stream()), "chain_phase")

@@ -6,6 +6,15 @@
   attention_forms          every form of that kernel at a grid of head shapes, beside the form the rule picks
   decode_attention_shapes  every launch shape of the decode attention kernel at a grid of requests and contexts,
                            beside the one the rule picks
+  chain                    a captured chain of 150 dependent matrix-vector products of the 135M sizes' shapes, each
+                           the leanest kernel there is (what a decode step of one request costs at the least); the
+                           same chain with its kernels alternating on two streams and handing over through counters
+                           in memory instead of the stream's order; and two independent chains on two streams
+  reread                   GB/s of a kernel that reads the same buffer again and again, by the buffer's size (what
+                           the L2 caches and the memory-side cache hold from kernel to kernel)
+  hot_weights              decode steps with every layer sharing one layer's weights (the order of layers names one
+                           layer for every place) against distinct layers: what weights that are already in a cache
+                           are worth, the bound of anything that fetches weights ahead
 """
 import argparse
 import json
@@ -244,15 +253,178 @@ def decode_attention_shapes(args):
     return 0
 
 
+def chain(args):
+    """See the module's text.  One line: microseconds a link."""
+    import statistics
+    import torch
+    from runtime import measure
+    dev = torch.device("cuda:0")
+    layers = args.chain_layers
+    shapes = [(512, 512), (512, 512), (512, 512), (1536, 512), (512, 1536)] * layers      # (N, K): five products a layer
+    gen = torch.Generator(device=dev).manual_seed(0)
+    weights = [(torch.rand(n, k, generator=gen, device=dev) * 2 - 1).mul_(1.7 / k ** 0.5).bfloat16() for n, k in shapes]
+    links = len(shapes)
+
+    def buffers():
+        acts = torch.zeros(links + 1, 1536, device=dev)
+        acts[0, :512] = torch.linspace(0.5, 1.0, 512, device=dev)
+        return acts
+    acts, acts2 = buffers(), buffers()
+    counters = torch.zeros((links + 2) * 64, dtype=torch.int32, device=dev)
+    err = counters[(links + 1) * 64:]
+
+    def run(i, buf, wait):
+        cnt = None
+        if wait:
+            cnt = (counters[i * 64:], 0 if i == 0 else shapes[i - 1][0] // 4, counters[(i + 1) * 64:], err)
+        measure.chain_phase(weights[i], buf[i], buf[i + 1], cnt, wait)
+
+    def capture(stream, body):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(stream):
+            body(); stream.synchronize()
+            with torch.cuda.graph(graph, stream=stream):
+                body()
+        return graph
+
+    def timed(step, reps=15):
+        times = []
+        for _ in range(reps):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            step()
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t0)
+        return statistics.median(times) * 1e6
+
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    plain = capture(s1, lambda: [run(i, acts, False) for i in range(links)])
+    torch.cuda.synchronize()
+    reference = acts[links, :512].clone()
+    out = {"links": links, "weights_mb": round(sum(w.numel() * 2 for w in weights) / 2 ** 20, 1)}
+    out["one_stream_us_a_link"] = round(timed(lambda: plain.replay()) / links, 3)
+    # the same kernels with the hand-over through counters, still in one stream's order: what the hand-over itself costs
+    in_order = capture(s1, lambda: (counters.zero_(), [run(i, acts, True) for i in range(links)]))
+    out["one_stream_with_counters_us_a_link"] = round(timed(lambda: in_order.replay()) / links, 3)
+    # even links on one stream, odd links on the other, nothing but the counters between them
+    even = capture(s1, lambda: [run(i, acts, True) for i in range(0, links, 2)])
+    odd = capture(s2, lambda: [run(i, acts, True) for i in range(1, links, 2)])
+
+    def two_streams():
+        with torch.cuda.stream(s1):
+            counters.zero_()
+            s2.wait_stream(s1)
+            even.replay()
+        with torch.cuda.stream(s2):
+            odd.replay()
+    acts[links].zero_()
+    out["two_streams_with_counters_us_a_link"] = round(timed(two_streams) / links, 3)
+    torch.cuda.synchronize()
+    out["two_streams_same_result"] = bool(torch.equal(acts[links, :512], reference)) and int(err[0]) == 0
+    # two independent chains, a stream each: what running two steps side by side costs
+    other = capture(s2, lambda: [run(i, acts2, False) for i in range(links)])
+
+    def side_by_side():
+        with torch.cuda.stream(s1):
+            plain.replay()
+        with torch.cuda.stream(s2):
+            other.replay()
+    out["two_independent_chains_us_a_link_of_each"] = round(timed(side_by_side) / links, 3)
+    print(json.dumps({"metric": "microseconds a link of a captured chain of dependent matrix-vector kernels", "unit": "us",
+                      "value": out["one_stream_us_a_link"], "higher_is_better": False, "n_gpus": 1, **out}))
+    return 0
+
+
+def reread(args):
+    """GB/s of the read-only kernel over a buffer that it reads again and again (20 or more passes in one captured
+    graph, the median of five replays), by the buffer's size."""
+    import statistics
+    import torch
+    from runtime import measure
+    sink = torch.zeros(1, dtype=torch.int32, device="cuda")
+    out = {}
+    for mb in (8, 16, 32, 64, 128, 256, 512, 2048):
+        a = torch.empty(mb << 20, dtype=torch.uint8, device="cuda")
+        a.zero_()
+        passes = max(4, 2048 // mb)
+        graph = torch.cuda.CUDAGraph()
+        measure.stream_read(a, sink, 1024); torch.cuda.synchronize()
+        with torch.cuda.graph(graph):
+            for _ in range(passes):
+                measure.stream_read(a, sink, 1024)
+        graph.replay(); torch.cuda.synchronize()
+        times = []
+        for _ in range(5):
+            t0 = time.perf_counter(); graph.replay(); torch.cuda.synchronize(); times.append((time.perf_counter() - t0) / passes)
+        out[f"{mb}_MB"] = {"us_a_pass": round(statistics.median(times) * 1e6, 1), "GB/s": round((mb << 20) / statistics.median(times) / 1e9)}
+        del a, graph
+    print(json.dumps({"metric": "GB/s of a read-only kernel over a buffer that is read again and again, by size", "unit": "GB/s",
+                      "value": out["32_MB"]["GB/s"], "higher_is_better": True, "n_gpus": 1, "sizes": out}))
+    return 0
+
+
+def hot_weights(args):
+    """Decode steps (captured programs, steps overlapped, as the benchmark times them) of 1, 8 and 64 requests after
+    2,048-token prompts: a model whose layers are distinct against the same model with one layer's weights at every
+    place of the order (every place still keeps a cache of its own)."""
+    import statistics
+    import numpy as np
+    import torch
+    from runtime.config import preset
+    from runtime.engine import ModelRunner, StepEntry, random_model
+    from runtime.models import ScheduleEntry
+    from runtime.sampling import Sampler
+    out = {}
+    for name, layers in (("smollm2-135m", 30), ("smollm2-1.7b", 8)):
+        raw = preset(name)
+        raw["num_hidden_layers"] = layers
+        raw["max_position_embeddings"] = 4096
+        for shared in (False, True):
+            model = random_model(raw, seed=0)
+            if shared:
+                model.schedule = [ScheduleEntry(0) for _ in range(layers)]
+            sampler, rng = Sampler(), np.random.default_rng(0)
+            runner = ModelRunner(model, n_pages=64 * 4096 // 16, page_size=16, max_requests=64, execution="graph")
+            result = {}
+            for batch in (1, 8, 64):
+                keys = [f"{batch}-{i}" for i in range(batch)]
+                last = []
+                for key in keys:
+                    runner.create(key)
+                    logits = runner.step([StepEntry(key, rng.integers(0, raw["vocab_size"], size=2048, dtype=np.int32), [2047])])
+                    last.append(sampler.pick(logits, [(0.0, 0, 0)])[0])
+                params, unread, times = [(0.0, 0, 0)] * batch, None, []
+                for rep in range(4):
+                    torch.cuda.synchronize()
+                    t0 = time.perf_counter()
+                    for _ in range(64):
+                        entries = [StepEntry(k, [0], [0], pending=True) for k in keys] if unread is not None else [StepEntry(k, [t], [0]) for k, t in zip(keys, last)]
+                        unread = runner.pick(sampler, runner.step(entries), params)
+                    torch.cuda.synchronize()
+                    times.append((time.perf_counter() - t0) / 64)
+                for key in keys:
+                    runner.release(key)
+                result[f"b{batch}_ms"] = round(statistics.median(times[1:]) * 1e3, 4)
+            out[f"{name}_{layers}_layers_{'one_layers_weights_everywhere' if shared else 'distinct_layers'}"] = result
+            del runner, model
+            torch.cuda.empty_cache()
+    print(json.dumps({"metric": "ms a decode step with distinct layers and with one layer's weights at every place", "unit": "ms",
+                      "value": out["smollm2-135m_30_layers_distinct_layers"]["b8_ms"], "higher_is_better": False, "n_gpus": 1, "steps": out}))
+    return 0
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser(prog="python -m runtime.measure")
-    ap.add_argument("workload", choices=["floor", "attention", "attention_forms", "decode_attention_shapes"])
+    ap.add_argument("workload", choices=["floor", "attention", "attention_forms", "decode_attention_shapes", "chain", "reread", "hot_weights"])
+    ap.add_argument("--chain-layers", type=int, default=30, help="chain: layers of five products each (30: 113 MB of weights; 240: 904 MB, "
+                                                                 "more than the memory-side cache holds)")
     ap.add_argument("--model", default="smollm2-135m", help="floor: the preset whose decode step the floor is priced for")
     ap.add_argument("--page-size", type=int, default=16)
     ap.add_argument("--attention-rows", default="2048,7936", help="attention workloads: prompt lengths (comma separated)")
     args = ap.parse_args(argv)
     return {"floor": launch_floor, "attention": prompt_attention, "attention_forms": attention_forms,
-            "decode_attention_shapes": decode_attention_shapes}[args.workload](args)
+            "decode_attention_shapes": decode_attention_shapes, "chain": chain, "reread": reread,
+            "hot_weights": hot_weights}[args.workload](args)
 
 
 if __name__ == "__main__":

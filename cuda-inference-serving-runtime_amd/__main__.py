@@ -38,6 +38,9 @@ def main(argv=None):
     parser.add_argument("--max-active", type=int, default=8)
     parser.add_argument("--overlap", action="store_true",
                         help="launch each step before the tokens of the step before are read (same tokens, less idle GPU)")
+    parser.add_argument("--report", action="store_true",
+                        help="add the step function's counters and memory (steps, programs captured and replayed, "
+                             "bytes of workspace, scratch, staging and cache) to the output")
     args = parser.parse_args(argv)
 
     from .config import read_config_json
@@ -81,6 +84,8 @@ def main(argv=None):
     report = dict(device="hip", dtype=args.dtype, execution=execution,
                   weights=f"random-{args.model}" if not args.checkpoint else "pretrained-local",
                   requests=[outcome(r) for r in engine.run()])
+    if args.report:
+        report["runner"] = engine.runner.report()
     print(json.dumps(report, indent=2))
     return 0
 

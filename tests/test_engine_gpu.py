@@ -587,10 +587,13 @@ def test_command_line(folders, tmp_path):
     assert by_key["x"]["generated"] == P.greedy(cfg, w, [1, 2, 3, 4, 5], 4) and by_key["x"]["status"] == "finished"
     assert by_key["y"]["generated"] == P.greedy(cfg, w, [9], 3) and by_key["y"]["ttft_ms"] > 0
     proc = subprocess.run([sys.executable, "-m", "runtime", "--model", "tiny-b", "--tokens", "5,6,7", "--max-new-tokens", "3",
-                           "--execution", "graph", "--overlap", "--pages", "0"], capture_output=True, text=True, timeout=300, env=env, cwd=str(tmp_path))
+                           "--execution", "graph", "--overlap", "--pages", "0", "--report"], capture_output=True, text=True, timeout=300, env=env, cwd=str(tmp_path))
     assert proc.returncode == 0, proc.stderr[-2000:]
     out = json.loads(proc.stdout)
     assert out["weights"] == "random-tiny-b" and len(out["requests"][0]["generated"]) == 3
+    told = out["runner"]
+    assert told["steps"] == told["eager_steps"] + told["replays"] >= 3 and told["programs"] >= 1
+    assert told["workspace_bytes"] > 0 and told["cache"][0]["resident_pages"] == 0
 
 
 def test_smoke_entry():

@@ -10,6 +10,7 @@ import torch
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
+SEEN = []      # (launch value a step array was filled with, the batch's own), by RowsOfSegments.fill
 
 
 def build_toy():
@@ -47,16 +48,73 @@ def build_toy():
             return residual
 
     @dataclass(frozen=True)
+    class RowsOfSegments:
+        """A step array of this file's own (the framework has no such list): for every row of the step the first row
+        of its segment (-1 for a padding row), then for every row its segment (0 for a padding row).  Its launch
+        value, the longest portion of the step, is recorded in SEEN with the true one."""
+
+        def words(self, rows, segments):
+            return 2 * rows
+
+        def launch_value(self, batch):
+            return max(batch.counts)
+
+        def fill(self, out, batch, value):
+            rows = len(out) // 2
+            out[:rows], out[rows:] = -1, 0
+            for segment, (row, count) in enumerate(zip(batch.first_row, batch.counts)):
+                out[row:row + count], out[rows + row:rows + row + count] = row, segment
+            SEEN.append((value, max(batch.counts)))
+
+    class PrefixSumMixer(Mixer):
+        """s_t = s_{t-1} + h_t; out = s_t W^T: DecayMixer with a decay of 1, but as launches only (no host reads, so it
+        runs under graph capture too), which takes a list that no step carries by itself: RowsOfSegments."""
+
+        def __init__(self, name, hidden, decay, declared):
+            assert decay == 1.0
+            self.name, self.hidden, self.declared = name, hidden, declared
+
+        def state_need(self):
+            return StateNeed((self.hidden,), "float32")
+
+        def step_arrays(self):
+            return [RowsOfSegments()] if self.declared else []     # else: asked for at the first step
+
+        def tensor_specs(self):
+            return [TensorSpec(self.name + ".mix.weight", (self.hidden, self.hidden))]
+
+        def bind(self, tensors, dtype):
+            self.weight = tensors[self.name + ".mix.weight"].float()
+
+        def forward(self, h, residual, ctx, site):
+            links, _ = ctx.step_array(RowsOfSegments())
+            T = ctx.n_rows
+            first, segment = links[:T], links[T:2 * T].long()
+            valid = first >= 0
+            r = torch.arange(T, device=h.device)
+            earlier_of_the_same = (first[:, None] == first[None, :]) & (r[None, :] <= r[:, None]) & valid[None, :]
+            state = ctx.cache.state_storage[site]
+            slot = ctx.state_slots.long().index_select(0, segment)
+            x = h.float() * valid[:, None]
+            s = earlier_of_the_same.float() @ x + state.index_select(0, slot)
+            residual += (s @ self.weight.T) * valid[:, None]
+            state.index_add_(0, slot, x)
+            return residual
+
+    @dataclass(frozen=True)
     class ToyConfig:
         vocab_size: int
         hidden_size: int
         decay: float
         max_position_embeddings: int
         rms_norm_eps: float
+        mixer: str = "toy-decay"
+        declared: bool = False
 
         @classmethod
         def from_dict(cls, raw):
-            return cls(raw["vocab_size"], raw["hidden_size"], raw["decay"], raw["max_position_embeddings"], raw["rms_norm_eps"])
+            return cls(raw["vocab_size"], raw["hidden_size"], raw["decay"], raw["max_position_embeddings"], raw["rms_norm_eps"],
+                       raw.get("mixer", "toy-decay"), raw.get("declared", False))
 
     def build(c):
         emb = TokenEmbedding("embed", c.vocab_size, c.hidden_size)
@@ -66,7 +124,9 @@ def build_toy():
         layers = [
             make_part("block", "prenorm", mixer_norm=norm("l0.n1"), mixer=attention, ffn_norm=norm("l0.n2"),
                       ffn=make_part("ffn", "gated_mlp", name="l0.mlp", hidden=c.hidden_size, intermediate=40)),
-            make_part("block", "prenorm", mixer_norm=norm("l1.n1"), mixer=make_part("mixer", "toy-decay", name="l1", hidden=c.hidden_size, decay=c.decay),
+            make_part("block", "prenorm", mixer_norm=norm("l1.n1"),
+                      mixer=make_part("mixer", c.mixer, name="l1", hidden=c.hidden_size, decay=c.decay,
+                                      **({"declared": c.declared} if c.mixer == "toy-prefix-sum" else {})),
                       ffn_norm=norm("l1.n2"), ffn=make_part("ffn", "gated_mlp", name="l1.mlp", hidden=c.hidden_size, intermediate=24)),
         ]
         # layer 1 runs twice: shared weights, a state of its own at each place in the order
@@ -74,10 +134,12 @@ def build_toy():
                      schedule=[ScheduleEntry(1), ScheduleEntry(0), ScheduleEntry(1)])
 
     register_part("mixer", "toy-decay", DecayMixer)
+    register_part("mixer", "toy-prefix-sum", PrefixSumMixer)
     register_architecture("toy-decay-lm", ToyConfig, build)
 
     def cleanup():
         unregister_part("mixer", "toy-decay")
+        unregister_part("mixer", "toy-prefix-sum")
         unregister_architecture("toy-decay-lm")
     return cleanup
 
@@ -147,6 +209,51 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path):
         runner.release("x"); runner.create("z")
         out = runner.step([StepEntry("z", tokens["y"], list(range(17)))]).cpu().numpy()
         np.testing.assert_allclose(out, want["y"], rtol=2e-4, atol=2e-5)
+        runner.cache.check()
+    finally:
+        cleanup()
+
+
+@pytest.mark.parametrize("execution, declared", [("eager", True), ("eager", False), ("graph", True), ("graph", False)])
+def test_a_mixer_brings_a_step_array_of_its_own(tmp_path, execution, declared):
+    """A mixer defined here needs a list per step that the step function knows nothing of.  It declares it (or asks
+    for it at its first step), the step function carries it with its metadata, filled by the array's own code, and
+    under captured programs its launch value is part of a program's key, rounded up."""
+    import plain_llama as P
+    from runtime.engine import load_model, ModelRunner, StepEntry
+    cleanup = build_toy()
+    try:
+        raw = {"model_type": "toy-decay-lm", "vocab_size": 61, "hidden_size": 24, "decay": 1.0, "mixer": "toy-prefix-sum",
+               "declared": declared, "max_position_embeddings": 96, "rms_norm_eps": 1e-5}
+        from runtime.engine.loading import build_from_config_dict
+        from runtime.weights import write_model_folder
+        _, _, blueprint = build_from_config_dict(raw)
+        write_model_folder(tmp_path, raw, blueprint.tensor_specs(), seed=5, dtype=torch.float32)
+        cfg, w = P.read_folder(tmp_path)
+        model = load_model(tmp_path, dtype="float32")
+        assert any(type(a).__name__ == "RowsOfSegments" for a in model.step_arrays()) == declared
+        runner = ModelRunner(model, n_pages=16, page_size=8, max_requests=3, execution=execution)
+        tokens = {"x": np.random.default_rng(0).integers(0, 61, 38).tolist(), "y": np.random.default_rng(1).integers(0, 61, 25).tolist()}
+        want = {k: plain_toy(raw, w, v) for k, v in tokens.items()}
+        runner.create("x"); runner.create("y")
+        got, fed = {"x": [], "y": []}, {"x": 0, "y": 0}
+        plan = [[("x", 9), ("y", 2)], [("x", 1), ("y", 7)], [("y", 1)], [("x", 13), ("y", 1)], [("x", 7), ("y", 6)]] + [[("x", 1), ("y", 1)]] * 8
+        del SEEN[:]
+        for step in plan:
+            entries = [StepEntry(k, tokens[k][fed[k]:fed[k] + n], list(range(n))) for k, n in step]
+            out = runner.step(entries).cpu().numpy()
+            row = 0
+            for k, n in step:
+                got[k].append(out[row:row + n]); row += n; fed[k] += n
+        for k in tokens:
+            np.testing.assert_allclose(np.concatenate(got[k]), want[k], rtol=2e-4, atol=2e-5)
+        told = runner.report()
+        assert sum("RowsOfSegments" in a for a in told["step_arrays"]) == 1
+        assert len(SEEN) == len(plan)                                       # filled once a step, whoever asked
+        if execution == "eager":
+            assert all(value == true for value, true in SEEN)
+        else:
+            assert all(true <= value < 2 * true for value, true in SEEN) and told["replays"] >= 6
         runner.cache.check()
     finally:
         cleanup()

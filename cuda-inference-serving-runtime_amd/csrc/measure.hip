@@ -187,3 +187,119 @@ extern "C" int cisr_chain_phase(const void* W, const float* x, float* y, int N, 
     }
     return CISR_LAUNCH_CHECK();
 }
+
+// A whole decode step as ONE launch whose blocks meet inside the kernel, but only the blocks of one die (XCD) with each
+// other, through that die's L2: what `python -m runtime.measure one_launch` times against the step of 154 launches.
+// Blocks are dealt to the dies in turn (from a die that changes from launch to launch), so a grid of 8 n blocks puts n
+// on each; a block reads the number of its die from the hardware register, takes a ticket there, and the blocks of
+// the first `active` dies each run the step of a request of their own: 30 x (q/k/v, attention, output projection,
+// gate and up, down), every part a matrix-vector pass over that layer's weights with the traffic and the dependences of
+// the real kernels (activations of the part before: from L2, into LDS; a wave streams its contiguous share of the
+// rows, eight loads a lane in flight; lane sums meet; a store) and no arithmetic that means anything; attention reads
+// `kv16` 16-byte words of keys and values a layer.  Meetings: arrivals and polls are read-modify-writes without the
+// device-scope bit, which execute in the die's L2 (a poll adds a zero that the compiler cannot see, or it would turn
+// into a load that the compute unit's own cache answers for ever); what a block wrote before a meeting the others
+// read after it with device-scope loads, which pass the compute unit's cache and are answered by the same L2.
+// Bounded: after `spin_limit` polls a block sets words[1023] and its die's blocks leave at that meeting.
+// `words`: 1024 zeroed 32-bit words; `scratch`: 8 x 16384 floats.
+struct DieMeeting { unsigned* count; unsigned* flag; unsigned zero, blocks, limit, expected; };
+
+__device__ __forceinline__ bool die_meet(DieMeeting& m) {
+    __builtin_amdgcn_s_waitcnt(0);                       // this wave's stores are acknowledged by L2
+    __syncthreads();
+    __shared__ int gave_up;
+    if (threadIdx.x == 0) {
+        gave_up = 0;
+        __hip_atomic_fetch_add(m.count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        m.expected += m.blocks;
+        unsigned polls = 0;
+        while (__hip_atomic_fetch_add(m.count, m.zero, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < m.expected) {
+            if (++polls > m.limit) { *m.flag = 1u; gave_up = 1; break; }
+            __builtin_amdgcn_s_sleep(1);
+        }
+    }
+    __syncthreads();
+    return !gave_up;
+}
+
+__device__ __forceinline__ void die_pass(const float* x, int K, const read_word_t* W, int N, float* y, int rank, int blocks, float* lds) {
+    constexpr int NT = 512;
+    const int wave = threadIdx.x / 64, lane = threadIdx.x % 64, waves = NT / 64;
+    for (int i = threadIdx.x; i < K; i += NT) lds[i] = __hip_atomic_load(x + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    const int all = blocks * waves, me = rank * waves + wave;
+    const int r0 = (int)((long long)N * me / all), r1 = (int)((long long)N * (me + 1) / all);
+    const read_word_t* w = W + (size_t)r0 * (K / 8);
+    const int n16 = (r1 - r0) * (K / 8);
+    float acc = 0.f;
+    int c = lane;
+    for (; c + 7 * 64 < n16; c += 8 * 64) {
+        read_word_t v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = w[c + j * 64];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc += chain_bf(v[j].x, 1) * lds[(c + j) & 511] + chain_bf(v[j].y, 0) * lds[(c * 3 + j) & 511] + __uint_as_float(v[j].z ^ v[j].w) * 1e-30f;
+    }
+    for (; c < n16; c += 64) { const read_word_t v = w[c]; acc += chain_bf(v.x, 1) * lds[c & 511] + __uint_as_float(v.y ^ v.z ^ v.w) * 1e-30f; }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
+    if (lane < r1 - r0) y[r0 + lane] = acc;
+}
+
+__global__ void __launch_bounds__(512) one_launch_step_kernel(const read_word_t* __restrict__ weights, long long layer16, int layers, int H, int QKV, int I,
+                                                              const read_word_t* __restrict__ kv, long long kv16, float* scratch, unsigned* words,
+                                                              unsigned zero, int blocks, int active, unsigned spin_limit) {
+    extern __shared__ float lds[];
+    __shared__ int rank_here;
+    const int die = __builtin_amdgcn_s_getreg((3 << 11) | 20) & 15;      // bits 3:0 of the hardware register that names the die
+    if (die >= 8) return;
+    if (threadIdx.x == 0) rank_here = (int)__hip_atomic_fetch_add(words + 512 + die * 16, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    __syncthreads();
+    const int rank = rank_here;
+    if (die >= active || rank >= blocks) return;
+    DieMeeting m = {words + die * 16, words + 1023, zero, (unsigned)blocks, spin_limit, 0u};
+    float* res = scratch + (size_t)die * 16384, *q = res + 4096, *att = q + 4096, *act = att + 4096;
+    const read_word_t* kv_here = kv + (size_t)die * kv16 * layers;
+    for (int l = 0; l < layers; ++l) {
+        const read_word_t* W = weights + (size_t)l * layer16;
+        die_pass(res, H, W, QKV, q, rank, blocks, lds);
+        if (!die_meet(m)) return;
+        {   // attention: this block's share of the layer's keys and values, then its part of a result
+            read_word_t a = {0u, 0u, 0u, 0u};
+            const float q0 = __hip_atomic_load(q + threadIdx.x % QKV, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const read_word_t* mine = kv_here + (size_t)l * kv16;
+            for (long long i = (long long)rank * 512 + threadIdx.x; i < kv16; i += (long long)blocks * 512) a ^= mine[i];
+            if (threadIdx.x < 64 && rank * 64 + threadIdx.x < H) att[rank * 64 + threadIdx.x] = q0 + (float)(a.x ^ a.y ^ a.z ^ a.w) * 1e-30f;
+        }
+        if (!die_meet(m)) return;
+        W += (size_t)QKV * H / 8;
+        die_pass(att, H, W, H, res, rank, blocks, lds);
+        if (!die_meet(m)) return;
+        W += (size_t)H * H / 8;
+        die_pass(res, H, W, 2 * I, act, rank, blocks, lds);
+        if (!die_meet(m)) return;
+        W += (size_t)2 * I * H / 8;
+        die_pass(act, I, W, H, res, rank, blocks, lds);
+        if (!die_meet(m)) return;
+    }
+}
+
+// weights: bf16, `layers` x ((QKV + H + 2 I) H + H I) elements; kv: 8 x layers x kv16 16-byte words; blocks: 32 or 64 a die
+// (one or two a compute unit: all resident at once); H, I multiples of 8, at most 4096 floats a vector.
+extern "C" int cisr_one_launch_step(const void* weights, int layers, int H, int QKV, int I, const void* kv, long long kv16, void* scratch,
+                                    void* words, int blocks, int active, unsigned spin_limit, hipStream_t stream) {
+    if (layers <= 0) return 0;
+    if (!weights || !kv || !scratch || !words || (blocks != 32 && blocks != 64) || active < 1 || active > 8 || H % 8 || I % 8 ||
+        H <= 0 || I <= 0 || QKV <= 0 || H > 4096 || I > 4096 || QKV > 4096 || 2 * I > 4096 || kv16 < 0)
+        return (int)hipErrorInvalidValue;
+    int device = 0, per_unit = 0, units = 0;
+    const size_t lds_bytes = (size_t)(I > H ? I : H) * 4;
+    if (hipGetDevice(&device) != hipSuccess || hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess ||
+        hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_unit, one_launch_step_kernel, 512, lds_bytes) != hipSuccess ||
+        (long long)per_unit * units < 8ll * blocks)
+        return (int)hipErrorInvalidValue;
+    const long long layer16 = ((long long)(QKV + H + 2 * I) * H + (long long)H * I) / 8;
+    one_launch_step_kernel<<<8u * blocks, 512, lds_bytes, stream>>>((const read_word_t*)weights, layer16, layers, H, QKV, I, (const read_word_t*)kv, kv16,
+                                                                   (float*)scratch, (unsigned*)words, 0u, blocks, active, spin_limit);
+    return CISR_LAUNCH_CHECK();
+}

@@ -18,7 +18,8 @@ def _lib():
         p, i, ll = C.c_void_p, C.c_int, C.c_longlong
         for name, args in {"cisr_idle": [i, p], "cisr_stream_read": [p, ll, p, i, p],
                            "cisr_grid_meet": [p, p, i, i, i, C.c_uint, p],
-                           "cisr_chain_phase": [p, p, p, i, i, p, C.c_uint, p, p, i, p]}.items():
+                           "cisr_chain_phase": [p, p, p, i, i, p, C.c_uint, p, p, i, p],
+                           "cisr_one_launch_step": [p, i, i, i, i, p, ll, p, p, i, i, C.c_uint, p]}.items():
             fn = getattr(h, name)
             fn.argtypes, fn.restype = args, C.c_int
         _handle = h
@@ -67,3 +68,19 @@ def chain_phase(w, x, y, counters=None, wait=False):
     _check(_lib().cisr_chain_phase(_dev(w, "w"), x.data_ptr(), y.data_ptr(), n, k, None if cin is None else cin.data_ptr(), int(expect),
                                    None if cout is None else cout.data_ptr(), None if err is None else err.data_ptr(), int(bool(wait)),
                                    _stream()), "chain_phase")
+
+
+def one_launch_step(weights, layers, hidden, qkv, intermediate, kv, kv_words, scratch, words, blocks=32, active=8, spin_limit=200000):
+    """A mock decode step as ONE launch: the blocks of each die (XCD) meet inside the kernel through that die's L2, the
+    first `active` dies each run the step of a request of their own (30 x five matrix-vector passes with the traffic
+    of the real ones).  weights: bf16, layers x ((qkv + hidden + 2 intermediate) hidden + hidden intermediate)
+    elements; kv: 8 x layers x kv_words 16-byte words; scratch: 8 x 16384 floats; words: 1024 int32, zeroed before
+    every launch ([1023] is set when a block gave up waiting)."""
+    need = layers * ((qkv + hidden + 2 * intermediate) * hidden + hidden * intermediate)
+    if weights.dtype != torch.bfloat16 or weights.numel() < need or kv.numel() * kv.element_size() < 8 * layers * kv_words * 16:
+        raise KernelError("one_launch_step: weights or keys and values too small for the sizes")
+    if scratch.dtype != torch.float32 or scratch.numel() < 8 * 16384 or words.dtype != torch.int32 or words.numel() < 1024:
+        raise KernelError("one_launch_step: scratch of 8 x 16384 floats and 1024 int32 words")
+    _check(_lib().cisr_one_launch_step(_dev(weights, "weights"), int(layers), int(hidden), int(qkv), int(intermediate), _dev(kv, "kv"),
+                                       int(kv_words), scratch.data_ptr(), words.data_ptr(), int(blocks), int(active), int(spin_limit),
+                                       _stream()), "one_launch_step")

@@ -15,6 +15,8 @@
   hot_weights              decode steps with every layer sharing one layer's weights (the order of layers names one
                            layer for every place) against distinct layers: what weights that are already in a cache
                            are worth, the bound of anything that fetches weights ahead
+  one_launch               a mock decode step as ONE launch: the blocks of each die meet inside the kernel through
+                           that die's L2, a request a die (what a step fused into one kernel would cost at the least)
 """
 import argparse
 import json
@@ -335,6 +337,58 @@ def chain(args):
     return 0
 
 
+def one_launch(args):
+    """A decode step as one launch against the step of 154 launches: the mock of csrc/measure.hip (blocks of a die
+    meet inside the kernel through that die's L2; every die runs the step of a request of its own) at the sizes of
+    --model, with one die or all eight at work, 32 or 64 blocks a die, one row's keys a die or eight rows'.  What the
+    mock leaves out (norms, rotary embedding, softmax, the merge of split attention) would only add to its times."""
+    import statistics
+    import torch
+    from runtime import measure
+    from runtime.config import preset
+    dev = torch.device("cuda:0")
+    raw = preset(args.model)
+    H, I, L = raw["hidden_size"], raw["intermediate_size"], raw["num_hidden_layers"]
+    D = raw.get("head_dim") or H // raw["num_attention_heads"]
+    qkv = (raw["num_attention_heads"] + 2 * raw["num_key_value_heads"]) * D
+    context = 2048
+    row_words = context * raw["num_key_value_heads"] * D * 2 * 2 // 16           # keys and values of a layer, one row, 16-byte words
+    weights = torch.full((L * ((qkv + H + 2 * I) * H + H * I),), 0.01, dtype=torch.bfloat16, device=dev)
+    kv = torch.ones(8 * L * 8 * row_words * 4, dtype=torch.int32, device=dev)
+    scratch = torch.zeros(8 * 16384, device=dev)
+    words = torch.zeros(1024, dtype=torch.int32, device=dev)
+    stream = torch.cuda.Stream()
+    points = {}
+    for blocks in (32, 64):
+        for active in (1, 8):
+            for rows in (1, 8):
+                def body():
+                    words.zero_()
+                    measure.one_launch_step(weights, L, H, qkv, I, kv, rows * row_words, scratch, words, blocks=blocks, active=active)
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.stream(stream):
+                    body(); stream.synchronize()
+                    if int(words[1023]):
+                        raise SystemExit("a block gave up waiting at a meeting")
+                    with torch.cuda.graph(graph, stream=stream):
+                        body()
+                    times = []
+                    for _ in range(12):
+                        stream.synchronize()
+                        t0 = time.perf_counter()
+                        graph.replay()
+                        stream.synchronize()
+                        times.append(time.perf_counter() - t0)
+                    if int(words[1023]):
+                        raise SystemExit("a block gave up waiting at a meeting")
+                points[f"{blocks}_blocks_a_die_{active}_dies_{rows}_rows_each"] = round(statistics.median(times) * 1e3, 4)
+    print(json.dumps({"metric": "milliseconds of a mock decode step run as one launch, blocks meeting inside their die", "unit": "ms",
+                      "value": points["32_blocks_a_die_8_dies_1_rows_each"], "higher_is_better": False, "n_gpus": 1, "model": args.model,
+                      "layers": L, "weights_mb_a_layer": round(((qkv + H + 2 * I) * H + H * I) * 2 / 2 ** 20, 2),
+                      "keys_and_values_mb_a_layer_and_row": round(row_words * 16 / 2 ** 20, 2), "ms_a_step": points}))
+    return 0
+
+
 def reread(args):
     """GB/s of the read-only kernel over a buffer that it reads again and again (20 or more passes in one captured
     graph, the median of five replays), by the buffer's size."""
@@ -415,7 +469,7 @@ def hot_weights(args):
 
 def main(argv=None):
     ap = argparse.ArgumentParser(prog="python -m runtime.measure")
-    ap.add_argument("workload", choices=["floor", "attention", "attention_forms", "decode_attention_shapes", "chain", "reread", "hot_weights"])
+    ap.add_argument("workload", choices=["floor", "attention", "attention_forms", "decode_attention_shapes", "chain", "reread", "hot_weights", "one_launch"])
     ap.add_argument("--chain-layers", type=int, default=30, help="chain: layers of five products each (30: 113 MB of weights; 240: 904 MB, "
                                                                  "more than the memory-side cache holds)")
     ap.add_argument("--model", default="smollm2-135m", help="floor: the preset whose decode step the floor is priced for")
@@ -424,7 +478,7 @@ def main(argv=None):
     args = ap.parse_args(argv)
     return {"floor": launch_floor, "attention": prompt_attention, "attention_forms": attention_forms,
             "decode_attention_shapes": decode_attention_shapes, "chain": chain, "reread": reread,
-            "hot_weights": hot_weights}[args.workload](args)
+            "hot_weights": hot_weights, "one_launch": one_launch}[args.workload](args)
 
 
 if __name__ == "__main__":

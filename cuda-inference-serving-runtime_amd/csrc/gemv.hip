@@ -6,7 +6,7 @@
 // in turn (chunk c to lane c mod 64), the products are packed-bf16 dot instructions with float sums (v_dot2_f32_bf16),
 // the lanes' sums meet in a butterfly of lane exchanges, and a lane finishes each activation row.  No partial tiles
 // in LDS, no barrier after the prologue, no second kernel; the first loads of W are issued before the prologue's
-// barrier, because they do not depend on the activations.
+// barrier (right behind the activations' own loads), because they do not depend on the activations.
 //
 // Prologue, once a block (256 threads), into LDS as packed bf16 rows [M][K]:
 //   plain   A is bf16: copied;
@@ -79,11 +79,15 @@ gemv_kernel(SkinnyArgs p, int units, int per_wave) {
         }
     };
     gv_u32x4 wcur[R][CB];
-    load_batch(unit_of(0), 0, wcur);                  // on its way while the activations are prepared
 
     // ---- prologue: the activation rows as packed bf16 in LDS.  Every batch of loads is issued before the first of
     // them is used, for all rows at once, with clamped addresses instead of branches (a branch around a load makes it a
-    // trip to memory of its own: eight rows one after the other took 6 us)
+    // trip to memory of its own: eight rows one after the other took 6 us).  The first batch of W is asked for right
+    // behind the first batch of the activations and before these are used: loads return in the order they were asked
+    // for, so the activations (a few KB out of L2) must not stand behind W's first bytes (16 MB over all waves, out of
+    // memory), and W must be on its way while the activations are turned into operands.  Measured on an MI355X with time
+    // marks in the kernel (norm + gate/up of the 1.7B sizes): with W asked for first the block's barrier was passed
+    // 3.9 us after the kernel's start, 2.4 us of them with nothing more asked of memory.
     if constexpr (NORM) {
         const int words4 = K / 4;
         const float* xrow[M];
@@ -98,8 +102,8 @@ gemv_kernel(SkinnyArgs p, int units, int per_wave) {
 #pragma unroll
         for (int m = 0; m < M; ++m) sq[m] = 0.f;
         constexpr int G = M <= 2 ? 4 : 2;                // 16-byte words of a row a thread takes per batch
-        for (int k0 = 0; k0 < words4; k0 += GEMV_THREADS * G) {
-            gv_f32x4 nv[G], xv[M][G];
+        gv_f32x4 nv[G], xv[M][G];
+        auto ask = [&](int k0) {
 #pragma unroll
             for (int g = 0; g < G; ++g) {
                 const int k4 = k0 + g * GEMV_THREADS + tid, kk = k4 < words4 ? k4 : 0;
@@ -107,6 +111,8 @@ gemv_kernel(SkinnyArgs p, int units, int per_wave) {
 #pragma unroll
                 for (int m = 0; m < M; ++m) xv[m][g] = *(const gv_f32x4*)(xrow[m] + kk * 4);
             }
+        };
+        auto use = [&](int k0) {
 #pragma unroll
             for (int g = 0; g < G; ++g) {
                 const int k4 = k0 + g * GEMV_THREADS + tid;
@@ -121,7 +127,11 @@ gemv_kernel(SkinnyArgs p, int units, int per_wave) {
                     }
                 }
             }
-        }
+        };
+        ask(0);
+        load_batch(unit_of(0), 0, wcur);
+        use(0);
+        for (int k0 = GEMV_THREADS * G; k0 < words4; k0 += GEMV_THREADS * G) { ask(k0); use(k0); }
 #pragma unroll
         for (int m = 0; m < M; ++m) {
             const float total = wave_sum(sq[m]);
@@ -131,9 +141,9 @@ gemv_kernel(SkinnyArgs p, int units, int per_wave) {
         const int per_row = K / 8, n_items = M * per_row;
         const int D = p.merge_dim, nh = p.merge_heads;
         constexpr int G = MSPL <= 4 ? 2 : 1;             // items a thread merges per batch
-        for (int i0 = 0; i0 < n_items; i0 += GEMV_THREADS * G) {
-            gv_u32x4 po[G][MSPL];
-            float ms[G][MSPL], ls[G][MSPL];
+        gv_u32x4 po[G][MSPL];
+        float ms[G][MSPL], ls[G][MSPL];
+        auto ask = [&](int i0) {
 #pragma unroll
             for (int g = 0; g < G; ++g) {
                 const int item = i0 + g * GEMV_THREADS + tid, it = item < n_items ? item : 0;
@@ -145,6 +155,8 @@ gemv_kernel(SkinnyArgs p, int units, int per_wave) {
                     ms[g][sp] = p.part_ml[(base + sp) * 2]; ls[g][sp] = p.part_ml[(base + sp) * 2 + 1];
                 }
             }
+        };
+        auto use = [&](int i0) {
 #pragma unroll
             for (int g = 0; g < G; ++g) {
                 const int item = i0 + g * GEMV_THREADS + tid;
@@ -171,17 +183,23 @@ gemv_kernel(SkinnyArgs p, int units, int per_wave) {
                     (gv_u32x4){pack_bf16x2(num[0] * inv, num[1] * inv), pack_bf16x2(num[2] * inv, num[3] * inv),
                                pack_bf16x2(num[4] * inv, num[5] * inv), pack_bf16x2(num[6] * inv, num[7] * inv)};
             }
-        }
+        };
+        ask(0);
+        load_batch(unit_of(0), 0, wcur);
+        use(0);
+        for (int i0 = GEMV_THREADS * G; i0 < n_items; i0 += GEMV_THREADS * G) { ask(i0); use(i0); }
     } else {
         const int n_items = M * nchunks;
         constexpr int G = 4;
-        for (int i0 = 0; i0 < n_items; i0 += GEMV_THREADS * G) {
-            gv_u32x4 v[G];
+        gv_u32x4 v[G];
+        auto ask = [&](int i0) {
 #pragma unroll
             for (int g = 0; g < G; ++g) {
                 const int item = i0 + g * GEMV_THREADS + tid, it = item < n_items ? item : 0;
                 v[g] = *(const gv_u32x4*)((const bf16_t*)p.A + (size_t)min(it / nchunks, p.M - 1) * p.lda + (it % nchunks) * 8);
             }
+        };
+        auto use = [&](int i0) {
 #pragma unroll
             for (int g = 0; g < G; ++g) {
                 const int item = i0 + g * GEMV_THREADS + tid;
@@ -189,7 +207,11 @@ gemv_kernel(SkinnyArgs p, int units, int per_wave) {
                 const int row = item / nchunks;
                 *(gv_u32x4*)(a_lds + row * words + (item % nchunks) * 4) = row < p.M ? v[g] : (gv_u32x4){0u, 0u, 0u, 0u};
             }
-        }
+        };
+        ask(0);
+        load_batch(unit_of(0), 0, wcur);
+        use(0);
+        for (int i0 = GEMV_THREADS * G; i0 < n_items; i0 += GEMV_THREADS * G) { ask(i0); use(i0); }
     }
     __syncthreads();
 
@@ -335,10 +357,21 @@ static int gemv_launch_one(const SkinnyArgs& a, int units, hipStream_t stream) {
         hipError_t e = hipFuncSetAttribute((const void*)gemv_kernel<M, NORM, EPI, TC, MSPL>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return (int)e;
     }
-    // Blocks: with units enough, exactly two a compute unit (eight waves), so that every compute unit streams the same
-    // number of bytes (384 blocks on 256 units leave half of them with twice the work of the others); with fewer units
-    // than that many waves, one unit a wave.
-    const int waves = gemv_compute_units() * 8;
+    // Blocks: with units enough, two, three or four a compute unit (8, 12 or 16 waves), whichever leaves the waves the
+    // most equal numbers of units (the kernel is as long as its busiest wave: 3,072 rotary pairs are two units for half
+    // of 2,048 waves and one for the others, a third of the time idle, but one unit for each of 3,072; 384 blocks on
+    // 256 compute units leave half of them with twice the work of the others), the fewest of equals; with fewer units
+    // than eight waves a compute unit, one unit a wave.  Measured on an MI355X (a decode step of one request, 8 layers):
+    // always 8 waves 0.443 ms at the 1.7B sizes, always 12 0.427, always 16 0.432; 1.037, 1.041 and 1.020 at the 8B sizes.
+    const int cus = gemv_compute_units();
+    int waves = cus * 8;
+    if (units >= waves) {
+        long long best = -1;
+        for (int w = 8; w <= 16; w += 4) {
+            const long long all = (long long)cus * w, busiest = (units + all - 1) / all * all;   // unit-times the launch lasts
+            if (best < 0 || busiest < best) { best = busiest; waves = (int)all; }
+        }
+    }
     const int per_wave = (units + waves - 1) / waves;
     const int blocks = units >= waves ? waves / GEMV_WAVES : (units + GEMV_WAVES - 1) / GEMV_WAVES;
     gemv_kernel<M, NORM, EPI, TC, MSPL><<<blocks, GEMV_THREADS, lds, stream>>>(a, units, per_wave);

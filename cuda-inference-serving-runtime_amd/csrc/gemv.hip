@@ -368,6 +368,7 @@ static int gemv_launch_one(const SkinnyArgs& a, int units, hipStream_t stream) {
     if (units >= waves) {
         long long best = -1;
         for (int w = 8; w <= 16; w += 4) {
+            if (w > 8 && (size_t)(w / GEMV_WAVES) * lds > 160 * 1024) break;                     // (that many blocks' rows do not fit a unit's LDS)
             const long long all = (long long)cus * w, busiest = (units + all - 1) / all * all;   // unit-times the launch lasts
             if (best < 0 || busiest < best) { best = busiest; waves = (int)all; }
         }

@@ -14,7 +14,7 @@ had passed, which no later query reads.
 """
 from dataclasses import dataclass, field
 
-from .pages import CacheGroup, KVNeed, OutOfPages, StateNeed
+from .pages import CacheGroup, OutOfPages
 from .state import StateSlots
 
 

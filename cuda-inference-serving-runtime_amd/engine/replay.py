@@ -19,7 +19,6 @@ import json
 import sys
 from pathlib import Path
 
-import numpy as np
 import torch
 
 from .loading import load_model

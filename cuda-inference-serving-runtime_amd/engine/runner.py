@@ -18,7 +18,7 @@ from typing import List, Sequence
 import numpy as np
 import torch
 
-from ..cache import CacheManager, OutOfPages
+from ..cache import CacheManager
 from ..kernels import ops
 from .context import Batch, GroupView, StepContext, Workspace
 

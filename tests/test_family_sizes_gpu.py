@@ -41,7 +41,8 @@ def test_family_layer_sizes(family_folders, name, dtype):
     runner = ModelRunner(model, n_pages=24, page_size=16, max_requests=4)
     runner.create("a"); runner.create("b")
     got = {"a": [], "b": []}
-    plan = [[("a", 100), ("b", 3)], [("a", 30), ("b", 1)], [("a", 1), ("b", 66)]] + [[("a", 1)]] * 19
+    # (portions, then six steps of two single tokens and thirteen of one: the products of one and of two rows)
+    plan = [[("a", 100), ("b", 3)], [("a", 30), ("b", 1)], [("a", 1), ("b", 60)]] + [[("a", 1), ("b", 1)]] * 6 + [[("a", 1)]] * 13
     fed = {"a": 0, "b": 0}
     seqs = {"a": a, "b": b}
     for step in plan:

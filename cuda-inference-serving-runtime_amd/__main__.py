@@ -38,13 +38,17 @@ def main(argv=None):
     parser.add_argument("--max-active", type=int, default=8)
     parser.add_argument("--overlap", action="store_true",
                         help="launch each step before the tokens of the step before are read (same tokens, less idle GPU)")
+    parser.add_argument("--plugin", action="append", default=[], metavar="MODULE",
+                        help="import this module first: it may register parts or an architecture of its own (may be given more than once)")
     parser.add_argument("--report", action="store_true",
                         help="add the step function's counters and memory (steps, programs captured and replayed, "
                              "bytes of workspace, scratch, staging and cache) to the output")
     args = parser.parse_args(argv)
 
     from .config import read_config_json
+    from .engine.loading import import_plugins
     from .engine.scheduler import Engine, Request
+    import_plugins(args.plugin)
 
     tokenizer, raw = None, {}
     execution = "graph" if args.execution == "graph" else "eager"

@@ -22,6 +22,15 @@ def parse_dtype(dtype):
         raise ValueError(f"dtype {dtype!r} is not one of {sorted(DTYPES)}") from None
 
 
+def import_plugins(names):
+    """Import the modules `names`: a module that registers parts or an architecture of its own at import
+    (runtime.register_part, runtime.register_architecture) thereby makes them known to the entry points, which choose
+    the model class by config.json.  The modules come from the caller's command line, never from a model folder."""
+    import importlib
+    for name in names or ():
+        importlib.import_module(name)
+
+
 def build_from_config_dict(raw):
     arch = architecture_of(raw)
     config = arch.config_cls.from_dict(raw)

@@ -21,7 +21,7 @@ from pathlib import Path
 
 import torch
 
-from .loading import load_model
+from .loading import import_plugins, load_model
 from .runner import ModelRunner, StepEntry
 
 PAGE_SIZE = 16          # divides 64, so a request rounded up to 64 tokens never holds more than its share
@@ -71,7 +71,10 @@ def main(argv=None):
     parser.add_argument("--page-size", type=int, default=PAGE_SIZE, help="tokens a cache page (a power of two that divides 64)")
     parser.add_argument("--execution", choices=["eager", "graph"], default="eager",
                         help="eager: kernels launched one by one; graph: every step as a captured program")
+    parser.add_argument("--plugin", action="append", default=[], metavar="MODULE",
+                        help="import this module first: it may register parts or an architecture of its own (may be given more than once)")
     args = parser.parse_args(argv)
+    import_plugins(args.plugin)
 
     def echo(text):
         print(text, flush=True)

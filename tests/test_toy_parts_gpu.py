@@ -1105,3 +1105,97 @@ def test_scheduler_generates_with_a_model_of_two_page_groups(tmp_path, execution
         assert max(step["active"] for step in engine.trace) <= 3
     finally:
         cleanup()
+
+
+PLUGIN = '''"""An architecture of a module of its own: the framework's parts under other config.json keys."""
+from dataclasses import dataclass
+
+from runtime import make_part, register_architecture
+from runtime.models import Model
+from runtime.parts import LMHead, TokenEmbedding
+
+
+@dataclass(frozen=True)
+class KeysConfig:
+    width: int
+    depth: int
+    n_heads: int
+    n_kv: int
+    head: int
+    ffn: int
+    vocab: int
+    theta: float
+    eps: float
+    max_len: int
+
+    @classmethod
+    def from_dict(cls, raw):
+        return cls(*(raw[k] for k in ("width", "depth", "n_heads", "n_kv", "head", "ffn", "vocab", "theta", "eps", "max_len")))
+
+
+def build(c):
+    def norm(name):
+        return make_part("norm", "rmsnorm", name=name, dim=c.width, eps=c.eps)
+    position = make_part("position", "rotary", head_dim=c.head, theta=c.theta, max_positions=c.max_len)
+    layers = []
+    for i in range(c.depth):
+        p = f"model.layers.{i}"
+        layers.append(make_part(
+            "block", "prenorm", mixer_norm=norm(p + ".input_layernorm"),
+            mixer=make_part("mixer", "attention", name=p + ".self_attn", hidden=c.width, heads=c.n_heads, kv_heads=c.n_kv,
+                            head_dim=c.head, position=position),
+            ffn_norm=norm(p + ".post_attention_layernorm"),
+            ffn=make_part("ffn", "gated_mlp", name=p + ".mlp", hidden=c.width, intermediate=c.ffn)))
+    return Model(c, TokenEmbedding("model.embed_tokens", c.vocab, c.width), layers, norm("model.norm"),
+                 LMHead("lm_head", c.vocab, c.width), max_positions=c.max_len, vocab_size=c.vocab)
+
+
+register_architecture(["other-keys-lm"], KeysConfig, build)
+'''
+
+
+def test_an_architecture_of_a_module_of_its_own_runs_through_both_programs(tmp_path):
+    """A module outside the package registers an architecture at import; `--plugin` names it to the command line and to
+    the replay program, which then choose it by config.json as they choose the framework's own.  Without the option the
+    registry's error names the architecture it does not know."""
+    import json, os, subprocess, sys
+    from pathlib import Path
+    import plain_llama as P
+    from runtime.config import unregister_architecture
+    from runtime.engine.loading import build_from_config_dict, import_plugins
+    from runtime.weights import write_model_folder
+    root = Path(__file__).resolve().parent.parent
+    (tmp_path / "other_keys_plugin.py").write_text(PLUGIN)
+    raw = {"model_type": "other-keys-lm", "width": 72, "depth": 2, "n_heads": 6, "n_kv": 2, "head": 16, "ffn": 120, "vocab": 211,
+           "theta": 5e4, "eps": 1e-6, "max_len": 128}
+    sys.path.insert(0, str(tmp_path))
+    try:
+        import_plugins(["other_keys_plugin"])
+        _, _, blueprint = build_from_config_dict(raw)
+        folder = tmp_path / "model"
+        write_model_folder(folder, raw, blueprint.tensor_specs(), seed=9, dtype=torch.float32)
+    finally:
+        sys.path.remove(str(tmp_path))
+        sys.modules.pop("other_keys_plugin", None)
+        unregister_architecture("other-keys-lm")
+    _, w = P.read_folder(folder)
+    cfg = dict(num_hidden_layers=2, hidden_size=72, num_attention_heads=6, num_key_value_heads=2, head_dim=16, rope_theta=5e4,
+               rms_norm_eps=1e-6, tie_word_embeddings=False)
+    env = dict(os.environ, PYTHONPATH=os.pathsep.join([str(root), str(tmp_path)]))
+    base = [sys.executable, "-m", "runtime", "--checkpoint", str(folder), "--dtype", "float32", "--tokens", "5,6,7", "--max-new-tokens", "4",
+            "--execution", "eager"]
+    proc = subprocess.run(base + ["--plugin", "other_keys_plugin"], capture_output=True, text=True, timeout=300, env=env, cwd=str(tmp_path))
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert json.loads(proc.stdout)["requests"][0]["generated"] == P.greedy(cfg, w, [5, 6, 7], 4)
+    proc = subprocess.run(base, capture_output=True, text=True, timeout=300, env=env, cwd=str(tmp_path))
+    assert proc.returncode != 0 and "other-keys-lm" in proc.stderr
+    tokens = np.random.default_rng(3).integers(0, 211, 40).tolist()
+    trace = [{"step": 0, "entries": [{"id": "a", "tokens": tokens[:33], "want": [32]}], "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": tokens[33:], "want": list(range(7))}], "end": ["a"]}]
+    proc = subprocess.run([sys.executable, str(root / "bin" / "trace_run"), "--model", str(folder), "--dtype", "float32", "--out", str(tmp_path / "out"),
+                           "--max-tokens", "64", "--plugin", "other_keys_plugin"], input="".join(json.dumps(t) + "\n" for t in trace),
+                          capture_output=True, text=True, timeout=300, env=env, cwd=str(tmp_path))
+    assert proc.returncode == 0 and proc.stdout.split() == ["done", "0", "done", "1"], proc.stderr[-2000:]
+    want = P.forward(cfg, w, tokens)
+    got = np.concatenate([np.fromfile(tmp_path / "out" / f"{i}.f32", dtype="<f4").reshape(-1, 211) for i in (0, 1)])
+    np.testing.assert_allclose(got, want[32:], rtol=2e-4, atol=2e-5)

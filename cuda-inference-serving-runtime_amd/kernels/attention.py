@@ -33,6 +33,10 @@ class AttentionTuning:
     # segments get a launch of their own instead, which splits their keys over blocks
     split_single_from: int = 4096
     rows_launch: Optional[tuple] = None   # (wavefronts a block, blocks along the keys) of decode rows
+    # A step of single tokens whose keys are not split runs a block for every (row, key head).  From this many blocks on
+    # (several rounds of what the compute units hold at once) the rows are listed longest first, so that the launch does
+    # not end with the blocks of a long row alone
+    order_rows_from: int = 1024
 
 
 DEFAULT_TUNING = AttentionTuning()
@@ -87,6 +91,25 @@ class SingleRows:
         if value:
             own = [int(batch.first_row[s]) for s, c in enumerate(batch.counts) if c == 1]
             out[:len(own)] = own
+
+
+@dataclass(frozen=True)
+class RowsLongestFirst:
+    """Step array: the rows of a step of one-token segments by the number of keys they attend to, most first (rows of
+    equal length in their own order), then the padding rows (which have no keys: zeros are written for them).  Blocks
+    are handed out in this order."""
+
+    def words(self, rows, segments):
+        return rows
+
+    def launch_value(self, batch):
+        return None
+
+    def fill(self, out, batch, value):
+        out[:] = np.arange(len(out))
+        if batch.decode_only:
+            order = np.argsort(-np.asarray(batch.starts, dtype=np.int64), kind="stable")
+            out[:len(order)] = np.asarray(batch.first_row, dtype=np.int64)[order]
 
 
 @dataclass(frozen=True)
@@ -283,7 +306,10 @@ def paged_attention(ctx, q, q_row_stride, kcache, vcache, view, out, heads, kv_h
                 ops.attention_mfma(*common, None, fused, workspace, waves, merge=False)
                 return workspace[0], workspace[1], fused
         workspace = _split_workspace(ctx, rows, heads, splits, head_dim) if splits > 1 else None
-        ops.attention_mfma(*common, None, splits, workspace, waves)
+        order = None
+        if splits == 1 and rows * chunks >= tuning.order_rows_from:
+            order = ctx.step_array(RowsLongestFirst())[0][:rows]
+        ops.attention_mfma(*common, None, splits, workspace, waves, row_ids=order)
         return None
     singles = SingleRows(tuning.split_single_from)
     single_rows, n_single = ctx.step_array(singles)

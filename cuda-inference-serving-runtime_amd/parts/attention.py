@@ -40,7 +40,7 @@ class PagedAttention(Mixer):
         return kernel.kernel_units(self.head_dim, dtype)
 
     def step_arrays(self):
-        return [kernel.SingleRows(self.tuning.split_single_from)]
+        return [kernel.SingleRows(self.tuning.split_single_from), kernel.RowsLongestFirst()]
 
     def cache_need(self):
         return KVNeed(self.kv_heads, self.head_dim, self.window) if self.own_kv else None

@@ -11,7 +11,7 @@ import pytest
 import torch
 
 import plain_llama as P
-from conftest import ROOT, TINY, random_tokens
+from conftest import ROOT, TINY, assert_close, plain_logits, random_tokens
 
 pytestmark = pytest.mark.gpu
 
@@ -569,6 +569,38 @@ def test_fork_shares_a_prefix_and_copies_on_write(folders):
     assert_close(out[6:], plain_logits(folders["a"], prefix + tail_b)[21:], "float32", "fork")
     r.release("src"); r.release("dst"); r.cache.check()
     assert r.cache.free_pages() == [12]
+
+
+@pytest.mark.parametrize("execution", ["eager", "graph"])
+def test_decode_rows_handed_out_longest_first_give_the_same_logits(folders, execution):
+    """From many blocks on, an unsplit decode launch lists its rows longest first (told here to do so always): the same
+    logits bit for bit as in the rows' own order, for requests of very different lengths, also under captured programs
+    with padding rows."""
+    from runtime.engine import load_model, ModelRunner, StepEntry
+    from conftest import tune_attention
+    name = "a"
+    V = TINY[name]["vocab_size"]
+    seqs = {k: random_tokens(700 + i, n, V) for i, (k, n) in enumerate(zip("uvwxy", (90, 12, 47, 90, 9)))}
+    outs = []
+    for order_from in (1, 10 ** 9):
+        model = load_model(folders[name], dtype="bfloat16")
+        tune_attention(model, order_rows_from=order_from, rows_launch=(4, 1))
+        runner = ModelRunner(model, n_pages=64, page_size=8, max_requests=8, execution=execution)
+        for k, toks in seqs.items():
+            runner.create(k)
+            runner.step([StepEntry(k, toks[:-6], [])])
+        got = []
+        for t in range(6):
+            live = [k for k in seqs if not (t >= 3 and k == "v")]                  # five rows (padded to eight), then four
+            got.append(runner.step([StepEntry(k, [seqs[k][len(seqs[k]) - 6 + t]], [0]) for k in live]).float().cpu())
+        outs.append(got)
+        assert any("RowsLongestFirst" in a for a in runner.report()["step_arrays"])
+    for with_order, without in zip(*outs):
+        assert torch.equal(with_order, without)
+    ref = {k: plain_logits(folders[name], seqs[k]) for k in seqs}
+    first = outs[0][0].numpy()
+    for row, k in enumerate(seqs):
+        assert_close(first[row:row + 1], ref[k][len(seqs[k]) - 6:len(seqs[k]) - 5], "bfloat16", f"request {k}")
 
 
 def test_command_line(folders, tmp_path):

@@ -1,7 +1,7 @@
 """Host-side metadata of a step: the attention task lists and the sizes that captured programs pad to."""
 import numpy as np
 
-from runtime.kernels.attention import SingleRows, TileTasks, fill_tasks
+from runtime.kernels.attention import RowsLongestFirst, SingleRows, TileTasks, fill_tasks
 from runtime.engine.context import Batch
 from runtime.engine.runner import _bucket
 
@@ -88,3 +88,19 @@ def test_step_arrays_of_the_attention_kernels():
     batch.launch_values[singles] = 0
     tiles.fill(tasks.reshape(-1), batch, None)
     assert sorted(tasks[tasks[:, 0] >= 0][:, 0].tolist()) == [0, 1, 1, 2, 3]
+
+
+def test_rows_of_a_decode_step_longest_first():
+    """The order in which an unsplit decode launch hands out its blocks: rows by keys, most first, rows of equal
+    length in their own order, then the padding rows of a captured program; a mixed step lists every row in place."""
+    order = RowsLongestFirst()
+    starts = [5, 900, 17, 900, 0, 300]
+    batch = Batch([1] * 6, starts, np.arange(6, dtype=np.int32), True, {})
+    assert order.launch_value(batch) is None and order.words(8, 8) == 8
+    out = np.full(8, -9, dtype=np.int32)
+    order.fill(out, batch, None)
+    assert out.tolist() == [1, 3, 5, 2, 0, 4, 6, 7]
+    mixed = Batch([1, 4], [50, 0], np.array([0, 1], dtype=np.int32), False, {})
+    out = np.full(5, -9, dtype=np.int32)
+    order.fill(out, mixed, None)
+    assert out.tolist() == [0, 1, 2, 3, 4]

@@ -1,6 +1,6 @@
 """Paged attention as one call: which kernel, in which form and launch shape, and the step metadata it wants.
 
-`paged_attention` is what a mixer calls.  bfloat16 with a head size in steps of 8 and pages of a power of two >= 4
+`paged_attention` is what a mixer calls.  bfloat16 with a head size in steps of 8 and pages of a power of two >= 8
 runs on the matrix cores (one block per row for decode steps, tiles of rows from a task list otherwise); everything
 else runs the exact row-wise kernel.  The rules that pick a form or a launch shape are plain functions of sizes
 (`rows_launch`, `prompt_form`, `rowwise_splits`), each settled by measurements on an MI355X that its comments quote;

@@ -770,7 +770,7 @@ def gemm_merged(partials, heads, dim, w, out, residual):
 
 
 def mfma_attention_supported(dtype, dim, page_size):
-    return (dtype == torch.bfloat16 and dim % 8 == 0 and dim <= 256 and page_size >= 4
+    return (dtype == torch.bfloat16 and dim % 8 == 0 and dim <= 256 and page_size >= 8
             and page_size & (page_size - 1) == 0)
 
 

@@ -432,7 +432,7 @@ def square_modes(dim):
 
 
 @pytest.mark.parametrize("heads, kv_heads, dim, page_size", [
-    (4, 2, 16, 4), (6, 6, 24, 8), (9, 3, 64, 16), (8, 1, 128, 64), (2, 2, 256, 4), (5, 5, 40, 16), (32, 1, 64, 16), (20, 1, 32, 8)])
+    (4, 2, 16, 8), (6, 6, 24, 8), (9, 3, 64, 16), (8, 1, 128, 64), (2, 2, 256, 8), (5, 5, 40, 16), (32, 1, 64, 16), (20, 1, 32, 8)])
 def test_attention_mfma_rows(ops, heads, kv_heads, dim, page_size):
     """Decode form: single rows at scattered positions, every split count, including more splits than 32-key steps."""
     qt, kt, vt, tables, rows = paged_case(heads, kv_heads, dim, page_size, [17, 7, 1, 130, 333], torch.bfloat16, seed=dim + heads)
@@ -454,7 +454,7 @@ def test_attention_mfma_rows(ops, heads, kv_heads, dim, page_size):
         assert (got[[1, 2, 4]] == 9.0).all()
 
 
-@pytest.mark.parametrize("heads, kv_heads, dim, page_size", [(9, 3, 64, 16), (4, 2, 32, 4), (8, 2, 128, 32), (6, 6, 24, 8)])
+@pytest.mark.parametrize("heads, kv_heads, dim, page_size", [(9, 3, 64, 16), (4, 2, 32, 8), (8, 2, 128, 32), (6, 6, 24, 8)])
 def test_attention_mfma_rows_over_many_steps(ops, heads, kv_heads, dim, page_size):
     """Decode form with many 32-key steps a wave (long contexts, few or no splits): the loop that keeps several steps'
     loads in flight, with wave counts and splits that give a wave 1 to 35 steps, a far key that stands out, and a
@@ -488,7 +488,7 @@ def portion_case(heads, kv_heads, dim, page_size, plan, seed):
 
 
 @pytest.mark.parametrize("heads, kv_heads, dim, page_size", [
-    (4, 2, 16, 4), (6, 6, 24, 8), (9, 3, 64, 16), (8, 2, 128, 16), (3, 3, 256, 64), (32, 1, 64, 16), (7, 7, 48, 16)])
+    (4, 2, 16, 8), (6, 6, 24, 8), (9, 3, 64, 16), (8, 2, 128, 16), (3, 3, 256, 64), (32, 1, 64, 16), (7, 7, 48, 16)])
 def test_attention_mfma_tiles(ops, heads, kv_heads, dim, page_size):
     """Prompt portions: rows of a portion attend to the cached prefix and causally to
     the portion itself; portions of 1, 2 and many rows, starting at and off page edges."""
@@ -1228,11 +1228,12 @@ def test_kernels_refuse_what_they_cannot_take(ops):
         run_rowwise(ops, rnd(1, 2, 258), rnd(1, 2, 4, 258), rnd(1, 2, 258, 4), torch.zeros(1, 1, dtype=torch.int32, device=DEV), [(0, 0)], 4)
     with pytest.raises(KernelError, match="divide"):
         run_rowwise(ops, rnd(1, 3, 16), rnd(1, 2, 4, 16), rnd(1, 2, 16, 4), torch.zeros(1, 1, dtype=torch.int32, device=DEV), [(0, 0)], 4)
-    with pytest.raises(KernelError, match="not supported"):   # the matrix-core kernel takes bf16, head sizes in steps of 8, pages 4, 8, 16, ...
+    with pytest.raises(KernelError, match="not supported"):   # the matrix-core kernel takes bf16, head sizes in steps of 8, pages of 8, 16, ... keys
         ops.attention_mfma(rnd(1, 2 * 12, dtype=torch.bfloat16), 24, rnd(1, 2, 4, 12, dtype=torch.bfloat16), rnd(1, 2, 12, 4, dtype=torch.bfloat16),
                            torch.zeros(1, 1, dtype=torch.int32, device=DEV), torch.zeros(1, dtype=torch.int32, device=DEV),
                            torch.zeros(1, dtype=torch.int32, device=DEV), torch.empty(1, 24, dtype=torch.bfloat16, device=DEV), 2, 2, 12, 4, None, 1.0)
     assert not ops.mfma_attention_supported(torch.bfloat16, 64, 3) and not ops.mfma_attention_supported(torch.float32, 64, 16)
+    assert not ops.mfma_attention_supported(torch.bfloat16, 64, 4) and ops.mfma_attention_supported(torch.bfloat16, 64, 8)   # (a lane takes 8 keys of a value page at once)
     with pytest.raises(KernelError):
         ops.rmsnorm(rnd(2, 8), rnd(9), torch.empty(2, 8, device=DEV), 1e-5)
     with pytest.raises(KernelError):

@@ -326,32 +326,62 @@ static int launch_bf16_swiglu(const bf16_t* A, int lda, const bf16_t* W, int ldw
     return CISR_LAUNCH_CHECK();
 }
 
-extern "C" int cisr_gemm_bf16_swiglu(const void* A, int lda, const void* W, int ldw, void* C, int ldc, int M, int N, int K,
-                                     int dual_off, hipStream_t stream) {
+// `tile`: 0 picks by the rule below; TM * 100 + TN * 10 + WM asks for that block tile (a tile that is not built: an error).
+extern "C" int cisr_gemm_bf16_swiglu_tile(const void* A, int lda, const void* W, int ldw, void* C, int ldc, int M, int N, int K,
+                                          int dual_off, int tile, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
     if (K <= 0 || K % 8 || lda % 8 || ldw % 8 || ((uintptr_t)A) % 16 || ((uintptr_t)W) % 16 || dual_off < N)
         return (int)hipErrorInvalidValue;
     const bf16_t* a = (const bf16_t*)A; const bf16_t* w = (const bf16_t*)W;
     auto blocks = [&](int bm, int bn) { return (long long)((M + bm - 1) / bm) * ((2 * N + bn - 1) / bn); };
-    if (blocks(128, 128) >= 512) return launch_bf16_swiglu<4, 4, 64>(a, lda, w, ldw, (bf16_t*)C, ldc, M, N, K, dual_off, stream);
-    if (blocks(128, 64) >= 512) return launch_bf16_swiglu<4, 2, 64>(a, lda, w, ldw, (bf16_t*)C, ldc, M, N, K, dual_off, stream);
-    if (blocks(64, 64) < 256) return launch_bf16_swiglu<1, 2, 64>(a, lda, w, ldw, (bf16_t*)C, ldc, M, N, K, dual_off, stream);
-    return launch_bf16_swiglu<2, 2, 64>(a, lda, w, ldw, (bf16_t*)C, ldc, M, N, K, dual_off, stream);
+    if (tile == 0) {
+        if (blocks(128, 128) >= 512) tile = 442;
+        else if (blocks(128, 64) >= 512) tile = 422;
+        else if (blocks(64, 64) < 256) tile = 122;
+        else tile = 222;
+    }
+#define SWIGLU_TILE(TM, TN, WM) \
+    case TM * 100 + TN * 10 + WM: return launch_bf16_swiglu<TM, TN, 64, WM>(a, lda, w, ldw, (bf16_t*)C, ldc, M, N, K, dual_off, stream);
+    switch (tile) {
+        SWIGLU_TILE(1, 2, 2) SWIGLU_TILE(2, 2, 2) SWIGLU_TILE(4, 2, 2) SWIGLU_TILE(4, 4, 2)
+    }
+#undef SWIGLU_TILE
+    return (int)hipErrorInvalidValue;
+}
+
+extern "C" int cisr_gemm_bf16_swiglu(const void* A, int lda, const void* W, int ldw, void* C, int ldc, int M, int N, int K,
+                                     int dual_off, hipStream_t stream) {
+    return cisr_gemm_bf16_swiglu_tile(A, lda, W, ldw, C, ldc, M, N, K, dual_off, 0, stream);
 }
 
 // Tile choice: the largest tile that still gives the 256 compute units a few blocks each; when even 64 x 64 leaves
 // most of them idle (a portion of a few hundred rows against small weights), 32 x 64 and 32 x 32 (measured on an
 // MI355X at 128 and 512 rows: 10-30 % faster there, slower from about one block a compute unit on).
-extern "C" int cisr_gemm_bf16(const void* A, int lda, const void* W, int ldw, void* C, int ldc, const float* R,
-                              int ldr, int M, int N, int K, int out_dtype, hipStream_t stream) {
+// `tile`: 0 picks by this rule; TM * 100 + TN * 10 + WM asks for that block tile (a tile that is not built: an error).
+extern "C" int cisr_gemm_bf16_tile(const void* A, int lda, const void* W, int ldw, void* C, int ldc, const float* R,
+                                   int ldr, int M, int N, int K, int out_dtype, int tile, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
     if (K <= 0 || (R && out_dtype != DT_F32)) return (int)hipErrorInvalidValue;
     const bf16_t* a = (const bf16_t*)A; const bf16_t* w = (const bf16_t*)W;
     auto blocks = [&](int bm, int bn) { return (long long)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
-    if (M <= 32) return launch_bf16<1, 2, 64>(a, lda, w, ldw, C, ldc, R, ldr, M, N, K, out_dtype, stream);
-    if (blocks(128, 128) >= 512) return launch_bf16<4, 4, 64>(a, lda, w, ldw, C, ldc, R, ldr, M, N, K, out_dtype, stream);
-    if (blocks(128, 64) >= 512) return launch_bf16<4, 2, 64>(a, lda, w, ldw, C, ldc, R, ldr, M, N, K, out_dtype, stream);
-    if (blocks(32, 64) <= 64) return launch_bf16<1, 1, 64>(a, lda, w, ldw, C, ldc, R, ldr, M, N, K, out_dtype, stream);
-    if (blocks(64, 64) < 256) return launch_bf16<1, 2, 64>(a, lda, w, ldw, C, ldc, R, ldr, M, N, K, out_dtype, stream);
-    return launch_bf16<2, 2, 64>(a, lda, w, ldw, C, ldc, R, ldr, M, N, K, out_dtype, stream);
+    if (tile == 0) {
+        if (M <= 32) tile = 122;
+        else if (blocks(128, 128) >= 512) tile = 442;
+        else if (blocks(128, 64) >= 512) tile = 422;
+        else if (blocks(32, 64) <= 64) tile = 112;
+        else if (blocks(64, 64) < 256) tile = 122;
+        else tile = 222;
+    }
+#define GEMM_TILE(TM, TN, WM) \
+    case TM * 100 + TN * 10 + WM: return launch_bf16<TM, TN, 64, WM>(a, lda, w, ldw, C, ldc, R, ldr, M, N, K, out_dtype, stream);
+    switch (tile) {
+        GEMM_TILE(1, 1, 2) GEMM_TILE(1, 2, 2) GEMM_TILE(2, 2, 2) GEMM_TILE(4, 2, 2) GEMM_TILE(4, 4, 2)
+    }
+#undef GEMM_TILE
+    return (int)hipErrorInvalidValue;
+}
+
+extern "C" int cisr_gemm_bf16(const void* A, int lda, const void* W, int ldw, void* C, int ldc, const float* R,
+                              int ldr, int M, int N, int K, int out_dtype, hipStream_t stream) {
+    return cisr_gemm_bf16_tile(A, lda, W, ldw, C, ldc, R, ldr, M, N, K, out_dtype, 0, stream);
 }

@@ -51,6 +51,8 @@ def _declare(h):
         "cisr_gemm_f32": [p, i, p, i, p, i, p, i, i, i, i, p],
         "cisr_gemm_bf16": [p, i, p, i, p, i, p, i, i, i, i, i, p],
         "cisr_gemm_bf16_swiglu": [p, i, p, i, p, i, i, i, i, i, p],
+        "cisr_gemm_bf16_tile": [p, i, p, i, p, i, p, i, i, i, i, i, i, p],
+        "cisr_gemm_bf16_swiglu_tile": [p, i, p, i, p, i, i, i, i, i, i, p],
         "cisr_gemm_skinny_bf16": [p, i, p, i, p, i, p, i, i, i, i, i, i, p, f, p, p],
         "cisr_qkv_rope_skinny": [p, i, p, i, p, i, i, i, p, f, p, p, p, p, p, p, i, i, i, i, i, p],
         "cisr_attn_merge": [p, p, p, i, i, i, i, p, p],

@@ -1122,6 +1122,33 @@ def test_gemm_bf16(ops, M, N, K):
     np.testing.assert_allclose(f64(out), want + f64(r), rtol=1e-4, atol=1e-4 * math.sqrt(K))
 
 
+@pytest.mark.parametrize("tile", [112, 122, 222, 422, 442])
+def test_gemm_bf16_every_block_tile_alone(ops, tile):
+    """The rule picks a block tile by the shape; here each built tile (rows / 16 a wave x 100, columns / 16 a wave x 10,
+    waves along the rows) multiplies shapes that no tile divides, with and without the residual, and the activation
+    where the tile pairs column tiles."""
+    stream = torch.cuda.current_stream().cuda_stream
+    for M, N, K in ((150, 200, 136), (70, 1000, 72), (333, 96, 520)):
+        a, w, r = rnd(M, K, dtype=torch.bfloat16, seed=1), rnd(N, K, dtype=torch.bfloat16, seed=2), rnd(M, N, seed=3)
+        want = f64(a) @ f64(w).T
+        out = r.clone()
+        assert ops.lib().cisr_gemm_bf16_tile(a.data_ptr(), K, w.data_ptr(), K, out.data_ptr(), N, out.data_ptr(), N, M, N, K,
+                                             0, tile, stream) == 0
+        np.testing.assert_allclose(f64(out), want + f64(r), rtol=1e-4, atol=1e-4 * math.sqrt(K))
+        half = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+        assert ops.lib().cisr_gemm_bf16_tile(a.data_ptr(), K, w.data_ptr(), K, half.data_ptr(), N, None, 0, M, N, K, 1, tile, stream) == 0
+        np.testing.assert_allclose(f64(half), want, rtol=1e-2, atol=1e-2 * math.sqrt(K))
+        if tile in (122, 222, 422, 442) and N % 2 == 0:
+            H = N // 2
+            act = torch.empty(M, H, dtype=torch.bfloat16, device=DEV)
+            assert ops.lib().cisr_gemm_bf16_swiglu_tile(a.data_ptr(), K, w.data_ptr(), K, act.data_ptr(), H, M, H, K, H, tile, stream) == 0
+            g, u = f64(torch.from_numpy(want[:, :H]).bfloat16()), f64(torch.from_numpy(want[:, H:]).bfloat16())
+            np.testing.assert_allclose(f64(act), g / (1 + np.exp(-g)) * u, rtol=2e-2, atol=2e-2)
+    a, w = rnd(40, 64, dtype=torch.bfloat16), rnd(48, 64, dtype=torch.bfloat16)
+    out = torch.empty(40, 48, device=DEV)
+    assert ops.lib().cisr_gemm_bf16_tile(a.data_ptr(), 64, w.data_ptr(), 64, out.data_ptr(), 48, None, 0, 40, 48, 64, 0, 999, stream) != 0
+
+
 def test_gemm_strided_rows_and_bad_operands(ops):
     from runtime.kernels.ops import KernelError
     big = rnd(9, 50, dtype=torch.bfloat16)

@@ -80,8 +80,10 @@ gemv_kernel(SkinnyArgs p, int units, int per_wave) {
 #pragma unroll
         for (int c = 0; c < CB; ++c) {
             const int chunk = lane + WAVE * (b * CB + c), at = chunk < nchunks ? chunk * 8 : 0;
-            w[0][c] = *(const gv_u32x4*)(w0 + at);
-            if (R == 2) w[1][c] = *(const gv_u32x4*)(w1 + at);
+            // non-temporal: the weights are read once a step and the caches need not keep them (a decode step of
+            // one row at the 8B sizes 1.008 -> 0.937 ms, at the 1.7B sizes 0.420 -> 0.413)
+            w[0][c] = __builtin_nontemporal_load((const gv_u32x4*)(w0 + at));
+            if (R == 2) w[1][c] = __builtin_nontemporal_load((const gv_u32x4*)(w1 + at));
         }
     };
     gv_u32x4 wcur[R][CB];

@@ -33,6 +33,7 @@ class AttentionTuning:
     # segments get a launch of their own instead, which splits their keys over blocks
     split_single_from: int = 4096
     rows_launch: Optional[tuple] = None   # (wavefronts a block, blocks along the keys) of decode rows
+    stream_loads: Optional[bool] = None   # decode rows read keys and values with non-temporal loads (None: by the rule)
     # A step of single tokens whose keys are not split runs a block for every (row, key head).  From this many blocks on
     # (several rounds of what the compute units hold at once) the rows are listed longest first, so that the launch does
     # not end with the blocks of a long row alone
@@ -247,6 +248,21 @@ def rows_launch(blocks, span, heads_per_chunk, head_dim):
     return waves, splits
 
 
+def rows_stream_loads(blocks, span, waves, splits, head_dim):
+    """Whether the decode kernel launched as `blocks` x `splits` blocks of `waves` wavefronts reads keys and values with
+    non-temporal loads (no block reads them again; the caches then do not keep them).  Measured inside decode steps
+    of the three sizes at 448 to 32,000 keys and 1 to 64 rows: blocks of four waves never lose by them and gain up to
+    11 % of the whole step (64 rows at 8k keys of the 8B sizes 4.64 -> 4.12 ms, 32 rows at 2k of the 1.7B sizes 1.379 ->
+    1.275).  Blocks of eight waves (head sizes up to 64) gain 2-3 % of the step where they fill the GPU and a wave has
+    little more than two 32-key steps (8 and 16 rows at 2k of the 135M sizes, 4 rows at 8k), and lose 2-11 % where a
+    wave walks a longer run of keys (four steps and more: 32 and 64 rows at 2k to 32k) or the blocks are few (+4-6 %
+    below 96 blocks)."""
+    if head_dim > 64 or waves == 4:               # (larger heads run eight waves as four)
+        return True
+    steps = -(-span // 32)
+    return blocks * splits >= 160 and 2 * steps <= 5 * waves * splits
+
+
 def fused_merge_splits(splits, rows, accepts):
     """How many of the `splits` blocks along a decode row's keys the product that follows may merge itself
     (`accepts(n)` says whether it takes n), or None: then the merge kernel runs.  That product merges 2, 4 or 8
@@ -297,19 +313,26 @@ def paged_attention(ctx, q, q_row_stride, kcache, vcache, view, out, heads, kv_h
     group = heads // kv_heads
     heads_per_chunk = min(group, 16)
     chunks = kv_heads * -(-group // heads_per_chunk)
+
+    def stream(blocks, waves, splits):
+        if tuning.stream_loads is not None:
+            return tuning.stream_loads
+        return rows_stream_loads(blocks, span, waves, splits, head_dim)
+
     if ctx.decode_only:
         waves, splits = tuning.rows_launch or rows_launch(rows * chunks, span, heads_per_chunk, head_dim)
         if splits > 1 and defer_merge is not None:
             fused = fused_merge_splits(splits, rows, defer_merge)
             if fused is not None:
                 workspace = _split_workspace(ctx, rows, heads, fused, head_dim, torch.bfloat16, "attn.part_o16")
-                ops.attention_mfma(*common, None, fused, workspace, waves, merge=False)
+                ops.attention_mfma(*common, None, fused, workspace, waves, merge=False,
+                                   stream_loads=stream(rows * chunks, waves, fused))
                 return workspace[0], workspace[1], fused
         workspace = _split_workspace(ctx, rows, heads, splits, head_dim) if splits > 1 else None
         order = None
         if splits == 1 and rows * chunks >= tuning.order_rows_from:
             order = ctx.step_array(RowsLongestFirst())[0][:rows]
-        ops.attention_mfma(*common, None, splits, workspace, waves, row_ids=order)
+        ops.attention_mfma(*common, None, splits, workspace, waves, row_ids=order, stream_loads=stream(rows * chunks, waves, splits))
         return None
     singles = SingleRows(tuning.split_single_from)
     single_rows, n_single = ctx.step_array(singles)
@@ -317,7 +340,8 @@ def paged_attention(ctx, q, q_row_stride, kcache, vcache, view, out, heads, kv_h
         # the decoded tokens of this mixed step: a launch of their own that splits their keys
         waves, splits = tuning.rows_launch or rows_launch(n_single * chunks, span, heads_per_chunk, head_dim)
         workspace = _split_workspace(ctx, n_single, heads, splits, head_dim) if splits > 1 else None
-        ops.attention_mfma(*common, None, splits, workspace, waves, row_ids=single_rows[:n_single])
+        ops.attention_mfma(*common, None, splits, workspace, waves, row_ids=single_rows[:n_single],
+                           stream_loads=stream(n_single * chunks, waves, splits))
     form = prompt_form(rows, ctx.n_segments, span, heads, kv_heads, head_dim, view.page_size, tuning)
     kind, item_tiles, halves = form
     tasks, _ = ctx.step_array(TileTasks(rows_per_tile_of(form, heads, kv_heads), singles))

@@ -676,7 +676,7 @@ def qkv_rope(a, w, q_out, positions, slots, cos, sin, kcache, vcache, heads, kv_
 
 def attention_mfma(q, q_row_stride, kcache, vcache, tables, seg_of_row, positions, out, heads, kv_heads, dim,
                    page_size, window, scale, tasks=None, splits=1, workspace=None, waves=4, block_tiles=False,
-                   item_tiles=1, row_ids=None, merge=True, key_groups=1):
+                   item_tiles=1, row_ids=None, merge=True, key_groups=1, stream_loads=False):
     """Matrix-core attention (bf16).  tasks int32 [n, 4] = (segment, first row, rows, 0) runs tiles of
     prompt rows: one tile of 16/GC rows a block whose waves share the keys (with item_tiles=2, head sizes up to
     64: 32/GC rows, two item tiles a wave), or with `block_tiles` (head sizes up to 128) one tile of
@@ -687,7 +687,8 @@ def attention_mfma(q, q_row_stride, kcache, vcache, tables, seg_of_row, position
     the rows it lists are computed and written (negative entries are skipped): the decode rows of a mixed step.
     `merge` False (rows mode with splits > 1): the partial outputs are left unmerged in the workspace, whose first
     buffer is then bfloat16, for gemm_merged; `out` is not written.  `key_groups` 2 (block_tiles 32): a block is two
-    halves that take the even and the odd 32-key steps of its items and merge at the end."""
+    halves that take the even and the odd 32-key steps of its items and merge at the end.  `stream_loads` (rows mode):
+    keys and values are read with non-temporal loads, which the caches do not keep."""
     rows = out.shape[0]
     if not mfma_attention_supported(out.dtype, dim, page_size):
         raise KernelError(f"attention_mfma: head size {dim} / page size {page_size} / dtype {out.dtype} not supported")
@@ -740,7 +741,8 @@ def attention_mfma(q, q_row_stride, kcache, vcache, tables, seg_of_row, position
               _dev(vcache, "vcache", None, (pages, kv_heads, dim, page_size)), _dev(tables, "tables", torch.int32),
               tables.shape[1], tp, n_tasks, _dev(seg_of_row, "seg_of_row", torch.int32, (rows,)),
               _dev(positions, "positions", torch.int32, (rows,)), _dev(out, "out", None, (rows, heads * dim)), po, pm,
-              heads, kv_heads, dim, page_size.bit_length() - 1, int(window or 0), float(scale), int(splits), mode, int(waves),
+              heads, kv_heads, dim, page_size.bit_length() - 1, int(window or 0), float(scale), int(splits),
+              11 if mode == 1 and stream_loads else mode, int(waves),
               int(mode == 1 and splits > 1 and not merge), _stream()), "attention_mfma")
     if mode == 1 and splits > 1 and merge:
         _check(lib().cisr_attn_merge(po, pm, out.data_ptr(), n_tasks, heads, dim, int(splits), tp, _stream()), "attention_merge")

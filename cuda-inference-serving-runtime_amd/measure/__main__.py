@@ -191,7 +191,7 @@ def decode_attention_shapes(args):
     import torch
     from runtime.config import preset
     from runtime.kernels import ops
-    from runtime.kernels.attention import rows_launch
+    from runtime.kernels.attention import rows_launch, rows_stream_loads
     dev, P = torch.device("cuda:0"), args.page_size
     points, losses = {}, []
     for name in ("smollm2-135m", "smollm2-1.7b", "llama-3-8b"):
@@ -216,14 +216,16 @@ def decode_attention_shapes(args):
                 out = torch.empty(B, heads * D, device=dev).bfloat16()
                 blocks = B * kv * -(-group // per_chunk)
                 pick = tuple(rows_launch(blocks, C, per_chunk, D))
-                shapes = {(w, n) for w in (4, 8) for n in (1, 2, 4, 8, 16, 32) if (n == 1 or n * 32 <= C) and blocks * n <= 16384} | {pick}
+                pick += (rows_stream_loads(blocks, C, pick[0], pick[1], D),)
+                shapes = {(w, n, nt) for w in (4, 8) for n in (1, 2, 4, 8, 16, 32) for nt in (False, True)
+                          if (n == 1 or n * 32 <= C) and blocks * n <= 16384} | {pick}
                 us = {}
-                for waves, splits in sorted(shapes):
+                for waves, splits, stream_loads in sorted(shapes):
                     ws = (torch.empty(B * heads * splits * D, device=dev), torch.empty(B * heads * splits * 2, device=dev))
 
                     def run(i):
                         ops.attention_mfma(q, heads * D, ks[i], vs[i], tables, seg, pos, out, heads, kv, D, P, None, 1 / math.sqrt(D),
-                                           None, splits, ws, waves)
+                                           None, splits, ws, waves, stream_loads=stream_loads)
                     calls = max(copies, 4)
                     for i in range(copies):
                         run(i)
@@ -240,15 +242,15 @@ def decode_attention_shapes(args):
                         graph.replay()
                         torch.cuda.synchronize()
                         times.append((time.perf_counter() - t0) / calls * 1e6)
-                    us[(waves, splits)] = sorted(times)[1]
+                    us[(waves, splits, stream_loads)] = sorted(times)[1]
                 best = min(us, key=us.get)
                 loss = us[pick] / us[best] - 1
                 losses.append(loss)
-                label = lambda shape: f"{shape[0]} waves x {shape[1]}"
+                label = lambda shape: f"{shape[0]} waves x {shape[1]}" + (" nt" if shape[2] else "")
                 points[f"{name}_{B}x{C}"] = {"pick": label(pick), "pick_us": round(us[pick], 1), "best": label(best),
                                              "best_us": round(us[best], 1), "loss": round(loss, 3)}
                 print(f"{name:13s} {B:3d} rows x {C:5d} keys  pick {label(pick):13s} {us[pick]:7.1f} us   best {label(best):13s} {us[best]:7.1f} us   "
-                      + "  ".join(f"{w}x{n}: {v:.1f}" for (w, n), v in sorted(us.items())), file=sys.stderr, flush=True)
+                      + "  ".join(f"{w}x{n}{'nt' if nt else ''}: {v:.1f}" for (w, n, nt), v in sorted(us.items())), file=sys.stderr, flush=True)
     print(json.dumps({"metric": "loss of the rule that picks the decode attention launch shape against the best shape of each point",
                       "unit": "fraction", "n_gpus": 1, "value": round(max(losses), 3), "higher_is_better": False,
                       "mean": round(sum(losses) / len(losses), 4), "points": points}))

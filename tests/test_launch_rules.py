@@ -3,7 +3,7 @@ measurements settled them (profiles/prompt_attention_forms_and_the_rule_that_pic
 profiles/decode_attention_launch_shapes_and_the_rule_that_picks.txt), so that a change of a rule shows."""
 import pytest
 
-from runtime.kernels.attention import fused_merge_splits, prompt_form, rows_launch
+from runtime.kernels.attention import fused_merge_splits, prompt_form, rows_launch, rows_stream_loads
 
 
 @pytest.mark.parametrize("heads, kv_heads, dim, rows, form", [
@@ -41,6 +41,21 @@ def test_prompt_attention_form_needs_long_portions_and_pages_of_eight_keys():
 ])
 def test_decode_attention_launch_at_measured_points(blocks, keys, group, dim, launch):
     assert tuple(rows_launch(blocks, keys, group, dim)) == launch
+
+
+@pytest.mark.parametrize("blocks, keys, group, dim, streams", [
+    (24, 2048, 3, 64, True),           # eight requests of the 135M sizes: 192 blocks of eight waves, one step a wave
+    (3, 2048, 3, 64, False),           # one request: few blocks
+    (192, 2048, 3, 64, False),         # 64 requests unsplit: a wave walks eight steps
+    (24, 8192, 3, 64, False),
+    (12, 8192, 3, 64, True),           # 4 requests at 8k: 21 splits, a step and a half a wave
+    (2048, 2048, 1, 64, True),         # four waves a block: always
+    (8, 8192, 4, 128, True),           # large heads: always
+    (512, 512, 4, 128, True),
+])
+def test_decode_attention_streams_keys_and_values_at_measured_points(blocks, keys, group, dim, streams):
+    waves, splits = rows_launch(blocks, keys, group, dim)
+    assert rows_stream_loads(blocks, keys, waves, splits, dim) is streams
 
 
 @pytest.mark.parametrize("splits, rows, fused", [

@@ -152,6 +152,18 @@ def test_decode_rows_with_sixteen_and_thirty_two_splits(heads, kv_heads, D, laun
     check(got, want, f"{heads}/{kv_heads}x{D}, {launch[0]} waves x {launch[1]} splits")
 
 
+@pytest.mark.parametrize("heads, kv_heads, D", SHAPES)
+@pytest.mark.parametrize("launch", [(4, 1), (8, 4), (4, 8)])
+def test_decode_rows_read_with_non_temporal_loads_give_the_same_bits(heads, kv_heads, D, launch):
+    """The two kinds of load differ in what the caches keep, not in what arrives: the outputs are equal bit for bit."""
+    from runtime.kernels.attention import AttentionTuning
+    step = Step([1] * 5, [4099, 2047, 31, 700, 0])
+    plain, want = attend(step, heads, kv_heads, D, seed=sum(launch), tuning=AttentionTuning(rows_launch=launch, stream_loads=False))
+    streamed, _ = attend(step, heads, kv_heads, D, seed=sum(launch), tuning=AttentionTuning(rows_launch=launch, stream_loads=True))
+    check(streamed, want, f"{heads}/{kv_heads}x{D}, {launch[0]} waves x {launch[1]} splits, non-temporal loads")
+    assert torch.equal(plain, streamed)
+
+
 @pytest.mark.parametrize("heads, kv_heads, D, start, form", [
     (9, 3, 64, 0, ("square", 2, 2)),
     (32, 32, 64, 0, ("square", 3, 1)),

@@ -34,10 +34,11 @@ class AttentionTuning:
     split_single_from: int = 4096
     rows_launch: Optional[tuple] = None   # (wavefronts a block, blocks along the keys) of decode rows
     stream_loads: Optional[bool] = None   # decode rows read keys and values with non-temporal loads (None: by the rule)
-    # A step of single tokens whose keys are not split runs a block for every (row, key head).  From this many blocks on
-    # (several rounds of what the compute units hold at once) the rows are listed longest first, so that the launch does
-    # not end with the blocks of a long row alone
-    order_rows_from: int = 1024
+    # A step of single tokens whose keys are not split runs a block for every (row, key head), the key heads of a row
+    # side by side.  From this many blocks on (more than one block a compute unit) the rows are listed longest first,
+    # so that the launch does not end with the blocks of a long row alone (64 rows of 228 to 2,304 keys at the 1.7B
+    # sizes: 126.6 -> 119.7 us, what 64 rows of their mean length take; 128 rows at the 135M sizes 36.3 -> 34.2)
+    order_rows_from: int = 320
 
 
 DEFAULT_TUNING = AttentionTuning()

@@ -246,6 +246,12 @@ def rows_launch(blocks, span, heads_per_chunk, head_dim):
         target = 768 if head_dim <= 64 else 512
         per = target // blocks if head_dim <= 64 and blocks > 256 else -(-target // blocks)
         splits = int(max(1, min(steps // (waves * 4), per, 64)))
+    if waves == 8 and blocks >= 48 and span >= (16384 if blocks < 96 else 6144):
+        # Eight-wave blocks whose waves walk long runs of keys: four waves and more blocks along the keys instead, about
+        # 1,536 in all, which read with non-temporal loads (`rows_stream_loads`).  Decode steps of the 135M sizes: 32
+        # rows at 8k keys 1.865 -> 1.779 ms, 64 rows 2.798 -> 2.755; at 32k 16, 32 and 64 rows 2.695 -> 2.625, 4.713 ->
+        # 4.455 and 8.539 -> 8.107; 16 rows at 8k gain nothing.
+        waves, splits = 4, int(min(max(1, 1536 // blocks), 16, max(1, steps // 16)))
     return waves, splits
 
 

@@ -233,6 +233,11 @@ def rows_launch(blocks, span, heads_per_chunk, head_dim):
         # At most 32 splits: a single row of 8 key heads at 8k takes 23 us with 32 and 30 with 64.
         room = 256 if waves == 8 else 512
         splits = int(max(1, min(steps // waves, room // blocks, 32)))
+        if splits > 16 and steps < 2 * waves * splits:
+            # more than 16 splits only with two steps a wave and more: their merge costs more than a second step (one
+            # and four rows at 8k keys of the 135M sizes: decode steps of 0.829 and 0.901 ms with 31 and 21 splits,
+            # 0.796 and 0.877 with 16; at 32k 32 and 21 splits stay, 16 would take 1.33 against 1.02 ms)
+            splits = max(16, steps // (2 * waves))
     elif head_dim <= 64 and 140 <= blocks <= 256:
         # enough rows to give most compute units one block of eight waves, and no more than one each: the
         # keys are not split and no merge follows (9-11 % faster than four waves and three or four splits at

@@ -33,6 +33,10 @@ def test_prompt_attention_form_needs_long_portions_and_pages_of_eight_keys():
     (24, 2048, 3, 64, (8, 8)),         # eight
     (192, 2048, 3, 64, (8, 1)),        # 64: one block of eight waves a compute unit, no split
     (24, 8192, 3, 64, (8, 10)),        # eight waves at long contexts too
+    (3, 8192, 3, 64, (8, 16)),         # one request at 8k: 16 splits of two steps a wave, not 31 of one
+    (12, 8192, 3, 64, (8, 16)),
+    (3, 32768, 3, 64, (8, 32)),        # at 32k a wave has steps enough for 32 splits
+    (12, 32768, 3, 64, (8, 21)),
     (96, 8192, 3, 64, (4, 16)),        # but from 16 rows on four waves and about 1,536 blocks in all (non-temporal loads)
     (192, 32768, 3, 64, (4, 8)),
     (48, 8192, 3, 64, (8, 5)),         # 16 rows at 8k stay

@@ -20,16 +20,18 @@ static int launch_rows(const SkinnyArgs& a, int blocks, bool norm, int epi, int 
 
 static bool aligned16(const void* p) { return ((uintptr_t)p) % 16 == 0; }
 
-// One or two rows against weights of 4 MB and more: the matrix-vector kernel (gemv.hip).  Measured on an MI355X, decode
+// Up to four rows against weights of 4 MB and more: the matrix-vector kernel (gemv.hip).  Measured on an MI355X, decode
 // steps in captured programs (ms a step without it -> with it): 1.7B sizes, 8 layers, one request 0.537 -> 0.441, two
-// 0.571 -> 0.506; 8B sizes, 8 layers, 1.239 -> 1.066 and 1.254 -> 1.130.  Four rows lose (0.608 -> 0.636, 1.325 ->
-// 1.448: every row more is another read of LDS and another set of dot instructions for every 16 bytes of W), and so do
-// the small weights of the 135M sizes at any number of rows (one request 0.670 -> 0.751: there a product is its
+// 0.571 -> 0.506; 8B sizes, 8 layers, 1.239 -> 1.066 and 1.254 -> 1.130.  Three and four rows lost while it read the
+// weights with ordinary loads (0.608 -> 0.636, 1.325 -> 1.448) and win with non-temporal ones (1.7B sizes 0.604 ->
+// 0.568 and 0.609 -> 0.578, 8B sizes 1.315 -> 1.236 and 1.322 -> 1.241); six and eight rows lose by half (0.673 ->
+// 1.026, 1.311 -> 1.780: every row more is another read of LDS and another set of dot instructions for every 16 bytes
+// of W), and so do the small weights of the 135M sizes at any number of rows (one request 0.670 -> 0.751: there a product is its
 // prologue and epilogue, and the narrow kernel's are shorter; a form of this kernel for such weights that is a single
 // trip to memory, a unit a wave, no LDS and no barrier, came to the narrow kernel's times within 3 %, one request 0.668
 // -> 0.684, and lost with two, 0.682 -> 0.799: not kept).  The most rows it is given and the least bytes can be
 // set (cisr_gemv_set: rows 0 switches it off), for measurements of one kernel against the other and for tests.
-static int gemv_rows = 2;
+static int gemv_rows = 4;
 static long long gemv_bytes = 4ll << 20;
 extern "C" void cisr_gemv_set(int rows, long long least_bytes) {
     gemv_rows = rows < 0 ? 0 : rows > GEMV_MAX_ROWS ? GEMV_MAX_ROWS : rows;

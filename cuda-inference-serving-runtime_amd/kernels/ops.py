@@ -443,7 +443,7 @@ def wide_ok(m, w, swiglu=False, after_norm=False):
     `after_norm`: the rows are the output of an RMSNorm, which the other kernel would fuse (it then reads the
     float residual and the norm's weights for every 16 rows of W, which costs it more than bf16 rows do)."""
     n, k = w.shape
-    if gemv_ok(m, n, k):   # one or two rows against large weights: the matrix-vector kernel takes them
+    if gemv_ok(m, n, k):   # up to four rows against large weights: the matrix-vector kernel takes them
         return False
     least = WIDE_MIN_BYTES_FEW_ROWS if m <= 16 else WIDE_MIN_BYTES if m <= 32 else WIDE_MIN_BYTES_MANY_ROWS
     if m <= 16 and n < 16 * _compute_units(w.device) and k >= 4096:
@@ -458,11 +458,11 @@ def wide_ok(m, w, swiglu=False, after_norm=False):
     return _wide_plan(m, n // 2 if swiglu else n, k, swiglu) >= 0
 
 
-GEMV_ROWS, GEMV_MIN_BYTES = 2, 4 << 20
+GEMV_ROWS, GEMV_MIN_BYTES = 4, 4 << 20
 
 
 def gemv_ok(m, n, k):
-    """Whether a product of m rows with weights [n, k] runs the matrix-vector kernel (one or two rows against weights
+    """Whether a product of m rows with weights [n, k] runs the matrix-vector kernel (up to four rows against weights
     of 4 MB and more with an inner size of at least 1024: a wave owns whole rows of the weights; see csrc/gemv.hip
     and the measurements in csrc/gemm_skinny.hip).  The weight-streaming entry points choose it themselves; callers ask only to know that
     the wide kernel and its separate norm are not wanted."""

@@ -163,11 +163,11 @@ def test_which_products_take_this_kernel(ops):
     assert not ops.gemv_ok(8, 64, 16384)                                                            # eight rows of it do not fit LDS
     assert ops.gemv_ok(4, 64, 16384)
     assert not ops.wide_ok(8, w)
-    ops.set_gemv()              # the engine's rule: one or two rows, weights of 4 MB and more
+    ops.set_gemv()              # the engine's rule: up to four rows, weights of 4 MB and more
     try:
         assert ops.gemv_ok(1, 2048, 2048) and ops.gemv_ok(2, 6144, 4096) and ops.gemv_ok(1, 49152, 2048)
         assert not ops.gemv_ok(1, 49152, 576)          # rows of W too short to fill a wave's lanes twice
-        assert not ops.gemv_ok(3, 6144, 4096) and not ops.gemv_ok(1, 3072, 576)
+        assert ops.gemv_ok(3, 6144, 4096) and ops.gemv_ok(4, 6144, 4096) and not ops.gemv_ok(5, 6144, 4096) and not ops.gemv_ok(1, 3072, 576)
         ops.set_gemv(0)
         assert not ops.gemv_ok(1, 6144, 4096)
     finally:

@@ -17,6 +17,9 @@
                            are worth, the bound of anything that fetches weights ahead
   one_launch               a mock decode step as ONE launch: the blocks of each die meet inside the kernel through
                            that die's L2, a request a die (what a step fused into one kernel would cost at the least)
+  stream_loads             decode steps with ordinary and with non-temporal loads of keys and values beside the rule's
+                           choice, and the decode attention kernel alone over rows of mixed lengths, in row order and
+                           longest first
 """
 import argparse
 import json
@@ -419,15 +422,41 @@ def reread(args):
     return 0
 
 
+def _decode_step_ms(runner, sampler, rng, vocab, batch, prompt, steps=64, repeats=4):
+    """Seconds a decode step of `batch` requests takes after prompts of `prompt` random tokens: overlapped steps, as the
+    benchmark times them; the median of the repeats but the first.  The requests are released again."""
+    import statistics
+    import numpy as np
+    import torch
+    from runtime.engine import StepEntry
+    keys = [f"{batch}-{prompt}-{i}" for i in range(batch)]
+    last = []
+    for key in keys:
+        runner.create(key)
+        logits = runner.step([StepEntry(key, rng.integers(0, vocab, size=prompt, dtype=np.int32), [prompt - 1])])
+        last.append(sampler.pick(logits, [(0.0, 0, 0)])[0])
+    params, unread, times = [(0.0, 0, 0)] * batch, None, []
+    for rep in range(repeats):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            entries = [StepEntry(k, [0], [0], pending=True) for k in keys] if unread is not None else [StepEntry(k, [t], [0]) for k, t in zip(keys, last)]
+            unread = runner.pick(sampler, runner.step(entries), params)
+        torch.cuda.synchronize()
+        times.append((time.perf_counter() - t0) / steps)
+    for key in keys:
+        runner.release(key)
+    return statistics.median(times[1:])
+
+
 def hot_weights(args):
     """Decode steps (captured programs, steps overlapped, as the benchmark times them) of 1, 8 and 64 requests after
     2,048-token prompts: a model whose layers are distinct against the same model with one layer's weights at every
     place of the order (every place still keeps a cache of its own)."""
-    import statistics
     import numpy as np
     import torch
     from runtime.config import preset
-    from runtime.engine import ModelRunner, StepEntry, random_model
+    from runtime.engine import ModelRunner, random_model
     from runtime.models import ScheduleEntry
     from runtime.sampling import Sampler
     out = {}
@@ -441,26 +470,7 @@ def hot_weights(args):
                 model.schedule = [ScheduleEntry(0) for _ in range(layers)]
             sampler, rng = Sampler(), np.random.default_rng(0)
             runner = ModelRunner(model, n_pages=64 * 4096 // 16, page_size=16, max_requests=64, execution="graph")
-            result = {}
-            for batch in (1, 8, 64):
-                keys = [f"{batch}-{i}" for i in range(batch)]
-                last = []
-                for key in keys:
-                    runner.create(key)
-                    logits = runner.step([StepEntry(key, rng.integers(0, raw["vocab_size"], size=2048, dtype=np.int32), [2047])])
-                    last.append(sampler.pick(logits, [(0.0, 0, 0)])[0])
-                params, unread, times = [(0.0, 0, 0)] * batch, None, []
-                for rep in range(4):
-                    torch.cuda.synchronize()
-                    t0 = time.perf_counter()
-                    for _ in range(64):
-                        entries = [StepEntry(k, [0], [0], pending=True) for k in keys] if unread is not None else [StepEntry(k, [t], [0]) for k, t in zip(keys, last)]
-                        unread = runner.pick(sampler, runner.step(entries), params)
-                    torch.cuda.synchronize()
-                    times.append((time.perf_counter() - t0) / 64)
-                for key in keys:
-                    runner.release(key)
-                result[f"b{batch}_ms"] = round(statistics.median(times[1:]) * 1e3, 4)
+            result = {f"b{batch}_ms": round(_decode_step_ms(runner, sampler, rng, raw["vocab_size"], batch, 2048) * 1e3, 4) for batch in (1, 8, 64)}
             out[f"{name}_{layers}_layers_{'one_layers_weights_everywhere' if shared else 'distinct_layers'}"] = result
             del runner, model
             torch.cuda.empty_cache()
@@ -469,9 +479,94 @@ def hot_weights(args):
     return 0
 
 
+def stream_loads(args):
+    """Non-temporal loads of keys and values in decode attention, and the order in which its rows are handed out.
+    First whole decode steps (captured programs, overlapped) at the three sizes, with ordinary loads, with non-temporal
+    ones and with what `kernels.attention.rows_stream_loads` picks; then the kernel alone over 64 rows of mixed lengths
+    (228 to 2,304 keys, the serving workload's) at the 1.7B head shape, in row order and longest first, against 64 rows
+    of their mean length.  One line a point on stderr, then one JSON line."""
+    import math
+    import numpy as np
+    import torch
+    from runtime.config import preset
+    from runtime.engine import ModelRunner, random_model
+    from runtime.kernels import attention, ops
+    from runtime.sampling import Sampler
+    rule = attention.rows_stream_loads
+    steps = {}
+    grid = [("smollm2-135m", 30, [(1984, [1, 8, 16, 64]), (7936, [8, 64])]),
+            ("smollm2-1.7b", 8, [(1984, [1, 8, 32, 64]), (7936, [1, 8])]),
+            ("llama-3-8b", 8, [(1984, [1, 8, 64]), (7936, [8, 64])])]
+    try:
+        for name, layers, points in grid:
+            raw = preset(name)
+            raw["num_hidden_layers"] = layers
+            raw["max_position_embeddings"] = 8448
+            model = random_model(raw, seed=0)
+            sampler, rng = Sampler(), np.random.default_rng(0)
+            runner = ModelRunner(model, n_pages=64 * 8448 // args.page_size, page_size=args.page_size, max_requests=64, execution="graph")
+            for prompt, batches in points:
+                for batch in batches:
+                    ms = {}
+                    for how, pick in (("ordinary", lambda *a: False), ("non_temporal", lambda *a: True), ("rule", rule)):
+                        attention.rows_stream_loads = pick
+                        runner.programs.clear()          # the choice is part of a captured program
+                        ms[how] = round(_decode_step_ms(runner, sampler, rng, raw["vocab_size"], batch, prompt, steps=32) * 1e3, 4)
+                    steps[f"{name}_{layers}_layers_{batch}x{prompt}"] = ms
+                    print(f"{name:13s} {batch:3d} rows x {prompt:5d} keys  ordinary {ms['ordinary']:.4f} ms  non-temporal {ms['non_temporal']:.4f}"
+                          f" ({100 * (ms['non_temporal'] / ms['ordinary'] - 1):+5.1f} %)  rule {ms['rule']:.4f}", file=sys.stderr, flush=True)
+            del runner, model
+            torch.cuda.empty_cache()
+    finally:
+        attention.rows_stream_loads = rule
+    # the kernel alone: 64 rows, 32 key heads of 64 (the 1.7B sizes), pages scattered, three layers' keys and values in turn
+    dev, P, heads, kv, D = torch.device("cuda:0"), args.page_size, 32, 32, 64
+    gen = torch.Generator().manual_seed(0)
+    mixed = [int(x) for x in torch.randint(228, 2305, (64,), generator=gen)]
+    kernel = {}
+    for label, lengths in (("mixed_228_to_2304", mixed), (f"all_{sum(mixed) // 64}", [sum(mixed) // 64] * 64)):
+        pages_per = -(-max(lengths) // P)
+        n_pages = 64 * pages_per
+        ks = [torch.randn(n_pages, kv, P, D, device=dev).bfloat16() for _ in range(3)]
+        vs = [torch.randn(n_pages, kv, D, P, device=dev).bfloat16() for _ in range(3)]
+        tables = torch.randperm(n_pages, device=dev).int().view(64, pages_per)
+        q = torch.randn(64, heads * D, device=dev).bfloat16()
+        seg = torch.arange(64, device=dev, dtype=torch.int32)
+        pos = torch.tensor([n - 1 for n in lengths], device=dev, dtype=torch.int32)
+        out = torch.empty(64, heads * D, device=dev).bfloat16()
+        longest_first = torch.argsort(-pos.long(), stable=True).int()
+        for order_name, ids in (("row_order", None), ("longest_first", longest_first)):
+            for nt in (False, True):
+                def run(i):
+                    ops.attention_mfma(q, heads * D, ks[i], vs[i], tables, seg, pos, out, heads, kv, D, P, None, 1 / math.sqrt(D),
+                                       None, 1, None, 4, row_ids=ids, stream_loads=nt)
+                for i in range(3):
+                    run(i)
+                torch.cuda.synchronize()
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph):
+                    for i in range(6):
+                        run(i % 3)
+                graph.replay()
+                torch.cuda.synchronize()
+                times = []
+                for _ in range(5):
+                    t0 = time.perf_counter()
+                    graph.replay()
+                    torch.cuda.synchronize()
+                    times.append((time.perf_counter() - t0) / 6 * 1e6)
+                kernel[f"{label}_{order_name}_{'non_temporal' if nt else 'ordinary'}"] = round(sorted(times)[2], 1)
+        print(f"kernel alone, 64 rows {label}: " + "  ".join(f"{k[len(label) + 1:]} {v} us" for k, v in kernel.items() if k.startswith(label)),
+              file=sys.stderr, flush=True)
+    print(json.dumps({"metric": "ms a decode step of 8 requests at the 135M sizes with the rule's choice of loads for keys and values",
+                      "unit": "ms", "value": steps["smollm2-135m_30_layers_8x1984"]["rule"], "higher_is_better": False, "n_gpus": 1,
+                      "decode_steps_ms": steps, "kernel_alone_us": kernel}))
+    return 0
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser(prog="python -m runtime.measure")
-    ap.add_argument("workload", choices=["floor", "attention", "attention_forms", "decode_attention_shapes", "chain", "reread", "hot_weights", "one_launch"])
+    ap.add_argument("workload", choices=["floor", "attention", "attention_forms", "decode_attention_shapes", "chain", "reread", "hot_weights", "one_launch", "stream_loads"])
     ap.add_argument("--chain-layers", type=int, default=30, help="chain: layers of five products each (30: 113 MB of weights; 240: 904 MB, "
                                                                  "more than the memory-side cache holds)")
     ap.add_argument("--model", default="smollm2-135m", help="floor: the preset whose decode step the floor is priced for")
@@ -479,7 +574,7 @@ def main(argv=None):
     ap.add_argument("--attention-rows", default="2048,7936", help="attention workloads: prompt lengths (comma separated)")
     args = ap.parse_args(argv)
     return {"floor": launch_floor, "attention": prompt_attention, "attention_forms": attention_forms,
-            "decode_attention_shapes": decode_attention_shapes, "chain": chain, "reread": reread,
+            "decode_attention_shapes": decode_attention_shapes, "chain": chain, "reread": reread, "stream_loads": stream_loads,
             "hot_weights": hot_weights, "one_launch": one_launch}[args.workload](args)
 
 
